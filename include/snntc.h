@@ -1,0 +1,153 @@
+/*
+ * snntc.h -- C ABI of the MI355X (gfx950) implementation of the four SNN-TC custom ops.
+ *
+ * One entry point per reference op; each replaces the op's OpKernel::Compute (shape rules, error
+ * checks) together with its GPU functor (device work).  Paths below are relative to the
+ * reference checkout.
+ *
+ *   snntc_fc_forward   <- SnnFcOp::Compute      snntc/snnfc_kernels.cc:160-207
+ *                         SnnFcFunctor<GPU>     snntc/snnfc_kernels.cu.cc:93-194
+ *                         REGISTER_OP("SnnFc")  snntc/snnfc_ops.cc:6-27
+ *   snntc_fc_backward  <- SnnFcGradOp::Compute  snntc/snnfcgrad_kernels.cc:93-131
+ *                         SnnFcGradFunctor<GPU> snntc/snnfcgrad_kernels.cu.cc:137-225
+ *                         REGISTER_OP("SnnFcGrad") snntc/snnfcgrad_ops.cc:6-20
+ *   snntc_cv_forward   <- SnnCvOp::Compute      snntc/snncv_kernels.cc:191-242
+ *                         SnnCvFunctor<GPU>     snntc/snncv_kernels.cu.cc:95-210
+ *                         REGISTER_OP("SnnCv")  snntc/snncv_ops.cc:6-32
+ *   snntc_cv_backward  <- SnnCvGradOp::Compute  snntc/snncvgrad_kernels.cc:131-183
+ *                         SnnCvGradFunctor<GPU> snntc/snncvgrad_kernels.cu.cc:164-263
+ *                         REGISTER_OP("SnnCvGrad") snntc/snncvgrad_ops.cc:6-20
+ *
+ * Conventions
+ *  - All tensors are float32, row-major (images NHWC), and live in DEVICE memory, except
+ *    `params`, which is a HOST pointer (the reference pins it with HostMemory("params"),
+ *    snntc/snnfc_kernels.cc:224, snntc/snncv_kernels.cc:259).
+ *  - The caller owns every buffer, including the scratch `workspace` (device memory, 256-byte
+ *    aligned, at least snntc_*_workspace_bytes() long).  The library allocates nothing, keeps no
+ *    state between calls and is re-entrant.
+ *  - Work is enqueued on `stream` (a hipStream_t passed as void*; NULL = the default stream) and
+ *    the call returns without synchronising.
+ *  - Every function returns SNNTC_OK (0) or one of the codes below; snntc_last_error() returns a
+ *    thread-local text for the last failure.  Invalid-argument codes mirror the reference's
+ *    OP_REQUIRES(... InvalidArgument) conditions one to one.
+ *
+ * Params vectors (float32, exactly as the reference's Python layers build them)
+ *  dense [6]  (SNN_TC_Modules.py:48-49):   {MAX_SPIKE_TIME, Epsilon, Spike_Threshold,
+ *                                           Thread_per_Block, Blocks, biasvolt}
+ *  conv  [12] (SNN_TC_Modules.py:121-123): {MAX_SPIKE_TIME, Thread_per_Block, Blocks, Epsilon,
+ *                                           Spike_Threshold, cudaflag, Kh, Kw, Sh, Sw,
+ *                                           padding==SAME, biasvolt}
+ *  biasvolt > 1e-8 means the weight matrix carries one extra (last) bias row.  Epsilon,
+ *  Thread_per_Block, Blocks and cudaflag are accepted and ignored (launch shapes are chosen for
+ *  gfx950 by the library; the reference's GPU scan does not read Epsilon either).
+ */
+#ifndef SNNTC_H_
+#define SNNTC_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#if defined(__GNUC__)
+#define SNNTC_API __attribute__((visibility("default")))
+#else
+#define SNNTC_API
+#endif
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    SNNTC_OK = 0,
+    SNNTC_ERR_DIM_MISMATCH = 1,   /* weight rows vs input size (+bias); grad rows != 2*batch    */
+    SNNTC_ERR_TOO_LARGE = 2,      /* a tensor (or the patch matrix) exceeds INT32_MAX elements  */
+    SNNTC_ERR_BAD_ARGUMENT = 3,   /* null pointer, negative size, kernel larger than the image  */
+    SNNTC_ERR_WORKSPACE = 4,      /* workspace missing, misaligned or too small                  */
+    SNNTC_ERR_UNSUPPORTED = 5,    /* segment longer than the largest supported sort (8192)       */
+    SNNTC_ERR_HIP = 6             /* a HIP runtime call or kernel launch failed                  */
+};
+
+/* Library identification: "snntc-hip gfx950 <version>". */
+SNNTC_API const char* snntc_version(void);
+/* Text of the last error raised on the calling thread ("" if none). */
+SNNTC_API const char* snntc_last_error(void);
+/* Fixed text for a status code. */
+SNNTC_API const char* snntc_status_string(int status);
+
+/* ---------------------------------------------------------------------------------------------
+ * Dense layer (SNN_dense).   x[B,I]   w[w_rows,J] with w_rows == I + (biasvolt > 1e-8)
+ * ------------------------------------------------------------------------------------------- */
+
+/* Scratch sizes.  Replaces the reference's allocate_temp calls (snntc/snnfc_kernels.cu.cc:110-137,
+ * snntc/snnfcgrad_kernels.cu.cc:159-164). */
+SNNTC_API int snntc_fc_forward_workspace_bytes(int64_t B, int64_t I, int64_t J, size_t* bytes);
+SNNTC_API int snntc_fc_backward_workspace_bytes(int64_t B, int64_t I, int64_t J, size_t* bytes);
+
+/* out[2B,J]: rows [0,B) = output spike times y (MAX_SPIKE_TIME for a neuron that never fires),
+ * rows [B,2B) = 1/(sum_{causal set} w - Spike_Threshold) (0 for a neuron that never fires).
+ * Errors: w_rows not in {I, I+1} or inconsistent with biasvolt -> DIM_MISMATCH
+ *         (snntc/snnfc_kernels.cc:171-172); B*I, w_rows*J or 2*B*J > INT32_MAX -> TOO_LARGE
+ *         (snntc/snnfc_kernels.cc:194-203). */
+SNNTC_API int snntc_fc_forward(const float* x, const float* w, const float* params_host, float* out,
+                     int64_t B, int64_t I, int64_t J, int64_t w_rows,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* Same as snntc_fc_forward with optional side outputs (any may be NULL):
+ *   sorted_z[B,I]  each input row sorted ascending (stable: equal values keep index order)
+ *   perm[B,I]      int32 source column of every sorted element
+ *   causal_k[B,J]  int32 number of sorted inputs in the causal set, -1 if the neuron never fired
+ * These are the reference's temporaries d_in / order (snntc/snnfc_kernels.cu.cc:110-155) and the
+ * loop counter k at exit of SnnFcCudaOutKernel (snntc/snnfc_kernels.cu.cc:43-62). */
+SNNTC_API int snntc_fc_forward_ex(const float* x, const float* w, const float* params_host, float* out,
+                        float* sorted_z, int32_t* perm, int32_t* causal_k,
+                        int64_t B, int64_t I, int64_t J, int64_t w_rows,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/* grad[grad_rows,J] (only rows [0,B) are read), oldout[2B,J] = the forward output.
+ * dx[B,I], dw[w_rows,J], dparams[6] (device, may be NULL; written with zeros).
+ * Errors: grad_rows != 2B -> DIM_MISMATCH (snntc/snnfcgrad_kernels.cc:119-120); sizes as above. */
+SNNTC_API int snntc_fc_backward(const float* grad, const float* x, const float* w, const float* params_host,
+                      const float* oldout, float* dx, float* dw, float* dparams,
+                      int64_t B, int64_t I, int64_t J, int64_t w_rows, int64_t grad_rows,
+                      void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Convolutional layer (SNN_conv).  xpad[B,H,W,C] is the input AFTER the Python layer's padding /
+ * cropping (SNN_TC_Modules.py:144-166); w[w_rows,Kc] with w_rows == Kh*Kw*C + (biasvolt > 1e-8);
+ * Nh = (H-Kh)/Sh + 1, Nw = (W-Kw)/Sw + 1 (snntc/snncv_kernels.cc:215).
+ * ------------------------------------------------------------------------------------------- */
+
+/* Output spatial size for a padded input, from the params vector. */
+SNNTC_API int snntc_cv_output_dims(int64_t H, int64_t W, const float* params_host, int64_t* Nh, int64_t* Nw);
+
+SNNTC_API int snntc_cv_forward_workspace_bytes(int64_t B, int64_t H, int64_t W, int64_t C, int64_t Kc,
+                                     const float* params_host, size_t* bytes);
+SNNTC_API int snntc_cv_backward_workspace_bytes(int64_t B, int64_t H, int64_t W, int64_t C, int64_t Kc,
+                                      const float* params_host, size_t* bytes);
+
+/* out[2B,Nh,Nw,Kc], halves as in the dense op.
+ * Errors: w_rows != Kh*Kw*C + bias -> DIM_MISMATCH (snntc/snncv_kernels.cc:218); input, weight,
+ *         output or B*Nh*Nw*w_rows > INT32_MAX -> TOO_LARGE (snntc/snncv_kernels.cc:231-238). */
+SNNTC_API int snntc_cv_forward(const float* xpad, const float* w, const float* params_host, float* out,
+                     int64_t B, int64_t H, int64_t W, int64_t C, int64_t Kc, int64_t w_rows,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* Side outputs per patch s=(b*Nh+nh)*Nw+nw, element order (kh,kw,c):
+ *   sorted_z[B*Nh*Nw, Kh*Kw*C], perm[B*Nh*Nw, Kh*Kw*C], causal_k[B*Nh*Nw, Kc]. */
+SNNTC_API int snntc_cv_forward_ex(const float* xpad, const float* w, const float* params_host, float* out,
+                        float* sorted_z, int32_t* perm, int32_t* causal_k,
+                        int64_t B, int64_t H, int64_t W, int64_t C, int64_t Kc, int64_t w_rows,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/* grad[grad_rows,Nh,Nw,Kc] (rows [0,B) read), oldout[2B,Nh,Nw,Kc].
+ * dxpad[B,H,W,C] (gradient w.r.t. the padded input), dw[w_rows,Kc], dparams[12] (may be NULL).
+ * Errors: grad_rows != 2B -> DIM_MISMATCH; sizes as in the forward op. */
+SNNTC_API int snntc_cv_backward(const float* grad, const float* xpad, const float* w, const float* params_host,
+                      const float* oldout, float* dxpad, float* dw, float* dparams,
+                      int64_t B, int64_t H, int64_t W, int64_t C, int64_t Kc, int64_t w_rows,
+                      int64_t grad_rows, void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SNNTC_H_ */

@@ -1,0 +1,352 @@
+// C ABI of the library (declared in include/snntc.h): argument checks that mirror the reference
+// OpKernels' OP_REQUIRES conditions, workspace carving, and the kernel chains of the four ops.
+#include <limits.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "snntc_common.h"
+
+namespace snntc {
+
+static thread_local char g_last_error[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+namespace {
+
+constexpr int64_t kInt32Max = INT32_MAX;
+
+NeuronParams neuron_params(float max_time, float theta, float biasvolt) {
+    NeuronParams np;
+    np.max_time = max_time;
+    np.max_cmp = max_time - 0.1f;
+    np.theta = theta;
+    np.biasvolt = biasvolt;
+    np.bias = biasvolt > 1e-8f ? 1 : 0;
+    return np;
+}
+
+// Hands out 256-byte aligned pieces of the caller's workspace.
+struct Carver {
+    char* base;
+    size_t used = 0;
+    explicit Carver(void* p) : base(static_cast<char*>(p)) {}
+    template <typename T>
+    T* take(int64_t count) {
+        T* p = base ? reinterpret_cast<T*>(base + used) : nullptr;
+        used += align_up((size_t)(count > 0 ? count : 0) * sizeof(T));
+        return p;
+    }
+};
+
+int check_workspace(const void* ws, size_t have, size_t need) {
+    if (need == 0) return SNNTC_OK;
+    if (!ws) return fail(SNNTC_ERR_WORKSPACE, "workspace is NULL but %zu bytes are required", need);
+    if (reinterpret_cast<uintptr_t>(ws) % kAlign != 0)
+        return fail(SNNTC_ERR_WORKSPACE, "workspace must be %zu-byte aligned", kAlign);
+    if (have < need) return fail(SNNTC_ERR_WORKSPACE, "workspace too small: %zu bytes given, %zu required", have, need);
+    return SNNTC_OK;
+}
+
+// ---- dense -------------------------------------------------------------------------------------
+
+int fc_check(int64_t B, int64_t I, int64_t J, int64_t w_rows, const float* params, const char* who) {
+    if (!params) return fail(SNNTC_ERR_BAD_ARGUMENT, "%s: params is NULL", who);
+    if (B < 0 || I < 1 || J < 0) return fail(SNNTC_ERR_BAD_ARGUMENT, "%s: bad sizes B=%lld I=%lld J=%lld", who,
+                                              (long long)B, (long long)I, (long long)J);
+    const int bias = params[5] > 1e-8f ? 1 : 0;
+    if (w_rows != I && w_rows != I + 1)
+        return fail(SNNTC_ERR_DIM_MISMATCH, "%s: Input & Weight inner-dim mismatch (input %lld, weight rows %lld)",
+                    who, (long long)I, (long long)w_rows);
+    if (w_rows != I + bias)
+        return fail(SNNTC_ERR_DIM_MISMATCH, "%s: weight rows %lld do not match input %lld with biasvolt %g", who,
+                    (long long)w_rows, (long long)I, (double)params[5]);
+    if (B * I > kInt32Max) return fail(SNNTC_ERR_TOO_LARGE, "%s: Too many elements in input tensor", who);
+    if (w_rows * J > kInt32Max) return fail(SNNTC_ERR_TOO_LARGE, "%s: Too many elements in weight tensor", who);
+    if (2 * B * J > kInt32Max) return fail(SNNTC_ERR_TOO_LARGE, "%s: Too many elements in output tensor", who);
+    if (I > kMaxSegment)
+        return fail(SNNTC_ERR_UNSUPPORTED, "%s: input size %lld exceeds the largest supported segment (%d)", who,
+                    (long long)I, kMaxSegment);
+    return SNNTC_OK;
+}
+
+struct FcFwdWs { float* sorted; int32_t* perm; size_t bytes; };
+FcFwdWs fc_fwd_ws(void* ws, int64_t S, int64_t I) {
+    Carver c(ws);
+    FcFwdWs r;
+    r.sorted = c.take<float>(S * I);
+    r.perm = c.take<int32_t>(S * I);
+    r.bytes = c.used;
+    return r;
+}
+
+struct BwdWs { float* upm; float* ym; float* wt; float* partial; int nsplit; size_t bytes; };
+BwdWs bwd_ws(void* ws, int64_t S, int64_t rows, int64_t J) {
+    Carver c(ws);
+    BwdWs r;
+    r.upm = c.take<float>(S * J);
+    r.ym = c.take<float>(S * J);
+    r.wt = c.take<float>(rows * J);
+    r.nsplit = weight_grad_splits(S, rows, J);
+    r.partial = c.take<float>(r.nsplit > 1 ? (int64_t)r.nsplit * rows * J : 0);
+    r.bytes = c.used;
+    return r;
+}
+
+int fc_forward_impl(const float* x, const float* w, const float* params, float* out, float* sorted_z,
+                    int32_t* perm, int32_t* causal_k, int64_t B, int64_t I, int64_t J, int64_t w_rows,
+                    void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = fc_check(B, I, J, w_rows, params, "snntc_fc_forward");
+    if (rc) return rc;
+    if (B == 0 || J == 0) return SNNTC_OK;
+    if (!x || !w || !out) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_fc_forward: NULL tensor pointer");
+    FcFwdWs ws = fc_fwd_ws(workspace, B, I);
+    rc = check_workspace(workspace, workspace_bytes, ws.bytes);
+    if (rc) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const NeuronParams np = neuron_params(params[0], params[2], params[5]);
+    float* sorted = sorted_z ? sorted_z : ws.sorted;
+    int32_t* order = perm ? perm : ws.perm;
+    SegmentSource src{};
+    src.base = x; src.conv = 0; src.I = (int)I;
+    rc = launch_sort(src, B, sorted, order, st);
+    if (rc) return rc;
+    return launch_scan(sorted, order, w, out, out + B * J, causal_k, B, I, J, np, st);
+}
+
+// ---- conv --------------------------------------------------------------------------------------
+
+int cv_geom(int64_t B, int64_t H, int64_t W, int64_t C, int64_t Kc, int64_t w_rows, const float* params,
+            bool check_rows, const char* who, ConvGeom* g) {
+    if (!params) return fail(SNNTC_ERR_BAD_ARGUMENT, "%s: params is NULL", who);
+    g->B = B; g->H = H; g->W = W; g->C = C; g->Kc = Kc;
+    g->Kh = (int64_t)params[6]; g->Kw = (int64_t)params[7];
+    g->Sh = (int64_t)params[8]; g->Sw = (int64_t)params[9];
+    if (B < 0 || H < 1 || W < 1 || C < 1 || Kc < 0)
+        return fail(SNNTC_ERR_BAD_ARGUMENT, "%s: bad sizes B=%lld H=%lld W=%lld C=%lld Kc=%lld", who, (long long)B,
+                    (long long)H, (long long)W, (long long)C, (long long)Kc);
+    if (g->Kh < 1 || g->Kw < 1 || g->Sh < 1 || g->Sw < 1)
+        return fail(SNNTC_ERR_BAD_ARGUMENT, "%s: bad kernel/stride in params (Kh=%lld Kw=%lld Sh=%lld Sw=%lld)", who,
+                    (long long)g->Kh, (long long)g->Kw, (long long)g->Sh, (long long)g->Sw);
+    if (g->Kh > H || g->Kw > W)
+        return fail(SNNTC_ERR_BAD_ARGUMENT, "%s: kernel %lldx%lld larger than the (padded) input %lldx%lld", who,
+                    (long long)g->Kh, (long long)g->Kw, (long long)H, (long long)W);
+    g->Nh = (H - g->Kh) / g->Sh + 1;
+    g->Nw = (W - g->Kw) / g->Sw + 1;
+    g->P = g->Kh * g->Kw * C;
+    g->S = B * g->Nh * g->Nw;
+    if (!check_rows) return SNNTC_OK;
+    const int bias = params[11] > 1e-8f ? 1 : 0;
+    if (w_rows != g->P + bias)
+        return fail(SNNTC_ERR_DIM_MISMATCH, "%s: Input & Weight dim mismatch (bias): weight rows %lld, expected %lld",
+                    who, (long long)w_rows, (long long)(g->P + bias));
+    if (B * H * W * C > kInt32Max) return fail(SNNTC_ERR_TOO_LARGE, "%s: Too many elements in input tensor", who);
+    if (w_rows * Kc > kInt32Max) return fail(SNNTC_ERR_TOO_LARGE, "%s: Too many elements in weight tensor", who);
+    if (2 * g->S * Kc > kInt32Max) return fail(SNNTC_ERR_TOO_LARGE, "%s: Too many elements in output tensor", who);
+    if (g->S * w_rows > kInt32Max) return fail(SNNTC_ERR_TOO_LARGE, "%s: Too many elements in patched tensor", who);
+    if (g->P > kMaxSegment)
+        return fail(SNNTC_ERR_UNSUPPORTED, "%s: patch length %lld exceeds the largest supported segment (%d)", who,
+                    (long long)g->P, kMaxSegment);
+    return SNNTC_OK;
+}
+
+SegmentSource conv_source(const float* xpad, const ConvGeom& g) {
+    SegmentSource src{};
+    src.base = xpad; src.conv = 1; src.I = (int)g.P;
+    src.H = (int)g.H; src.W = (int)g.W; src.C = (int)g.C;
+    src.Kh = (int)g.Kh; src.Kw = (int)g.Kw; src.Sh = (int)g.Sh; src.Sw = (int)g.Sw;
+    src.Nh = (int)g.Nh; src.Nw = (int)g.Nw;
+    return src;
+}
+
+int cv_forward_impl(const float* xpad, const float* w, const float* params, float* out, float* sorted_z,
+                    int32_t* perm, int32_t* causal_k, int64_t B, int64_t H, int64_t W, int64_t C, int64_t Kc,
+                    int64_t w_rows, void* workspace, size_t workspace_bytes, void* stream) {
+    ConvGeom g;
+    int rc = cv_geom(B, H, W, C, Kc, w_rows, params, true, "snntc_cv_forward", &g);
+    if (rc) return rc;
+    if (g.S == 0 || Kc == 0) return SNNTC_OK;
+    if (!xpad || !w || !out) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_cv_forward: NULL tensor pointer");
+    FcFwdWs ws = fc_fwd_ws(workspace, g.S, g.P);
+    rc = check_workspace(workspace, workspace_bytes, ws.bytes);
+    if (rc) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const NeuronParams np = neuron_params(params[0], params[4], params[11]);
+    float* sorted = sorted_z ? sorted_z : ws.sorted;
+    int32_t* order = perm ? perm : ws.perm;
+    rc = launch_sort(conv_source(xpad, g), g.S, sorted, order, st);
+    if (rc) return rc;
+    return launch_scan(sorted, order, w, out, out + g.S * Kc, causal_k, g.S, g.P, Kc, np, st);
+}
+
+}  // namespace
+}  // namespace snntc
+
+using namespace snntc;
+
+extern "C" {
+
+const char* snntc_version(void) { return "snntc-hip gfx950 0.1"; }
+
+const char* snntc_last_error(void) { return g_last_error; }
+
+const char* snntc_status_string(int status) {
+    switch (status) {
+        case SNNTC_OK: return "ok";
+        case SNNTC_ERR_DIM_MISMATCH: return "tensor dimension mismatch";
+        case SNNTC_ERR_TOO_LARGE: return "tensor exceeds INT32_MAX elements";
+        case SNNTC_ERR_BAD_ARGUMENT: return "bad argument";
+        case SNNTC_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
+        case SNNTC_ERR_UNSUPPORTED: return "segment longer than the largest supported sort";
+        case SNNTC_ERR_HIP: return "HIP runtime error";
+        default: return "unknown status";
+    }
+}
+
+int snntc_fc_forward_workspace_bytes(int64_t B, int64_t I, int64_t J, size_t* bytes) {
+    (void)J;
+    if (!bytes || B < 0 || I < 0) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_fc_forward_workspace_bytes: bad argument");
+    *bytes = fc_fwd_ws(nullptr, B, I).bytes;
+    return SNNTC_OK;
+}
+
+int snntc_fc_backward_workspace_bytes(int64_t B, int64_t I, int64_t J, size_t* bytes) {
+    if (!bytes || B < 0 || I < 0 || J < 0)
+        return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_fc_backward_workspace_bytes: bad argument");
+    *bytes = bwd_ws(nullptr, B, I + 1, J).bytes;
+    return SNNTC_OK;
+}
+
+int snntc_fc_forward(const float* x, const float* w, const float* params_host, float* out, int64_t B,
+                     int64_t I, int64_t J, int64_t w_rows, void* workspace, size_t workspace_bytes,
+                     void* stream) {
+    return fc_forward_impl(x, w, params_host, out, nullptr, nullptr, nullptr, B, I, J, w_rows, workspace,
+                           workspace_bytes, stream);
+}
+
+int snntc_fc_forward_ex(const float* x, const float* w, const float* params_host, float* out,
+                        float* sorted_z, int32_t* perm, int32_t* causal_k, int64_t B, int64_t I, int64_t J,
+                        int64_t w_rows, void* workspace, size_t workspace_bytes, void* stream) {
+    return fc_forward_impl(x, w, params_host, out, sorted_z, perm, causal_k, B, I, J, w_rows, workspace,
+                           workspace_bytes, stream);
+}
+
+int snntc_fc_backward(const float* grad, const float* x, const float* w, const float* params_host,
+                      const float* oldout, float* dx, float* dw, float* dparams, int64_t B, int64_t I,
+                      int64_t J, int64_t w_rows, int64_t grad_rows, void* workspace, size_t workspace_bytes,
+                      void* stream) {
+    int rc = fc_check(B, I, J, w_rows, params_host, "snntc_fc_backward");
+    if (rc) return rc;
+    if (grad_rows != 2 * B)
+        return fail(SNNTC_ERR_DIM_MISMATCH, "snntc_fc_backward: Grad/Oldout batch should be 2 * batch (got %lld for batch %lld)",
+                    (long long)grad_rows, (long long)B);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dparams) { rc = launch_fill_zero(dparams, 6, st); if (rc) return rc; }
+    if (!dx || !dw) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_fc_backward: NULL output pointer");
+    if (B == 0 || J == 0) {
+        rc = launch_fill_zero(dx, B * I, st); if (rc) return rc;
+        return launch_fill_zero(dw, w_rows * J, st);
+    }
+    if (!grad || !x || !w || !oldout) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_fc_backward: NULL tensor pointer");
+    BwdWs ws = bwd_ws(workspace, B, I + 1, J);
+    rc = check_workspace(workspace, workspace_bytes, ws.bytes);
+    if (rc) return rc;
+    const NeuronParams np = neuron_params(params_host[0], params_host[2], params_host[5]);
+    rc = launch_prep_upstream(grad, oldout, oldout + B * J, ws.upm, ws.ym, B * J, np, st);
+    if (rc) return rc;
+    rc = launch_transpose(w, ws.wt, I, J, st);          // wt[J, I]: bias row not needed for dX
+    if (rc) return rc;
+    rc = launch_fc_grad_input(x, ws.wt, ws.upm, ws.ym, dx, B, I, J, I, st);
+    if (rc) return rc;
+    SegmentSource src{};
+    src.base = x; src.conv = 0; src.I = (int)I;
+    int nsplit = weight_grad_splits(B, w_rows, J);
+    if (nsplit > ws.nsplit) nsplit = ws.nsplit;
+    return launch_grad_weight(src, ws.upm, ws.ym, dw, ws.partial, nsplit, B, J, np, st);
+}
+
+int snntc_cv_output_dims(int64_t H, int64_t W, const float* params_host, int64_t* Nh, int64_t* Nw) {
+    ConvGeom g;
+    int rc = cv_geom(0, H, W, 1, 0, 0, params_host, false, "snntc_cv_output_dims", &g);
+    if (rc) return rc;
+    if (Nh) *Nh = g.Nh;
+    if (Nw) *Nw = g.Nw;
+    return SNNTC_OK;
+}
+
+int snntc_cv_forward_workspace_bytes(int64_t B, int64_t H, int64_t W, int64_t C, int64_t Kc,
+                                     const float* params_host, size_t* bytes) {
+    ConvGeom g;
+    int rc = cv_geom(B, H, W, C, Kc, 0, params_host, false, "snntc_cv_forward_workspace_bytes", &g);
+    if (rc) return rc;
+    if (!bytes) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_cv_forward_workspace_bytes: bytes is NULL");
+    *bytes = fc_fwd_ws(nullptr, g.S, g.P).bytes;
+    return SNNTC_OK;
+}
+
+int snntc_cv_backward_workspace_bytes(int64_t B, int64_t H, int64_t W, int64_t C, int64_t Kc,
+                                      const float* params_host, size_t* bytes) {
+    ConvGeom g;
+    int rc = cv_geom(B, H, W, C, Kc, 0, params_host, false, "snntc_cv_backward_workspace_bytes", &g);
+    if (rc) return rc;
+    if (!bytes) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_cv_backward_workspace_bytes: bytes is NULL");
+    *bytes = bwd_ws(nullptr, g.S, g.P + 1, Kc).bytes;
+    return SNNTC_OK;
+}
+
+int snntc_cv_forward(const float* xpad, const float* w, const float* params_host, float* out, int64_t B,
+                     int64_t H, int64_t W, int64_t C, int64_t Kc, int64_t w_rows, void* workspace,
+                     size_t workspace_bytes, void* stream) {
+    return cv_forward_impl(xpad, w, params_host, out, nullptr, nullptr, nullptr, B, H, W, C, Kc, w_rows,
+                           workspace, workspace_bytes, stream);
+}
+
+int snntc_cv_forward_ex(const float* xpad, const float* w, const float* params_host, float* out,
+                        float* sorted_z, int32_t* perm, int32_t* causal_k, int64_t B, int64_t H, int64_t W,
+                        int64_t C, int64_t Kc, int64_t w_rows, void* workspace, size_t workspace_bytes,
+                        void* stream) {
+    return cv_forward_impl(xpad, w, params_host, out, sorted_z, perm, causal_k, B, H, W, C, Kc, w_rows,
+                           workspace, workspace_bytes, stream);
+}
+
+int snntc_cv_backward(const float* grad, const float* xpad, const float* w, const float* params_host,
+                      const float* oldout, float* dxpad, float* dw, float* dparams, int64_t B, int64_t H,
+                      int64_t W, int64_t C, int64_t Kc, int64_t w_rows, int64_t grad_rows, void* workspace,
+                      size_t workspace_bytes, void* stream) {
+    ConvGeom g;
+    int rc = cv_geom(B, H, W, C, Kc, w_rows, params_host, true, "snntc_cv_backward", &g);
+    if (rc) return rc;
+    if (grad_rows != 2 * B)
+        return fail(SNNTC_ERR_DIM_MISMATCH, "snntc_cv_backward: Grad/Oldout batch should be 2 * batch (got %lld for batch %lld)",
+                    (long long)grad_rows, (long long)B);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dparams) { rc = launch_fill_zero(dparams, 12, st); if (rc) return rc; }
+    if (!dxpad || !dw) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_cv_backward: NULL output pointer");
+    if (g.S == 0 || Kc == 0) {
+        rc = launch_fill_zero(dxpad, B * H * W * C, st); if (rc) return rc;
+        return launch_fill_zero(dw, w_rows * Kc, st);
+    }
+    if (!grad || !xpad || !w || !oldout) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_cv_backward: NULL tensor pointer");
+    BwdWs ws = bwd_ws(workspace, g.S, g.P + 1, Kc);
+    rc = check_workspace(workspace, workspace_bytes, ws.bytes);
+    if (rc) return rc;
+    const NeuronParams np = neuron_params(params_host[0], params_host[4], params_host[11]);
+    rc = launch_prep_upstream(grad, oldout, oldout + g.S * Kc, ws.upm, ws.ym, g.S * Kc, np, st);
+    if (rc) return rc;
+    rc = launch_transpose(w, ws.wt, g.P, Kc, st);       // wt[Kc, P]
+    if (rc) return rc;
+    rc = launch_cv_grad_input(xpad, ws.wt, ws.upm, ws.ym, dxpad, g, g.P, st);
+    if (rc) return rc;
+    int nsplit = weight_grad_splits(g.S, w_rows, Kc);
+    if (nsplit > ws.nsplit) nsplit = ws.nsplit;
+    return launch_grad_weight(conv_source(xpad, g), ws.upm, ws.ym, dw, ws.partial, nsplit, g.S, Kc, np, st);
+}
+
+}  // extern "C"

@@ -1,0 +1,332 @@
+// Backward kernels of the dense and conv SNN-TC layers.
+//
+// Contract (snntc/snnfcgrad_kernels.cu.cc:60,118-120,159-173; snntc/snncvgrad_kernels.cu.cc:71,143,
+// 190-204), with up = grad[:S] * oldout[S:], MAXc = MAX_SPIKE_TIME - 0.1:
+//   dX[s,i] = sum_j [x_si <= y_sj and y_sj <= MAXc] up_sj * W[i,j]
+//   dW[i,j] = sum_s [x_si <= MAXc and y_sj <= MAXc and x_si <= y_sj] (x_si - y_sj) * up_sj
+//   dW[I,j] = the same with x = biasvolt (bias row)
+// For the conv layer s runs over output pixels and x_si is gathered from the padded image; dX is
+// accumulated in gather form (every input pixel sums over the output pixels whose window covers
+// it), so no atomics are needed and the result does not depend on scheduling.
+//
+// The validity test on y is folded into two small arrays prepared once per call:
+//   upm = valid ? up : 0,   ym = valid ? y : -inf      (x <= -inf is false for every finite x)
+// and the weight-gradient mask is folded into arithmetic: for x <= y the term (x-y) is <= 0 and
+// for x > y it is > 0, hence [x <= y](x - y) == min(x - y, 0).
+#include "snntc_common.h"
+
+namespace snntc {
+namespace {
+
+__global__ void __launch_bounds__(256)
+prep_upstream_kernel(const float* __restrict__ grad, const float* __restrict__ y,
+                     const float* __restrict__ rcp, float* __restrict__ upm, float* __restrict__ ym,
+                     int64_t n, float max_cmp) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n) return;
+    const float yv = y[t];
+    const bool valid = yv <= max_cmp;
+    upm[t] = valid ? grad[t] * rcp[t] : 0.0f;
+    ym[t] = valid ? yv : -INFINITY;
+}
+
+// 32x32 tile transpose through LDS (padded against bank conflicts).
+__global__ void __launch_bounds__(256)
+transpose_kernel(const float* __restrict__ in, float* __restrict__ out, int rows, int cols) {
+    __shared__ float tile[32][33];
+    const int tx = threadIdx.x % 32, ty = threadIdx.x / 32;       // 32 x 8
+    const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+    for (int dy = ty; dy < 32; dy += 8) {
+        const int r = r0 + dy, c = c0 + tx;
+        tile[dy][tx] = (r < rows && c < cols) ? in[(size_t)r * cols + c] : 0.0f;
+    }
+    __syncthreads();
+    for (int dy = ty; dy < 32; dy += 8) {
+        const int c = c0 + dy, r = r0 + tx;
+        if (r < rows && c < cols) out[(size_t)c * rows + r] = tile[tx][dy];
+    }
+}
+
+__global__ void __launch_bounds__(256) fill_zero_kernel(float* __restrict__ p, int64_t n) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t < n) p[t] = 0.0f;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Dense dX.  Lanes run across inputs i (wt[j, i] is read coalesced), each thread carries RB
+// samples whose y/up values are wave-uniform; the four wavefronts of a block split the j range
+// and are summed through LDS in a fixed order.
+// ---------------------------------------------------------------------------------------------
+constexpr int DX_RB = 4;
+
+__global__ void __launch_bounds__(256)
+fc_grad_input_kernel(const float* __restrict__ x, const float* __restrict__ wt,
+                     const float* __restrict__ upm, const float* __restrict__ ym, float* __restrict__ dx,
+                     int B, int I, int J, int wt_stride) {
+    __shared__ float red[3][DX_RB][kWave];
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int i = blockIdx.y * kWave + lane;
+    const int ic = min(i, I - 1);
+    const int b0 = blockIdx.x * DX_RB;
+
+    float xr[DX_RB], acc[DX_RB];
+    int brow[DX_RB];
+#pragma unroll
+    for (int r = 0; r < DX_RB; ++r) {
+        brow[r] = min(b0 + r, B - 1);
+        xr[r] = x[(size_t)brow[r] * I + ic];
+        acc[r] = 0.0f;
+    }
+    const int jq = (J + 3) / 4;
+    const int j_lo = wave * jq, j_hi = min(J, j_lo + jq);
+    for (int j = j_lo; j < j_hi; ++j) {
+        const float wv = wt[(size_t)j * wt_stride + ic];
+#pragma unroll
+        for (int r = 0; r < DX_RB; ++r) {
+            const float yv = ym[(size_t)brow[r] * J + j];
+            const float uv = upm[(size_t)brow[r] * J + j];
+            acc[r] = __fmaf_rn(xr[r] <= yv ? uv : 0.0f, wv, acc[r]);
+        }
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int r = 0; r < DX_RB; ++r) red[wave - 1][r][lane] = acc[r];
+    }
+    __syncthreads();
+    if (wave == 0 && i < I) {
+#pragma unroll
+        for (int r = 0; r < DX_RB; ++r) {
+            if (b0 + r < B)
+                dx[(size_t)(b0 + r) * I + i] = ((acc[r] + red[0][r][lane]) + red[1][r][lane]) + red[2][r][lane];
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// dW for dense rows or implicit conv patches.  Lanes run across outputs j (y/up rows are read
+// coalesced); each thread carries RI consecutive weight rows whose x values are wave-uniform.
+// The segment range is cut into gridDim.z slices; a slice is further split over the four
+// wavefronts of the block.  With more than one slice the per-slice sums go to `partial` and are
+// added in slice order by reduce_partials_kernel.
+// ---------------------------------------------------------------------------------------------
+constexpr int DW_RI = 8;
+
+__global__ void __launch_bounds__(256)
+grad_weight_kernel(SegmentSource src, const float* __restrict__ upm, const float* __restrict__ ym,
+                   float* __restrict__ dst, int S, int J, int rows, int seg_per_slice, float biasvolt) {
+    __shared__ float red[3][DW_RI][kWave];
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int j = blockIdx.x * kWave + lane;
+    const int jc = min(j, J - 1);
+    const int i0 = blockIdx.y * DW_RI;
+    const int I = src.I;
+
+    // per-row source offsets relative to the segment base (dense: the column; conv: kh/kw/c)
+    int off[DW_RI];
+    bool is_bias[DW_RI];
+#pragma unroll
+    for (int r = 0; r < DW_RI; ++r) {
+        const int i = min(i0 + r, rows - 1);
+        is_bias[r] = i >= I;
+        const int e = min(i, I - 1);
+        if (src.conv) {
+            const int span = src.Kw * src.C;
+            const int kh = e / span;
+            off[r] = kh * src.W * src.C + (e - kh * span);
+        } else {
+            off[r] = e;
+        }
+    }
+
+    const int s_begin = blockIdx.z * seg_per_slice;
+    const int s_end = min(S, s_begin + seg_per_slice);
+    const int per_wave = (s_end - s_begin + 3) / 4;
+    const int s_lo = s_begin + wave * per_wave;
+    const int s_hi = min(s_end, s_lo + per_wave);
+
+    float acc[DW_RI];
+#pragma unroll
+    for (int r = 0; r < DW_RI; ++r) acc[r] = 0.0f;
+
+    // walk (a, nh, nw) incrementally for conv sources
+    int a = 0, nh = 0, nw = 0;
+    if (src.conv && s_lo < s_hi) {
+        const int per_img = src.Nh * src.Nw;
+        a = s_lo / per_img;
+        const int r2 = s_lo - a * per_img;
+        nh = r2 / src.Nw;
+        nw = r2 - nh * src.Nw;
+    }
+    for (int s = s_lo; s < s_hi; ++s) {
+        const float* xb;
+        if (src.conv) {
+            xb = src.base + ((size_t)(a * src.H + nh * src.Sh) * src.W + (size_t)nw * src.Sw) * src.C;
+            if (++nw == src.Nw) { nw = 0; if (++nh == src.Nh) { nh = 0; ++a; } }
+        } else {
+            xb = src.base + (size_t)s * I;
+        }
+        const float yv = ym[(size_t)s * J + jc];
+        const float uv = upm[(size_t)s * J + jc];
+#pragma unroll
+        for (int r = 0; r < DW_RI; ++r) {
+            const float xv = is_bias[r] ? biasvolt : xb[off[r]];
+            acc[r] = __fmaf_rn(fminf(xv - yv, 0.0f), uv, acc[r]);
+        }
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int r = 0; r < DW_RI; ++r) red[wave - 1][r][lane] = acc[r];
+    }
+    __syncthreads();
+    if (wave == 0 && j < J) {
+        float* out = dst + (size_t)blockIdx.z * rows * J;
+#pragma unroll
+        for (int r = 0; r < DW_RI; ++r) {
+            if (i0 + r < rows)
+                out[(size_t)(i0 + r) * J + j] = ((acc[r] + red[0][r][lane]) + red[1][r][lane]) + red[2][r][lane];
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256)
+reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ out, int64_t n, int nsplit) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n) return;
+    float acc = 0.0f;
+    for (int z = 0; z < nsplit; ++z) acc += partial[(size_t)z * n + t];
+    out[t] = acc;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Conv dX, gather form.  One thread per element of the padded image (channel fastest, so lanes
+// read wt[kc, (kh,kw,c)] coalesced); it visits every output pixel whose window covers its pixel.
+// ---------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+cv_grad_input_kernel(const float* __restrict__ xpad, const float* __restrict__ wt,
+                     const float* __restrict__ upm, const float* __restrict__ ym, float* __restrict__ dxpad,
+                     int64_t n, int H, int W, int C, int Kc, int Kh, int Kw, int Sh, int Sw, int Nh, int Nw,
+                     int wt_stride) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n) return;
+    const int c = (int)(t % C);
+    const int64_t pix = t / C;
+    const int wx = (int)(pix % W);
+    const int64_t rowi = pix / W;
+    const int h = (int)(rowi % H);
+    const int a = (int)(rowi / H);
+    const float xv = xpad[t];
+
+    // output rows nh with nh*Sh <= h <= nh*Sh + Kh - 1
+    const int nh_lo = max(0, (h - Kh + Sh) / Sh);      // ceil((h-Kh+1)/Sh) for the non-negative case
+    const int nh_hi = min(Nh - 1, h / Sh);
+    const int nw_lo = max(0, (wx - Kw + Sw) / Sw);
+    const int nw_hi = min(Nw - 1, wx / Sw);
+
+    float acc = 0.0f;
+    for (int nh = nh_lo; nh <= nh_hi; ++nh) {
+        const int kh = h - nh * Sh;
+        for (int nw = nw_lo; nw <= nw_hi; ++nw) {
+            const int kw = wx - nw * Sw;
+            const int i = (kh * Kw + kw) * C + c;
+            const size_t so = ((size_t)(a * Nh + nh) * Nw + nw) * Kc;
+            const float* __restrict__ wrow = wt + i;
+            for (int kc = 0; kc < Kc; ++kc) {
+                const float yv = ym[so + kc];
+                const float uv = upm[so + kc];
+                acc = __fmaf_rn(xv <= yv ? uv : 0.0f, wrow[(size_t)kc * wt_stride], acc);
+            }
+        }
+    }
+    dxpad[t] = acc;
+}
+
+int blocks_for(int64_t n, int block) { return (int)((n + block - 1) / block); }
+
+}  // namespace
+
+int launch_prep_upstream(const float* grad, const float* y, const float* rcp, float* upm, float* ym,
+                         int64_t n, const NeuronParams& np, hipStream_t stream) {
+    if (n <= 0) return SNNTC_OK;
+    hipLaunchKernelGGL(prep_upstream_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream, grad, y, rcp,
+                       upm, ym, n, np.max_cmp);
+    SNNTC_HIP_CHECK(hipGetLastError());
+    return SNNTC_OK;
+}
+
+int launch_transpose(const float* w, float* wt, int64_t rows, int64_t cols, hipStream_t stream) {
+    if (rows <= 0 || cols <= 0) return SNNTC_OK;
+    dim3 grid((unsigned)((cols + 31) / 32), (unsigned)((rows + 31) / 32));
+    hipLaunchKernelGGL(transpose_kernel, grid, dim3(256), 0, stream, w, wt, (int)rows, (int)cols);
+    SNNTC_HIP_CHECK(hipGetLastError());
+    return SNNTC_OK;
+}
+
+int launch_fill_zero(float* p, int64_t n, hipStream_t stream) {
+    if (n <= 0) return SNNTC_OK;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream, p, n);
+    SNNTC_HIP_CHECK(hipGetLastError());
+    return SNNTC_OK;
+}
+
+int launch_fc_grad_input(const float* x, const float* wt, const float* upm, const float* ym, float* dx,
+                         int64_t B, int64_t I, int64_t J, int64_t wt_stride, hipStream_t stream) {
+    if (B <= 0 || I <= 0) return SNNTC_OK;
+    if (J <= 0) return launch_fill_zero(dx, B * I, stream);
+    dim3 grid((unsigned)((B + DX_RB - 1) / DX_RB), (unsigned)((I + kWave - 1) / kWave));
+    if (grid.y > 65535u) return fail(SNNTC_ERR_TOO_LARGE, "dense backward: input size %lld too large", (long long)I);
+    hipLaunchKernelGGL(fc_grad_input_kernel, grid, dim3(256), 0, stream, x, wt, upm, ym, dx, (int)B, (int)I,
+                       (int)J, (int)wt_stride);
+    SNNTC_HIP_CHECK(hipGetLastError());
+    return SNNTC_OK;
+}
+
+// Number of slices the segment range is cut into for dW: enough blocks to fill the chip,
+// at least 64 segments per slice, at most 256 slices.
+int weight_grad_splits(int64_t S, int64_t rows, int64_t J) {
+    const int64_t base_blocks = ((J + kWave - 1) / kWave) * ((rows + DW_RI - 1) / DW_RI);
+    int64_t want = (2048 + base_blocks - 1) / (base_blocks > 0 ? base_blocks : 1);
+    int64_t cap = S / 64;
+    if (want > cap) want = cap;
+    if (want > 256) want = 256;
+    if (want < 1) want = 1;
+    return (int)want;
+}
+
+int launch_grad_weight(const SegmentSource& src, const float* upm, const float* ym, float* dw,
+                       float* partial, int nsplit, int64_t S, int64_t J, const NeuronParams& np,
+                       hipStream_t stream) {
+    const int64_t rows = (int64_t)src.I + np.bias;
+    if (rows <= 0 || J <= 0) return SNNTC_OK;
+    if (S <= 0) return launch_fill_zero(dw, rows * J, stream);
+    if (nsplit < 1) nsplit = 1;
+    const int seg_per_slice = (int)((S + nsplit - 1) / nsplit);
+    dim3 grid((unsigned)((J + kWave - 1) / kWave), (unsigned)((rows + DW_RI - 1) / DW_RI), (unsigned)nsplit);
+    if (grid.y > 65535u) return fail(SNNTC_ERR_TOO_LARGE, "weight gradient: too many weight rows");
+    float* dst = nsplit > 1 ? partial : dw;
+    hipLaunchKernelGGL(grad_weight_kernel, grid, dim3(256), 0, stream, src, upm, ym, dst, (int)S, (int)J,
+                       (int)rows, seg_per_slice, np.biasvolt);
+    SNNTC_HIP_CHECK(hipGetLastError());
+    if (nsplit > 1) {
+        const int64_t n = rows * J;
+        hipLaunchKernelGGL(reduce_partials_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream, partial, dw,
+                           n, nsplit);
+        SNNTC_HIP_CHECK(hipGetLastError());
+    }
+    return SNNTC_OK;
+}
+
+int launch_cv_grad_input(const float* xpad, const float* wt, const float* upm, const float* ym,
+                         float* dxpad, const ConvGeom& g, int64_t wt_stride, hipStream_t stream) {
+    const int64_t n = g.B * g.H * g.W * g.C;
+    if (n <= 0) return SNNTC_OK;
+    if (g.Kc <= 0 || g.S <= 0) return launch_fill_zero(dxpad, n, stream);
+    hipLaunchKernelGGL(cv_grad_input_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream, xpad, wt, upm, ym,
+                       dxpad, n, (int)g.H, (int)g.W, (int)g.C, (int)g.Kc, (int)g.Kh, (int)g.Kw, (int)g.Sh,
+                       (int)g.Sw, (int)g.Nh, (int)g.Nw, (int)wt_stride);
+    SNNTC_HIP_CHECK(hipGetLastError());
+    return SNNTC_OK;
+}
+
+}  // namespace snntc

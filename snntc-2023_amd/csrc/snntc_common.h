@@ -1,0 +1,82 @@
+// Shared declarations of the gfx950 SNN-TC library: status plumbing, the parsed form of the two
+// params vectors, conv geometry and the launcher prototypes that api.hip chains together.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/snntc.h"
+
+namespace snntc {
+
+constexpr int kWave = 64;              // CDNA wavefront width
+constexpr int kMaxSegment = 8192;      // longest sortable segment (power-of-two padded)
+constexpr size_t kAlign = 256;         // workspace sub-buffer alignment
+
+// Records a formatted message for snntc_last_error() and returns `code`.
+int fail(int code, const char* fmt, ...);
+
+#define SNNTC_HIP_CHECK(expr)                                                              \
+    do {                                                                                   \
+        hipError_t e_ = (expr);                                                            \
+        if (e_ != hipSuccess)                                                              \
+            return ::snntc::fail(SNNTC_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e_)); \
+    } while (0)
+
+inline size_t align_up(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
+
+// The scalar knobs every kernel needs, taken from either params layout.
+struct NeuronParams {
+    float max_time;   // MAX_SPIKE_TIME
+    float max_cmp;    // MAX_SPIKE_TIME - 0.1 evaluated in fp32 (snntc/snnfc_kernels.cu.cc:27)
+    float theta;      // Spike_Threshold
+    float biasvolt;   // input value of the bias row
+    int bias;         // biasvolt > 1e-8
+};
+
+// Where a segment's elements come from: rows of a dense matrix, or patches of an NHWC image
+// gathered on the fly (patch s=(a*Nh+nh)*Nw+nw, element i=(kh*Kw+kw)*C+c).
+struct SegmentSource {
+    const float* base;
+    int conv;         // 0: dense rows of length I;  1: implicit im2col
+    int I;            // segment length (dense in_size or Kh*Kw*C)
+    int H, W, C, Kh, Kw, Sh, Sw, Nh, Nw;
+};
+
+struct ConvGeom {
+    int64_t B, H, W, C, Kc, Kh, Kw, Sh, Sw, Nh, Nw, P, S;
+};
+
+// ---- launchers (each enqueues on `stream` and returns a status) --------------------------------
+
+// Segmented stable ascending sort: sorted[S,I] and perm[S,I].
+int launch_sort(const SegmentSource& src, int64_t S, float* sorted, int32_t* perm, hipStream_t stream);
+
+// Causal-set scan over sorted segments: y[S,J], rcp[S,J], optional causal_k[S,J].
+int launch_scan(const float* sorted, const int32_t* perm, const float* w, float* y, float* rcp,
+                int32_t* causal_k, int64_t S, int64_t I, int64_t J, const NeuronParams& np,
+                hipStream_t stream);
+
+// upm = valid ? grad*rcp : 0 ; ym = valid ? y : -inf   (valid: y <= MAX-0.1), n elements each.
+int launch_prep_upstream(const float* grad, const float* y, const float* rcp, float* upm, float* ym,
+                         int64_t n, const NeuronParams& np, hipStream_t stream);
+
+// wt[cols, rows] = w[rows, cols]^T
+int launch_transpose(const float* w, float* wt, int64_t rows, int64_t cols, hipStream_t stream);
+
+int launch_fc_grad_input(const float* x, const float* wt, const float* upm, const float* ym, float* dx,
+                         int64_t B, int64_t I, int64_t J, int64_t wt_stride, hipStream_t stream);
+
+// dW for dense rows or implicit patches; `partial` is scratch for the split reduction.
+int weight_grad_splits(int64_t S, int64_t rows, int64_t J);
+int launch_grad_weight(const SegmentSource& src, const float* upm, const float* ym, float* dw,
+                       float* partial, int nsplit, int64_t S, int64_t J, const NeuronParams& np,
+                       hipStream_t stream);
+
+int launch_cv_grad_input(const float* xpad, const float* wt, const float* upm, const float* ym,
+                         float* dxpad, const ConvGeom& g, int64_t wt_stride, hipStream_t stream);
+
+int launch_fill_zero(float* p, int64_t n, hipStream_t stream);
+
+}  // namespace snntc

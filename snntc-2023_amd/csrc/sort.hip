@@ -1,0 +1,175 @@
+// Segmented stable sort of spike times: one bitonic network per segment, emitting the sorted
+// values and the permutation.
+//
+// Replaces the reference's cub::DeviceSegmentedSort::SortPairs call plus the index-generation and
+// im2col temporaries in front of it (snntc/snnfc_kernels.cu.cc:110-155,
+// snntc/snncv_kernels.cu.cc:112-166).  Differences by design:
+//  * keys are 64-bit composites (order-preserving image of the fp32 value << 32 | source index), so
+//    the network -- although not stable by itself -- returns exactly the stable ascending order;
+//  * conv patches are gathered straight from the NHWC image, the [B*Nh*Nw, Kh*Kw*C] patch matrix
+//    is never written to memory;
+//  * a segment is owned by G threads holding EPT consecutive elements each: exchanges at distance
+//    < EPT stay in registers, distances below 64 threads use wavefront shuffles, and only
+//    segments wider than one wavefront go through LDS.
+#include "snntc_common.h"
+
+namespace snntc {
+namespace {
+
+typedef unsigned long long u64;
+
+__device__ __forceinline__ uint32_t float_to_key(float f) {
+    uint32_t u = __float_as_uint(f);
+    if (u == 0x80000000u) u = 0u;                         // -0 sorts together with +0
+    return u ^ ((u >> 31) ? 0xffffffffu : 0x80000000u);
+}
+
+__device__ __forceinline__ float key_to_float(uint32_t k) {
+    return __uint_as_float(k ^ ((k >> 31) ? 0x80000000u : 0xffffffffu));
+}
+
+template <int EPT, int G, int BLOCK>
+__global__ void __launch_bounds__(BLOCK)
+sort_segments_kernel(SegmentSource src, float* __restrict__ sorted, int32_t* __restrict__ perm, int S) {
+    constexpr int NPAD = EPT * G;
+    constexpr int SEGS = BLOCK / G;
+    constexpr bool CROSS_WAVE = G > kWave;
+    __shared__ u64 xchg[CROSS_WAVE ? NPAD : 1];
+
+    const int tseg = threadIdx.x % G;
+    const int seg = blockIdx.x * SEGS + threadIdx.x / G;
+    const bool live = seg < S;
+    const int I = src.I;
+
+    // ---- load EPT consecutive elements, pad with keys that sort after every real value --------
+    u64 v[EPT];
+    {
+        const float* p = src.base;
+        int kh = 0, rem = 0, row = 0, span = 1;
+        if (live) {
+            if (src.conv) {
+                const int per_img = src.Nh * src.Nw;
+                const int a = seg / per_img, r2 = seg - a * per_img;
+                const int nh = r2 / src.Nw, nw = r2 - nh * src.Nw;
+                p += ((size_t)(a * src.H + nh * src.Sh) * src.W + (size_t)nw * src.Sw) * src.C;
+                span = src.Kw * src.C;          // contiguous floats per kernel row
+                row = src.W * src.C;            // floats per image row
+                kh = (tseg * EPT) / span;
+                rem = tseg * EPT - kh * span;
+            } else {
+                p += (size_t)seg * I;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < EPT; ++r) {
+            const int e = tseg * EPT + r;
+            uint32_t key = 0xffffffffu;
+            if (live && e < I) {
+                float f;
+                if (src.conv) {
+                    f = p[(size_t)kh * row + rem];
+                    if (++rem == span) { rem = 0; ++kh; }
+                } else {
+                    f = p[e];
+                }
+                key = float_to_key(f);
+            }
+            v[r] = ((u64)key << 32) | (uint32_t)e;
+        }
+    }
+
+    // ---- bitonic network ------------------------------------------------------------------------
+#pragma unroll
+    for (int k = 2; k <= NPAD; k <<= 1) {
+        // partners in other threads: element distance j >= EPT
+#pragma unroll
+        for (int j = k >> 1; j >= EPT; j >>= 1) {
+            const int d = j / EPT;
+            const bool lower = (tseg & d) == 0;
+            const bool up = ((tseg * EPT) & k) == 0;
+            const bool keep_min = (lower == up);
+            if (CROSS_WAVE && d >= kWave) {
+                __syncthreads();
+#pragma unroll
+                for (int r = 0; r < EPT; ++r) xchg[r * G + tseg] = v[r];
+                __syncthreads();
+#pragma unroll
+                for (int r = 0; r < EPT; ++r) {
+                    const u64 o = xchg[r * G + (tseg ^ d)];
+                    const bool take = (o < v[r]) == keep_min;
+                    v[r] = take ? o : v[r];
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < EPT; ++r) {
+                    const u64 o = __shfl_xor(v[r], d, kWave);
+                    const bool take = (o < v[r]) == keep_min;
+                    v[r] = take ? o : v[r];
+                }
+            }
+        }
+        // partners inside the thread: element distance j < EPT
+#pragma unroll
+        for (int j = (EPT >> 1); j >= 1; j >>= 1) {
+            if (j <= (k >> 1)) {
+#pragma unroll
+                for (int r = 0; r < EPT; ++r) {
+                    if ((r & j) == 0) {
+                        const bool up = ((tseg * EPT + r) & k) == 0;
+                        const u64 a = v[r], b = v[r | j];
+                        const bool sw = (a > b) == up;
+                        v[r] = sw ? b : a;
+                        v[r | j] = sw ? a : b;
+                    }
+                }
+            }
+        }
+    }
+
+    // ---- store ------------------------------------------------------------------------------------
+    if (live) {
+        float* so = sorted + (size_t)seg * I;
+        int32_t* po = perm + (size_t)seg * I;
+#pragma unroll
+        for (int r = 0; r < EPT; ++r) {
+            const int e = tseg * EPT + r;
+            if (e < I) {
+                so[e] = key_to_float((uint32_t)(v[r] >> 32));
+                po[e] = (int32_t)(uint32_t)v[r];
+            }
+        }
+    }
+}
+
+template <int EPT, int G>
+int launch_sort_t(const SegmentSource& src, int64_t S, float* sorted, int32_t* perm, hipStream_t stream) {
+    constexpr int BLOCK = G > 256 ? G : 256;
+    constexpr int SEGS = BLOCK / G;
+    const int64_t blocks = (S + SEGS - 1) / SEGS;
+    if (blocks > 0x7fffffffLL) return fail(SNNTC_ERR_TOO_LARGE, "sort: too many segments (%lld)", (long long)S);
+    hipLaunchKernelGGL((sort_segments_kernel<EPT, G, BLOCK>), dim3((unsigned)blocks), dim3(BLOCK), 0, stream,
+                       src, sorted, perm, (int)S);
+    SNNTC_HIP_CHECK(hipGetLastError());
+    return SNNTC_OK;
+}
+
+}  // namespace
+
+int launch_sort(const SegmentSource& src, int64_t S, float* sorted, int32_t* perm, hipStream_t stream) {
+    if (S <= 0 || src.I <= 0) return SNNTC_OK;
+    const int I = src.I;
+    if (I > kMaxSegment)
+        return fail(SNNTC_ERR_UNSUPPORTED, "segment length %d exceeds the largest supported sort (%d)", I,
+                    kMaxSegment);
+    if (I <= 32)   return launch_sort_t<2, 16>(src, S, sorted, perm, stream);
+    if (I <= 64)   return launch_sort_t<2, 32>(src, S, sorted, perm, stream);
+    if (I <= 128)  return launch_sort_t<2, 64>(src, S, sorted, perm, stream);
+    if (I <= 256)  return launch_sort_t<4, 64>(src, S, sorted, perm, stream);
+    if (I <= 512)  return launch_sort_t<8, 64>(src, S, sorted, perm, stream);
+    if (I <= 1024) return launch_sort_t<16, 64>(src, S, sorted, perm, stream);
+    if (I <= 2048) return launch_sort_t<8, 256>(src, S, sorted, perm, stream);
+    if (I <= 4096) return launch_sort_t<8, 512>(src, S, sorted, perm, stream);
+    return launch_sort_t<8, 1024>(src, S, sorted, perm, stream);
+}
+
+}  // namespace snntc

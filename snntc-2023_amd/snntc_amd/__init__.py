@@ -1,0 +1,16 @@
+"""MI355X (gfx950) implementation of the SNN-TC custom ops behind the reference's Python API.
+
+Public names follow the reference module ``SNN_TC_Modules``: the op handles ``snnfc``,
+``snnfc_grad``, ``snncv``, ``snncv_grad`` and the layers ``SNN_dense``, ``SNN_conv``,
+``SNN_maxpool2d``, ``SNN_avgpool2d``, ``SNN_LRN``, plus ``init_weight`` and ``loss_func``.
+"""
+from . import _lib
+from ._lib import SnntcError, SnntcLibraryError
+from .ops import SnnCv, SnnFc, snncv, snncv_grad, snncv_output_dims, snnfc, snnfc_grad
+from .layers import (SNN_LRN, SNN_avgpool2d, SNN_conv, SNN_dense, SNN_maxpool2d, init_weight, loss_func)
+
+__all__ = [
+    "snnfc", "snnfc_grad", "snncv", "snncv_grad", "snncv_output_dims", "SnnFc", "SnnCv",
+    "SNN_dense", "SNN_conv", "SNN_maxpool2d", "SNN_avgpool2d", "SNN_LRN", "init_weight", "loss_func",
+    "SnntcError", "SnntcLibraryError",
+]

@@ -1,0 +1,103 @@
+"""Loader and raw bindings of ``libsnntc_hip.so`` (C ABI declared in ``include/snntc.h``).
+
+The library is looked up next to the HIP sources (``snntc-2023_amd/csrc/libsnntc_hip.so``, built
+in-tree by ``make -C snntc-2023_amd/csrc``) or at ``$SNNTC_HIP_LIB``.  There is no CPU fallback:
+if the library is missing, loading raises ``SnntcLibraryError``.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC_DIR = os.path.normpath(os.path.join(_HERE, "..", "csrc"))
+DEFAULT_LIB = os.path.join(CSRC_DIR, "libsnntc_hip.so")
+
+OK = 0
+ERR_DIM_MISMATCH = 1
+ERR_TOO_LARGE = 2
+ERR_BAD_ARGUMENT = 3
+ERR_WORKSPACE = 4
+ERR_UNSUPPORTED = 5
+ERR_HIP = 6
+
+#: every symbol include/snntc.h declares
+EXPORTS = (
+    "snntc_version", "snntc_last_error", "snntc_status_string",
+    "snntc_fc_forward_workspace_bytes", "snntc_fc_backward_workspace_bytes",
+    "snntc_fc_forward", "snntc_fc_forward_ex", "snntc_fc_backward",
+    "snntc_cv_output_dims", "snntc_cv_forward_workspace_bytes", "snntc_cv_backward_workspace_bytes",
+    "snntc_cv_forward", "snntc_cv_forward_ex", "snntc_cv_backward",
+)
+
+
+class SnntcLibraryError(RuntimeError):
+    """The HIP library is missing or does not export the expected ABI."""
+
+
+class SnntcError(RuntimeError):
+    """A library call failed with a non-argument error (workspace, HIP runtime, unsupported size)."""
+
+    def __init__(self, status, message):
+        super().__init__(f"snntc status {status}: {message}")
+        self.status = status
+
+
+_lib = None
+
+
+def lib_path():
+    return os.environ.get("SNNTC_HIP_LIB", DEFAULT_LIB)
+
+
+def load():
+    """Returns the ctypes handle, loading and prototyping the library on first use."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = lib_path()
+    if not os.path.exists(path):
+        raise SnntcLibraryError(
+            f"{path} not found: build it with `make -C {CSRC_DIR}` (hipcc, --offload-arch=gfx950). "
+            "There is no CPU fallback for the SNN-TC ops.")
+    try:
+        lib = ctypes.CDLL(path)
+    except OSError as e:  # missing ROCm runtime etc.
+        raise SnntcLibraryError(f"cannot load {path}: {e}") from e
+    missing = [s for s in EXPORTS if not hasattr(lib, s)]
+    if missing:
+        raise SnntcLibraryError(f"{path} lacks symbols {missing}")
+
+    c = ctypes
+    vp, i64, sz = c.c_void_p, c.c_int64, c.c_size_t
+    fparams = c.POINTER(c.c_float)
+    lib.snntc_version.restype = c.c_char_p
+    lib.snntc_last_error.restype = c.c_char_p
+    lib.snntc_status_string.restype = c.c_char_p
+    lib.snntc_status_string.argtypes = [c.c_int]
+    lib.snntc_fc_forward_workspace_bytes.argtypes = [i64, i64, i64, c.POINTER(sz)]
+    lib.snntc_fc_backward_workspace_bytes.argtypes = [i64, i64, i64, c.POINTER(sz)]
+    lib.snntc_fc_forward.argtypes = [vp, vp, fparams, vp, i64, i64, i64, i64, vp, sz, vp]
+    lib.snntc_fc_forward_ex.argtypes = [vp, vp, fparams, vp, vp, vp, vp, i64, i64, i64, i64, vp, sz, vp]
+    lib.snntc_fc_backward.argtypes = [vp, vp, vp, fparams, vp, vp, vp, vp, i64, i64, i64, i64, i64, vp, sz, vp]
+    lib.snntc_cv_output_dims.argtypes = [i64, i64, fparams, c.POINTER(i64), c.POINTER(i64)]
+    lib.snntc_cv_forward_workspace_bytes.argtypes = [i64, i64, i64, i64, i64, fparams, c.POINTER(sz)]
+    lib.snntc_cv_backward_workspace_bytes.argtypes = [i64, i64, i64, i64, i64, fparams, c.POINTER(sz)]
+    lib.snntc_cv_forward.argtypes = [vp, vp, fparams, vp, i64, i64, i64, i64, i64, i64, vp, sz, vp]
+    lib.snntc_cv_forward_ex.argtypes = [vp, vp, fparams, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, sz, vp]
+    lib.snntc_cv_backward.argtypes = [vp, vp, vp, fparams, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64,
+                                      vp, sz, vp]
+    for name in EXPORTS:
+        if name not in ("snntc_version", "snntc_last_error", "snntc_status_string"):
+            getattr(lib, name).restype = c.c_int
+    _lib = lib
+    return lib
+
+
+def check(status):
+    """Maps a status code to the exception the reference's Python caller would see:
+    InvalidArgument conditions -> ValueError, everything else -> SnntcError."""
+    if status == OK:
+        return
+    msg = load().snntc_last_error().decode("utf-8", "replace")
+    if status in (ERR_DIM_MISMATCH, ERR_TOO_LARGE, ERR_BAD_ARGUMENT):
+        raise ValueError(msg)
+    raise SnntcError(status, msg)

@@ -1,0 +1,207 @@
+"""The four SNN-TC ops over PyTorch-ROCm tensors, each a thin call into the C ABI.
+
+Counterparts of the reference's op handles (SNN_TC_Modules.py:29-33, 89-93):
+
+    snnfc(X, W, Params)                      -> Y[2B, J]
+    snnfc_grad(grad, X, W, Params, Y)        -> (dX, dW, dParams)
+    snncv(Xpad, W, Params)                   -> Y[2B, Nh, Nw, Kc]
+    snncv_grad(grad, Xpad, W, Params, Y)     -> (dXpad, dW, dParams)
+
+``SnnFc`` / ``SnnCv`` are the autograd bindings that replace ``@ops.RegisterGradient``.
+Tensors must be float32 on a ROCm device; ``Params`` is the host-side float32 vector the layers
+build.  PyTorch only supplies device memory and the current HIP stream.
+"""
+import ctypes
+
+import numpy as np
+import torch
+
+from . import _lib
+
+_workspaces = {}
+
+
+def _params(params, n):
+    p = np.ascontiguousarray(np.asarray(params, dtype=np.float32).reshape(-1))
+    if p.size != n:
+        raise ValueError(f"Params must hold {n} float32 values, got {p.size}")
+    return p, p.ctypes.data_as(ctypes.POINTER(ctypes.c_float))
+
+
+def _dev_f32(t, name, ndim):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise _lib.SnntcLibraryError(
+            f"{name} lives on {t.device}: the SNN-TC ops run on a ROCm GPU only (no CPU fallback)")
+    if t.dtype != torch.float32:
+        raise TypeError(f"{name} must be float32, got {t.dtype}")
+    if t.dim() != ndim:
+        raise ValueError(f"{name} must have {ndim} dimensions, got shape {tuple(t.shape)}")
+    return t.contiguous()
+
+
+def _workspace(device, nbytes):
+    """Grow-only scratch buffer per (device, stream); contents never outlive one op call."""
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+def _stream(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def snnfc(X, W, Params, return_aux=False):
+    """Dense forward.  X[B,I], W[I+bias,J] -> Y[2B,J] (spike times ; 1/(sum w - theta)).
+    With return_aux=True also returns (sorted_z[B,I], perm[B,I] int32, causal_k[B,J] int32)."""
+    lib = _lib.load()
+    X = _dev_f32(X, "X", 2)
+    W = _dev_f32(W, "W", 2)
+    p, pp = _params(Params, 6)
+    B, I = X.shape
+    w_rows, J = W.shape
+    with torch.cuda.device(X.device):
+        need = ctypes.c_size_t()
+        _lib.check(lib.snntc_fc_forward_workspace_bytes(B, I, J, ctypes.byref(need)))
+        ws = _workspace(X.device, need.value)
+        out = torch.empty((2 * B, J), dtype=torch.float32, device=X.device)
+        if return_aux:
+            sz = torch.empty((B, I), dtype=torch.float32, device=X.device)
+            perm = torch.empty((B, I), dtype=torch.int32, device=X.device)
+            ck = torch.empty((B, J), dtype=torch.int32, device=X.device)
+            _lib.check(lib.snntc_fc_forward_ex(_ptr(X), _ptr(W), pp, _ptr(out), _ptr(sz), _ptr(perm), _ptr(ck),
+                                               B, I, J, w_rows, _ptr(ws), ws.numel(), _stream(X.device)))
+            return out, sz, perm, ck
+        _lib.check(lib.snntc_fc_forward(_ptr(X), _ptr(W), pp, _ptr(out), B, I, J, w_rows, _ptr(ws), ws.numel(),
+                                        _stream(X.device)))
+    return out
+
+
+def snnfc_grad(grad, X, W, Params, Y):
+    """Dense backward.  grad[2B,J], Y[2B,J] = forward output -> (dX[B,I], dW like W, dParams[6])."""
+    lib = _lib.load()
+    grad = _dev_f32(grad, "grad", 2)
+    X = _dev_f32(X, "X", 2)
+    W = _dev_f32(W, "W", 2)
+    Y = _dev_f32(Y, "Y", 2)
+    p, pp = _params(Params, 6)
+    B, I = X.shape
+    w_rows, J = W.shape
+    if Y.shape[0] != 2 * B or Y.shape[1] != J or grad.shape[1] != J:
+        raise ValueError(f"Grad/Oldout batch should be 2 * batch: Y {tuple(Y.shape)}, grad {tuple(grad.shape)}, "
+                         f"X {tuple(X.shape)}, W {tuple(W.shape)}")
+    with torch.cuda.device(X.device):
+        need = ctypes.c_size_t()
+        _lib.check(lib.snntc_fc_backward_workspace_bytes(B, I, J, ctypes.byref(need)))
+        ws = _workspace(X.device, need.value)
+        dX = torch.empty_like(X)
+        dW = torch.empty_like(W)
+        dP = torch.empty(6, dtype=torch.float32, device=X.device)
+        _lib.check(lib.snntc_fc_backward(_ptr(grad), _ptr(X), _ptr(W), pp, _ptr(Y), _ptr(dX), _ptr(dW), _ptr(dP),
+                                         B, I, J, w_rows, grad.shape[0], _ptr(ws), ws.numel(), _stream(X.device)))
+    return dX, dW, dP
+
+
+def snncv_output_dims(H, W, Params):
+    lib = _lib.load()
+    p, pp = _params(Params, 12)
+    nh, nw = ctypes.c_int64(), ctypes.c_int64()
+    _lib.check(lib.snntc_cv_output_dims(H, W, pp, ctypes.byref(nh), ctypes.byref(nw)))
+    return nh.value, nw.value
+
+
+def snncv(X, W, Params, return_aux=False):
+    """Conv forward on the already padded / cropped NHWC input X[B,H,W,C]; W[Kh*Kw*C+bias,Kc]
+    -> Y[2B,Nh,Nw,Kc].  With return_aux=True also returns per-patch (sorted_z, perm, causal_k)."""
+    lib = _lib.load()
+    X = _dev_f32(X, "X", 4)
+    W = _dev_f32(W, "W", 2)
+    p, pp = _params(Params, 12)
+    B, H, Wd, C = X.shape
+    w_rows, Kc = W.shape
+    Nh, Nw = snncv_output_dims(H, Wd, p)
+    with torch.cuda.device(X.device):
+        need = ctypes.c_size_t()
+        _lib.check(lib.snntc_cv_forward_workspace_bytes(B, H, Wd, C, Kc, pp, ctypes.byref(need)))
+        ws = _workspace(X.device, need.value)
+        out = torch.empty((2 * B, Nh, Nw, Kc), dtype=torch.float32, device=X.device)
+        if return_aux:
+            S, P = B * Nh * Nw, int(p[6]) * int(p[7]) * C
+            sz = torch.empty((S, P), dtype=torch.float32, device=X.device)
+            perm = torch.empty((S, P), dtype=torch.int32, device=X.device)
+            ck = torch.empty((S, Kc), dtype=torch.int32, device=X.device)
+            _lib.check(lib.snntc_cv_forward_ex(_ptr(X), _ptr(W), pp, _ptr(out), _ptr(sz), _ptr(perm), _ptr(ck),
+                                               B, H, Wd, C, Kc, w_rows, _ptr(ws), ws.numel(), _stream(X.device)))
+            return out, sz, perm, ck
+        _lib.check(lib.snntc_cv_forward(_ptr(X), _ptr(W), pp, _ptr(out), B, H, Wd, C, Kc, w_rows, _ptr(ws),
+                                        ws.numel(), _stream(X.device)))
+    return out
+
+
+def snncv_grad(grad, X, W, Params, Y):
+    """Conv backward -> (dXpad like X, dW like W, dParams[12])."""
+    lib = _lib.load()
+    grad = _dev_f32(grad, "grad", 4)
+    X = _dev_f32(X, "X", 4)
+    W = _dev_f32(W, "W", 2)
+    Y = _dev_f32(Y, "Y", 4)
+    p, pp = _params(Params, 12)
+    B, H, Wd, C = X.shape
+    w_rows, Kc = W.shape
+    if Y.shape[0] != 2 * B or tuple(grad.shape[1:]) != tuple(Y.shape[1:]) or Y.shape[3] != Kc:
+        raise ValueError(f"Grad/Oldout batch should be 2 * batch: Y {tuple(Y.shape)}, grad {tuple(grad.shape)}, "
+                         f"X {tuple(X.shape)}, W {tuple(W.shape)}")
+    with torch.cuda.device(X.device):
+        need = ctypes.c_size_t()
+        _lib.check(lib.snntc_cv_backward_workspace_bytes(B, H, Wd, C, Kc, pp, ctypes.byref(need)))
+        ws = _workspace(X.device, need.value)
+        dX = torch.empty_like(X)
+        dW = torch.empty_like(W)
+        dP = torch.empty(12, dtype=torch.float32, device=X.device)
+        _lib.check(lib.snntc_cv_backward(_ptr(grad), _ptr(X), _ptr(W), pp, _ptr(Y), _ptr(dX), _ptr(dW), _ptr(dP),
+                                         B, H, Wd, C, Kc, w_rows, grad.shape[0], _ptr(ws), ws.numel(),
+                                         _stream(X.device)))
+    return dX, dW, dP
+
+
+class SnnFc(torch.autograd.Function):
+    """Y = snnfc(X, W, Params) with the gradient the reference registers for "SnnFc"
+    (SNN_TC_Modules.py:31-33): the backward op receives the full [2B,J] forward output."""
+
+    @staticmethod
+    def forward(ctx, X, W, Params):
+        Y = snnfc(X, W, Params)
+        ctx.save_for_backward(X, W, Y)
+        ctx.params = np.array(Params, dtype=np.float32, copy=True)
+        return Y
+
+    @staticmethod
+    def backward(ctx, grad):
+        X, W, Y = ctx.saved_tensors
+        dX, dW, _ = snnfc_grad(grad.contiguous(), X, W, ctx.params, Y)
+        return dX, dW, None
+
+
+class SnnCv(torch.autograd.Function):
+    """Y = snncv(Xpad, W, Params) with the gradient registered for "SnnCv" (SNN_TC_Modules.py:91-93)."""
+
+    @staticmethod
+    def forward(ctx, X, W, Params):
+        Y = snncv(X, W, Params)
+        ctx.save_for_backward(X, W, Y)
+        ctx.params = np.array(Params, dtype=np.float32, copy=True)
+        return Y
+
+    @staticmethod
+    def backward(ctx, grad):
+        X, W, Y = ctx.saved_tensors
+        dX, dW, _ = snncv_grad(grad.contiguous(), X, W, ctx.params, Y)
+        return dX, dW, None

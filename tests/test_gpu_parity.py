@@ -1,0 +1,122 @@
+"""GPU parity: the HIP library (through the Python ops, i.e. through the C ABI) against the CPU
+oracle on the same seeded inputs.
+
+Bars: sorted values, permutations and causal-set sizes bit-exact; spike times and reciprocals
+bit-exact (the scan reproduces the oracle's fp32 operation order); gradients within
+rel 1e-5 / abs 1e-6 of the oracle, where for sums the absolute term scales with the sum of the
+absolute summands (two fp32 summation orders of the same terms differ by that much).
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_close, conv_case, dense_case
+from oracle import capi
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def t(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def grad_tolerances(ref_abs):
+    """abs tolerance per element = 1e-6 * max(1, sum of |summands|)."""
+    return 1e-6 * np.maximum(1.0, np.abs(ref_abs))
+
+
+def check_grad(actual, ref, ref_abs, what):
+    a = np.asarray(actual, np.float64); e = np.asarray(ref, np.float64)
+    lim = 1e-5 * np.abs(e) + grad_tolerances(ref_abs)
+    err = np.abs(a - e)
+    bad = err > lim
+    if bad.any():
+        idx = np.unravel_index(np.argmax(err - lim), err.shape)
+        raise AssertionError(f"{what}: {bad.sum()}/{bad.size} out of tolerance; worst {idx}: got {a[idx]!r} "
+                             f"want {e[idx]!r} diff {err[idx]:.3e} lim {lim[idx]:.3e}")
+
+
+DENSE_CASES = [
+    # seed, B, I, J, bias, dist
+    (0, 128, 784, 800, True, "baseline"),      # BASELINE config 1
+    (1, 128, 784, 800, False, "baseline"),
+    (2, 32, 800, 10, True, "baseline"),        # classifier head: J < one wavefront
+    (3, 7, 1, 3, True, "reftest"),             # shortest possible segment
+    (4, 5, 33, 65, False, "reftest"),
+    (5, 19, 257, 129, True, "reftest"),
+    (6, 3, 1000, 70, True, "reftest"),
+    (7, 4, 2048, 96, True, "baseline"),        # cross-wavefront sort
+    (8, 2, 5000, 40, False, "reftest"),        # 8192-wide sort
+]
+
+
+@pytest.mark.parametrize("seed,B,I,J,bias,dist", DENSE_CASES)
+def test_dense_forward_backward(seed, B, I, J, bias, dist):
+    import snntc_amd as snn
+    x, w, p, g = dense_case(seed, B, I, J, bias, dist)
+    ref_out, ref_k, ref_sorted, ref_perm = capi.fc_forward_dev(x, w, p, want_aux=True)
+    out, sz, perm, ck = snn.snnfc(t(x), t(w), p, return_aux=True)
+    out2 = snn.snnfc(t(x), t(w), p)
+    torch.cuda.synchronize()
+    out, sz, perm, ck, out2 = (v.cpu().numpy() for v in (out, sz, perm, ck, out2))
+    assert np.array_equal(sz, ref_sorted), "sorted values differ"
+    assert np.array_equal(perm, ref_perm), "permutation differs"
+    assert np.array_equal(ck, ref_k), f"causal-set sizes differ at {np.argwhere(ck != ref_k)[:5]}"
+    assert np.array_equal(out.view(np.uint32), ref_out.view(np.uint32)), "y / 1/S not bit-exact"
+    assert np.array_equal(out2.view(np.uint32), out.view(np.uint32)), "plain and _ex entry points differ"
+
+    dx, dw, dp = snn.snnfc_grad(t(g), t(x), t(w), p, t(ref_out))
+    torch.cuda.synchronize()
+    dx, dw, dp = dx.cpu().numpy(), dw.cpu().numpy(), dp.cpu().numpy()
+    rdx, rdw, _ = capi.fc_backward_dev(g, x, w, p, ref_out, wide=True)
+    absout = ref_out.copy(); absout[B:] = np.abs(absout[B:])
+    adx, adw, _ = capi.fc_backward_dev(np.abs(g), x, np.abs(w), p, absout, wide=True)
+    check_grad(dx, rdx, adx, "dX")
+    check_grad(dw, rdw, adw, "dW")
+    assert np.all(dp == 0)
+    # the fp32 sequential oracle must sit inside the same band
+    sdx, sdw, _ = capi.fc_backward_dev(g, x, w, p, ref_out)
+    check_grad(sdx, rdx, adx * 8, "oracle fp32 dX")
+    check_grad(sdw, rdw, adw * 8, "oracle fp32 dW")
+
+
+CONV_CASES = [
+    # seed, B, H, W, C, Kc, Kh, Kw, Sh, Sw, same, bias, dist
+    (0, 2, 32, 32, 64, 64, 3, 3, 1, 1, True, True, "baseline"),     # BASELINE config 3 shape, small batch
+    (1, 4, 32, 32, 3, 32, 3, 3, 1, 1, True, True, "baseline"),      # first CIFAR layer, P = 27
+    (2, 2, 16, 16, 32, 64, 3, 3, 1, 1, True, False, "baseline"),
+    (3, 2, 29, 23, 3, 16, 7, 7, 2, 2, True, True, "baseline"),      # 7x7 stride 2
+    (4, 3, 11, 13, 5, 7, 2, 4, 3, 1, False, True, "reftest"),       # VALID, ragged everything
+    (5, 2, 9, 9, 4, 70, 5, 6, 2, 3, True, False, "reftest"),
+    (6, 1, 8, 8, 128, 128, 3, 3, 1, 1, True, True, "baseline"),     # P = 1152
+    (7, 1, 4, 4, 512, 96, 3, 3, 1, 1, True, True, "baseline"),      # P = 4608
+]
+
+
+@pytest.mark.parametrize("seed,B,H,W,C,Kc,Kh,Kw,Sh,Sw,same,bias,dist", CONV_CASES)
+def test_conv_forward_backward(seed, B, H, W, C, Kc, Kh, Kw, Sh, Sw, same, bias, dist):
+    import snntc_amd as snn
+    _, xpad, w, p, g = conv_case(seed, B, H, W, C, Kc, Kh, Kw, Sh, Sw, same, bias, dist)
+    ref_out, ref_k, ref_sorted, ref_perm = capi.cv_forward_dev(xpad, w, p, want_aux=True)
+    out, sz, perm, ck = snn.snncv(t(xpad), t(w), p, return_aux=True)
+    out2 = snn.snncv(t(xpad), t(w), p)
+    torch.cuda.synchronize()
+    out, sz, perm, ck, out2 = (v.cpu().numpy() for v in (out, sz, perm, ck, out2))
+    assert out.shape == ref_out.shape
+    assert np.array_equal(sz, ref_sorted), "sorted values differ"
+    assert np.array_equal(perm, ref_perm), "permutation differs"
+    assert np.array_equal(ck, ref_k), "causal-set sizes differ"
+    assert np.array_equal(out.view(np.uint32), ref_out.view(np.uint32)), "y / 1/S not bit-exact"
+    assert np.array_equal(out2.view(np.uint32), out.view(np.uint32))
+
+    dx, dw, dp = snn.snncv_grad(t(g), t(xpad), t(w), p, t(ref_out))
+    torch.cuda.synchronize()
+    dx, dw, dp = dx.cpu().numpy(), dw.cpu().numpy(), dp.cpu().numpy()
+    rdx, rdw, _ = capi.cv_backward_dev(g, xpad, w, p, ref_out, wide=True)
+    absout = ref_out.copy(); absout[B:] = np.abs(absout[B:])
+    adx, adw, _ = capi.cv_backward_dev(np.abs(g), xpad, np.abs(w), p, absout, wide=True)
+    check_grad(dx, rdx, adx, "dXpad")
+    check_grad(dw, rdw, adw, "dW")
+    assert np.all(dp == 0)
