@@ -147,6 +147,21 @@ SNNTC_API int snntc_cv_backward(const float* grad, const float* xpad, const floa
                       int64_t B, int64_t H, int64_t W, int64_t C, int64_t Kc, int64_t w_rows,
                       int64_t grad_rows, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Per-kernel timing (no counterpart in the reference, which only times whole scripts with
+ * time.time()).  While enabled, every kernel the library launches is bracketed by a pair of HIP
+ * events on its launch stream; this is the only process-wide state the library keeps and it is
+ * off by default.
+ *   snntc_profile_enable(1|0)  clear the totals and switch timing on / off
+ *   snntc_profile_collect()    wait for the recorded events, fold them into per-kernel totals and
+ *                              return the number of distinct kernels seen (>= 0)
+ *   snntc_profile_entry(i,...) name, launch count and summed duration (ms) of kernel i; `name`
+ *                              stays valid until the next collect/enable call
+ * ------------------------------------------------------------------------------------------- */
+SNNTC_API int snntc_profile_enable(int on);
+SNNTC_API int snntc_profile_collect(void);
+SNNTC_API int snntc_profile_entry(int index, const char** name, int64_t* launches, double* total_ms);
+
 #ifdef __cplusplus
 }
 #endif

@@ -5,11 +5,59 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
 #include "snntc_common.h"
 
 namespace snntc {
 
 static thread_local char g_last_error[512] = "";
+
+// ---- opt-in kernel timer ---------------------------------------------------------------------
+namespace {
+struct TimedLaunch { const char* name; hipEvent_t start, stop; };
+struct TimerTotals { int64_t launches = 0; double ms = 0.0; };
+std::mutex g_prof_mutex;
+bool g_prof_enabled = false;
+std::vector<TimedLaunch> g_prof_pending;
+std::map<std::string, TimerTotals> g_prof_totals;
+std::vector<std::pair<std::string, TimerTotals>> g_prof_snapshot;
+
+// Waits for every pending event pair and folds it into the totals.  Caller holds the mutex.
+void prof_drain() {
+    for (TimedLaunch& t : g_prof_pending) {
+        float ms = 0.0f;
+        if (hipEventSynchronize(t.stop) == hipSuccess && hipEventElapsedTime(&ms, t.start, t.stop) == hipSuccess) {
+            TimerTotals& tot = g_prof_totals[t.name];
+            tot.launches += 1;
+            tot.ms += ms;
+        }
+        (void)hipEventDestroy(t.start);
+        (void)hipEventDestroy(t.stop);
+    }
+    g_prof_pending.clear();
+}
+}  // namespace
+
+KernelTimerScope::KernelTimerScope(const char* name, hipStream_t st) : slot(-1), stream(st) {
+    if (!g_prof_enabled) return;
+    std::lock_guard<std::mutex> lock(g_prof_mutex);
+    TimedLaunch t{name, nullptr, nullptr};
+    if (hipEventCreate(&t.start) != hipSuccess) return;
+    if (hipEventCreate(&t.stop) != hipSuccess) { (void)hipEventDestroy(t.start); return; }
+    (void)hipEventRecord(t.start, stream);
+    g_prof_pending.push_back(t);
+    slot = (int)g_prof_pending.size() - 1;
+}
+
+KernelTimerScope::~KernelTimerScope() {
+    if (slot < 0) return;
+    std::lock_guard<std::mutex> lock(g_prof_mutex);
+    if (slot < (int)g_prof_pending.size()) (void)hipEventRecord(g_prof_pending[slot].stop, stream);
+}
 
 int fail(int code, const char* fmt, ...) {
     va_list ap;
@@ -208,6 +256,32 @@ const char* snntc_status_string(int status) {
         case SNNTC_ERR_HIP: return "HIP runtime error";
         default: return "unknown status";
     }
+}
+
+int snntc_profile_enable(int on) {
+    std::lock_guard<std::mutex> lock(g_prof_mutex);
+    prof_drain();
+    g_prof_totals.clear();
+    g_prof_snapshot.clear();
+    g_prof_enabled = on != 0;
+    return SNNTC_OK;
+}
+
+int snntc_profile_collect(void) {
+    std::lock_guard<std::mutex> lock(g_prof_mutex);
+    prof_drain();
+    g_prof_snapshot.assign(g_prof_totals.begin(), g_prof_totals.end());
+    return (int)g_prof_snapshot.size();
+}
+
+int snntc_profile_entry(int index, const char** name, int64_t* launches, double* total_ms) {
+    std::lock_guard<std::mutex> lock(g_prof_mutex);
+    if (index < 0 || index >= (int)g_prof_snapshot.size())
+        return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_profile_entry: index %d out of range", index);
+    if (name) *name = g_prof_snapshot[index].first.c_str();
+    if (launches) *launches = g_prof_snapshot[index].second.launches;
+    if (total_ms) *total_ms = g_prof_snapshot[index].second.ms;
+    return SNNTC_OK;
 }
 
 int snntc_fc_forward_workspace_bytes(int64_t B, int64_t I, int64_t J, size_t* bytes) {

@@ -249,8 +249,10 @@ int blocks_for(int64_t n, int block) { return (int)((n + block - 1) / block); }
 int launch_prep_upstream(const float* grad, const float* y, const float* rcp, float* upm, float* ym,
                          int64_t n, const NeuronParams& np, hipStream_t stream) {
     if (n <= 0) return SNNTC_OK;
+    { KernelTimerScope timer_("prep_upstream", stream);
     hipLaunchKernelGGL(prep_upstream_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream, grad, y, rcp,
                        upm, ym, n, np.max_cmp);
+    }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
 }
@@ -258,14 +260,18 @@ int launch_prep_upstream(const float* grad, const float* y, const float* rcp, fl
 int launch_transpose(const float* w, float* wt, int64_t rows, int64_t cols, hipStream_t stream) {
     if (rows <= 0 || cols <= 0) return SNNTC_OK;
     dim3 grid((unsigned)((cols + 31) / 32), (unsigned)((rows + 31) / 32));
+    { KernelTimerScope timer_("transpose_w", stream);
     hipLaunchKernelGGL(transpose_kernel, grid, dim3(256), 0, stream, w, wt, (int)rows, (int)cols);
+    }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
 }
 
 int launch_fill_zero(float* p, int64_t n, hipStream_t stream) {
     if (n <= 0) return SNNTC_OK;
+    { KernelTimerScope timer_("fill_zero", stream);
     hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream, p, n);
+    }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
 }
@@ -276,8 +282,10 @@ int launch_fc_grad_input(const float* x, const float* wt, const float* upm, cons
     if (J <= 0) return launch_fill_zero(dx, B * I, stream);
     dim3 grid((unsigned)((B + DX_RB - 1) / DX_RB), (unsigned)((I + kWave - 1) / kWave));
     if (grid.y > 65535u) return fail(SNNTC_ERR_TOO_LARGE, "dense backward: input size %lld too large", (long long)I);
+    { KernelTimerScope timer_("fc_grad_input", stream);
     hipLaunchKernelGGL(fc_grad_input_kernel, grid, dim3(256), 0, stream, x, wt, upm, ym, dx, (int)B, (int)I,
                        (int)J, (int)wt_stride);
+    }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
 }
@@ -305,13 +313,17 @@ int launch_grad_weight(const SegmentSource& src, const float* upm, const float* 
     dim3 grid((unsigned)((J + kWave - 1) / kWave), (unsigned)((rows + DW_RI - 1) / DW_RI), (unsigned)nsplit);
     if (grid.y > 65535u) return fail(SNNTC_ERR_TOO_LARGE, "weight gradient: too many weight rows");
     float* dst = nsplit > 1 ? partial : dw;
+    { KernelTimerScope timer_("grad_weight", stream);
     hipLaunchKernelGGL(grad_weight_kernel, grid, dim3(256), 0, stream, src, upm, ym, dst, (int)S, (int)J,
                        (int)rows, seg_per_slice, np.biasvolt);
+    }
     SNNTC_HIP_CHECK(hipGetLastError());
     if (nsplit > 1) {
         const int64_t n = rows * J;
+        { KernelTimerScope timer_("reduce_partials", stream);
         hipLaunchKernelGGL(reduce_partials_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream, partial, dw,
                            n, nsplit);
+        }
         SNNTC_HIP_CHECK(hipGetLastError());
     }
     return SNNTC_OK;
@@ -322,9 +334,11 @@ int launch_cv_grad_input(const float* xpad, const float* wt, const float* upm, c
     const int64_t n = g.B * g.H * g.W * g.C;
     if (n <= 0) return SNNTC_OK;
     if (g.Kc <= 0 || g.S <= 0) return launch_fill_zero(dxpad, n, stream);
+    { KernelTimerScope timer_("cv_grad_input", stream);
     hipLaunchKernelGGL(cv_grad_input_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream, xpad, wt, upm, ym,
                        dxpad, n, (int)g.H, (int)g.W, (int)g.C, (int)g.Kc, (int)g.Kh, (int)g.Kw, (int)g.Sh,
                        (int)g.Sw, (int)g.Nh, (int)g.Nw, (int)wt_stride);
+    }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
 }

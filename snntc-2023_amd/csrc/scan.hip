@@ -117,12 +117,15 @@ int launch_scan(const float* sorted, const int32_t* perm, const float* w, float*
     const int64_t blocks = (n_items + waves_per_block - 1) / waves_per_block;
     if (blocks > 0x7fffffffLL) return fail(SNNTC_ERR_TOO_LARGE, "scan: grid too large");
     dim3 grid((unsigned)blocks), block(waves_per_block * kWave);
-    if (causal_k)
-        hipLaunchKernelGGL(scan_kernel<true>, grid, block, 0, stream, sorted, perm, w, y, rcp, causal_k,
-                           n_items, (int)S, (int)I, (int)J, j_blocks, np);
-    else
-        hipLaunchKernelGGL(scan_kernel<false>, grid, block, 0, stream, sorted, perm, w, y, rcp, causal_k,
-                           n_items, (int)S, (int)I, (int)J, j_blocks, np);
+    {
+        KernelTimerScope timer_("scan", stream);
+        if (causal_k)
+            hipLaunchKernelGGL(scan_kernel<true>, grid, block, 0, stream, sorted, perm, w, y, rcp, causal_k,
+                               n_items, (int)S, (int)I, (int)J, j_blocks, np);
+        else
+            hipLaunchKernelGGL(scan_kernel<false>, grid, block, 0, stream, sorted, perm, w, y, rcp, causal_k,
+                               n_items, (int)S, (int)I, (int)J, j_blocks, np);
+    }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
 }

@@ -26,6 +26,15 @@ int fail(int code, const char* fmt, ...);
 
 inline size_t align_up(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
 
+// Opt-in per-kernel timing (snntc_profile_*): while enabled, every launcher brackets its kernel
+// with a pair of HIP events on the launch stream.  Disabled (the default) it costs one branch.
+struct KernelTimerScope {
+    KernelTimerScope(const char* name, hipStream_t stream);
+    ~KernelTimerScope();
+    int slot;
+    hipStream_t stream;
+};
+
 // The scalar knobs every kernel needs, taken from either params layout.
 struct NeuronParams {
     float max_time;   // MAX_SPIKE_TIME

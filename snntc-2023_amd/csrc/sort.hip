@@ -147,8 +147,10 @@ int launch_sort_t(const SegmentSource& src, int64_t S, float* sorted, int32_t* p
     constexpr int SEGS = BLOCK / G;
     const int64_t blocks = (S + SEGS - 1) / SEGS;
     if (blocks > 0x7fffffffLL) return fail(SNNTC_ERR_TOO_LARGE, "sort: too many segments (%lld)", (long long)S);
+    { KernelTimerScope timer_("sort_segments", stream);
     hipLaunchKernelGGL((sort_segments_kernel<EPT, G, BLOCK>), dim3((unsigned)blocks), dim3(BLOCK), 0, stream,
                        src, sorted, perm, (int)S);
+    }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
 }

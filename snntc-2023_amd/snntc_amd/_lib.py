@@ -26,6 +26,7 @@ EXPORTS = (
     "snntc_fc_forward", "snntc_fc_forward_ex", "snntc_fc_backward",
     "snntc_cv_output_dims", "snntc_cv_forward_workspace_bytes", "snntc_cv_backward_workspace_bytes",
     "snntc_cv_forward", "snntc_cv_forward_ex", "snntc_cv_backward",
+    "snntc_profile_enable", "snntc_profile_collect", "snntc_profile_entry",
 )
 
 
@@ -85,6 +86,9 @@ def load():
     lib.snntc_cv_forward_ex.argtypes = [vp, vp, fparams, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, sz, vp]
     lib.snntc_cv_backward.argtypes = [vp, vp, vp, fparams, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64,
                                       vp, sz, vp]
+    lib.snntc_profile_enable.argtypes = [c.c_int]
+    lib.snntc_profile_collect.argtypes = []
+    lib.snntc_profile_entry.argtypes = [c.c_int, c.POINTER(c.c_char_p), c.POINTER(i64), c.POINTER(c.c_double)]
     for name in EXPORTS:
         if name not in ("snntc_version", "snntc_last_error", "snntc_status_string"):
             getattr(lib, name).restype = c.c_int
@@ -101,3 +105,20 @@ def check(status):
     if status in (ERR_DIM_MISMATCH, ERR_TOO_LARGE, ERR_BAD_ARGUMENT):
         raise ValueError(msg)
     raise SnntcError(status, msg)
+
+
+def profile_enable(on=True):
+    """Switches the library's per-kernel event timing on (clearing the totals) or off."""
+    check(load().snntc_profile_enable(1 if on else 0))
+
+
+def profile_collect():
+    """Waits for the timed launches and returns {kernel name: (launches, total milliseconds)}."""
+    lib = load()
+    n = lib.snntc_profile_collect()
+    out = {}
+    for i in range(n):
+        name, cnt, ms = ctypes.c_char_p(), ctypes.c_int64(), ctypes.c_double()
+        check(lib.snntc_profile_entry(i, ctypes.byref(name), ctypes.byref(cnt), ctypes.byref(ms)))
+        out[name.value.decode()] = (cnt.value, ms.value)
+    return out
