@@ -1,0 +1,110 @@
+"""Host-side mirror of the reference's Python layers (no GPU): constructor contracts, Params layouts,
+padding / cropping arithmetic, the stock-op layers, and the refusal to run the ops off-GPU."""
+import numpy as np
+import pytest
+import torch
+
+import snntc_amd as snn
+from oracle import closed_form as cf
+
+
+def test_dense_layer_contract():
+    l = snn.SNN_dense(in_size=7, out_size=3)
+    assert l.weight.shape == (8, 3) and l.in_size == 8 and l.out_size == 3          # bias row included
+    assert torch.all(l.weight[7] == 0)                                              # init_weight: zero bias row
+    assert l.Params.dtype == np.float32
+    assert l.Params.tolist() == [np.float32(1e5), np.float32(1e-10), 1.0, 0.0, 0.0, 1.0]   # SNN_TC_Modules.py:48-49
+    l0 = snn.SNN_dense(7, 3, biasvolt=0.0, MAX_SPIKE_TIME=50.0, Spike_Threshold=2.0, Thread_per_Block=64, Blocks=9)
+    assert l0.weight.shape == (7, 3)
+    assert l0.Params.tolist() == [50.0, np.float32(1e-10), 2.0, 64.0, 9.0, 0.0]
+    w = np.arange(24, dtype=np.float64).reshape(8, 3)
+    lw = snn.SNN_dense(7, 3, weight=w)
+    assert lw.weight.dtype == torch.float32 and np.array_equal(lw.weight.detach().numpy(), w.astype(np.float32))
+    with pytest.raises(ValueError):
+        snn.SNN_dense(7, 3, weight=np.zeros((7, 3)))                                # bias row missing
+    assert lw.name == 'fckernel'
+
+
+def test_conv_layer_contract():
+    c = snn.SNN_conv(in_channel=4, out_channel=6, kernel_sizes=(3, 2), strides=(2, 1), padding='same')
+    assert c.weight.shape == (3 * 2 * 4 + 1, 6)
+    # {MAX, tpb, blocks, eps, theta, cudaflag, Kh, Kw, Sh, Sw, SAME, biasvolt}  (SNN_TC_Modules.py:121-123)
+    assert c.Params.tolist() == [np.float32(1e5), 0, 0, np.float32(1e-10), 1, 0, 3, 2, 2, 1, 1, 1]
+    v = snn.SNN_conv(4, 6, 3, 1, padding='VALID', biasvolt=0.0)
+    assert v.weight.shape == (36, 6) and v.Params[10] == 0 and v.Params[11] == 0
+    assert v.name == 'convkernel' and v.rates == [1, 1]
+
+
+@pytest.mark.parametrize("H,W,K,S", [(32, 32, 3, 1), (224, 224, 7, 2), (9, 7, 5, 3), (8, 8, 2, 2), (5, 6, 4, 1)])
+def test_conv_same_padding_uses_max_spike_time(H, W, K, S):
+    c = snn.SNN_conv(2, 3, K, S, 'SAME')
+    x = torch.rand(2, H, W, 2) + 1
+    xp = c.prepare_input(x)
+    (t, b), (l, r) = cf.same_pad(H, K, S), cf.same_pad(W, K, S)
+    assert xp.shape == (2, H + t + b, W + l + r, 2)
+    assert torch.equal(xp[:, t:t + H, l:l + W, :], x)
+    border = torch.ones_like(xp, dtype=torch.bool); border[:, t:t + H, l:l + W, :] = False
+    assert torch.all(xp[border] == 1e5)
+    assert (xp.shape[1] - K) // S + 1 == -(-H // S)                    # op output = ceil(H/S)
+
+
+@pytest.mark.parametrize("H,W,K,S", [(32, 32, 3, 1), (10, 11, 3, 2), (9, 7, 5, 3)])
+def test_conv_valid_crops_to_whole_windows(H, W, K, S):
+    c = snn.SNN_conv(2, 3, K, S, 'VALID')
+    x = torch.rand(1, H, W, 2)
+    xp = c.prepare_input(x)
+    nh, nw = (H - K) // S + 1, (W - K) // S + 1
+    assert xp.shape == (1, (nh - 1) * S + K, (nw - 1) * S + K, 2)       # SNN_TC_Modules.py:163-166
+    assert torch.equal(xp, x[:, :xp.shape[1], :xp.shape[2], :])
+
+
+def test_costs():
+    w = np.array([[0.2, 0.9], [0.3, 0.4], [0.0, 0.0]], np.float32)
+    l = snn.SNN_dense(2, 2, weight=w)
+    assert abs(float(l.w_sum_cost().detach()) - 0.25) < 1e-7                     # mean(max(0, 1 - colsum)) = (0.5 + 0)/2
+    assert abs(float(l.l2_cost().detach()) - float(np.mean(w ** 2))) < 1e-7
+
+
+def test_min_time_pool_and_avg_pool():
+    x = torch.rand(2, 5, 7, 3) + 1
+    mp = snn.SNN_maxpool2d(2, 2, 'SAME')
+    y = mp(x)
+    assert y.shape == (2, 3, 4, 3)
+    xn = np.pad(x.numpy(), ((0, 0), (0, 1), (0, 1), (0, 0)), constant_values=1e5)
+    want = xn.reshape(2, 3, 2, 4, 2, 3).min(axis=(2, 4))               # earliest spike in each window
+    assert np.allclose(y.numpy(), want)
+    ap = snn.SNN_avgpool2d(2, 2, 'VALID')
+    ya = ap(x)
+    assert ya.shape == (2, 2, 3, 3)
+    assert np.allclose(ya.numpy(), x.numpy()[:, :4, :6].reshape(2, 2, 2, 3, 2, 3).mean(axis=(2, 4)), atol=1e-6)
+
+
+def test_lrn_matches_its_formula():
+    x = torch.rand(1, 2, 2, 6) + 1
+    y = snn.SNN_LRN(depth_radius=5, bias=2, alpha=1e-4, beta=0.75)(x).numpy()
+    sq = np.pad(x.numpy() ** 2, ((0, 0), (0, 0), (0, 0), (2, 2)), constant_values=1e5)
+    scale = 2 + 1e-4 * sum(sq[..., i:i + 6] for i in range(5))
+    assert np.allclose(y, x.numpy() / scale ** 0.75, rtol=1e-6)
+
+
+def test_loss_is_cross_entropy_on_negated_times():
+    logit = torch.tensor([[1.0, 2.0, 4.0], [3.0, 1.5, 1.2]])
+    label = torch.tensor([[1.0, 0, 0], [0, 0, 1.0]])
+    want = np.mean([-np.log(np.exp(-1) / np.exp([-1, -2, -4]).sum()), -np.log(np.exp(-1.2) / np.exp([-3, -1.5, -1.2]).sum())])
+    assert abs(float(snn.loss_func(logit, label)) - want) < 1e-6
+
+
+def test_ops_refuse_cpu_tensors():
+    l = snn.SNN_dense(4, 2)
+    with pytest.raises(snn.SnntcLibraryError, match="no CPU fallback"):
+        l(torch.rand(3, 4) + 1)
+    with pytest.raises(snn.SnntcLibraryError):
+        snn.snncv(torch.rand(1, 4, 4, 1), torch.rand(10, 2), snn.SNN_conv(1, 2, 3, 1).Params)
+
+
+def test_init_weight_statistics():
+    np.random.seed(0)
+    w = snn.init_weight(400, 300, bias_volt=1.0, init_param=15.0)
+    assert w.shape == (401, 300) and w.dtype == np.float32 and np.all(w[400] == 0)
+    assert abs(w[:400].std() - np.sqrt(15.0 / 400)) < 0.005
+    assert snn.init_weight(5, 2, bias_volt=0.0).shape == (5, 2)
