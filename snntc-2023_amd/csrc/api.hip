@@ -125,14 +125,27 @@ int fc_check(int64_t B, int64_t I, int64_t J, int64_t w_rows, const float* param
     return SNNTC_OK;
 }
 
-struct FcFwdWs { float* sorted; int32_t* perm; size_t bytes; };
+struct FcFwdWs { float* sorted; int32_t* perm; int32_t* n_real; int64_t stride; size_t bytes; };
 FcFwdWs fc_fwd_ws(void* ws, int64_t S, int64_t I) {
     Carver c(ws);
     FcFwdWs r;
-    r.sorted = c.take<float>(S * I);
-    r.perm = c.take<int32_t>(S * I);
+    r.stride = padded_stride(I);
+    r.sorted = c.take<float>(S * r.stride);
+    r.perm = c.take<int32_t>(S * r.stride);
+    r.n_real = c.take<int32_t>(S);
     r.bytes = c.used;
     return r;
+}
+
+// sort -> (optional copy of the side outputs) -> scan, shared by the dense and the conv op
+int forward_chain(const SegmentSource& src, const FcFwdWs& ws, const float* w, float* out, float* sorted_z,
+                  int32_t* perm, int32_t* causal_k, int64_t S, int64_t I, int64_t J, const NeuronParams& np,
+                  hipStream_t st) {
+    int rc = launch_sort(src, S, ws.sorted, ws.perm, ws.n_real, (int)ws.stride, np.max_cmp, st);
+    if (rc) return rc;
+    rc = launch_unpad_rows(ws.sorted, ws.perm, sorted_z, perm, S, I, ws.stride, st);
+    if (rc) return rc;
+    return launch_scan(ws.sorted, ws.perm, ws.n_real, w, out, out + S * J, causal_k, S, I, ws.stride, J, np, st);
 }
 
 struct BwdWs { float* upm; float* ym; float* wt; float* partial; int nsplit; size_t bytes; };
@@ -160,13 +173,9 @@ int fc_forward_impl(const float* x, const float* w, const float* params, float* 
     if (rc) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const NeuronParams np = neuron_params(params[0], params[2], params[5]);
-    float* sorted = sorted_z ? sorted_z : ws.sorted;
-    int32_t* order = perm ? perm : ws.perm;
     SegmentSource src{};
     src.base = x; src.conv = 0; src.I = (int)I;
-    rc = launch_sort(src, B, sorted, order, st);
-    if (rc) return rc;
-    return launch_scan(sorted, order, w, out, out + B * J, causal_k, B, I, J, np, st);
+    return forward_chain(src, ws, w, out, sorted_z, perm, causal_k, B, I, J, np, st);
 }
 
 // ---- conv --------------------------------------------------------------------------------------
@@ -227,11 +236,7 @@ int cv_forward_impl(const float* xpad, const float* w, const float* params, floa
     if (rc) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const NeuronParams np = neuron_params(params[0], params[4], params[11]);
-    float* sorted = sorted_z ? sorted_z : ws.sorted;
-    int32_t* order = perm ? perm : ws.perm;
-    rc = launch_sort(conv_source(xpad, g), g.S, sorted, order, st);
-    if (rc) return rc;
-    return launch_scan(sorted, order, w, out, out + g.S * Kc, causal_k, g.S, g.P, Kc, np, st);
+    return forward_chain(conv_source(xpad, g), ws, w, out, sorted_z, perm, causal_k, g.S, g.P, Kc, np, st);
 }
 
 }  // namespace

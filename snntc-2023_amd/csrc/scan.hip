@@ -8,10 +8,12 @@
 // |ysum| > x*|wsum| with the product rounded on its own, and y = ysum * (1/wsum).
 //
 // Mapping: one wavefront per (segment, block of 64 neurons); lanes run across neurons, so the
-// weight row w[perm[k], j0..j0+63] is one coalesced 256-byte read and the sorted value / index
-// of step k are the same for every lane (fetched through the scalar path).  Steps are taken in
-// chunks of CHUNK so the weight reads of a chunk are in flight together; lanes that have closed
-// their causal set idle until the whole wavefront has, then the wavefront leaves the loop.
+// weight row w[perm[k], j0..j0+63] is one coalesced 256-byte read, while the sorted value and the
+// row index of step k are the same for every lane and travel through the scalar path, eight steps
+// per fetch (segment rows are padded to a multiple of 16 entries).  The weights of the next eight
+// steps are requested while the current eight are consumed.  A lane that has closed its causal set
+// drops out of the loop (it is masked off and issues no further reads); the wavefront leaves when
+// its last lane has.
 #include "snntc_common.h"
 
 namespace snntc {
@@ -19,12 +21,29 @@ namespace {
 
 constexpr int CHUNK = 8;
 
+struct LaneState {
+    float wsum, ysum, wa, ya;
+    bool fired;
+};
+
+// One scan step for a lane that is still open.  Returns false when the causal set closes before
+// consuming input x (the lane then keeps its state).
+__device__ __forceinline__ bool scan_step(LaneState& s, float x, float wv) {
+    if (s.fired && s.ya <= x * s.wa) return false;
+    s.wsum += wv;
+    s.ysum = __fmaf_rn(x, wv, s.ysum);
+    s.wa = fabsf(s.wsum);
+    s.ya = s.wsum < 0.0f ? -s.ysum : s.ysum;
+    s.fired = s.ya > x * s.wa;
+    return true;
+}
+
 template <bool WANT_K>
 __global__ void __launch_bounds__(256)
 scan_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
-            const float* __restrict__ w, float* __restrict__ y_out, float* __restrict__ rcp_out,
-            int32_t* __restrict__ k_out, int64_t n_items, int S, int I, int J, int j_blocks,
-            NeuronParams np) {
+            const int32_t* __restrict__ n_real, const float* __restrict__ w, float* __restrict__ y_out,
+            float* __restrict__ rcp_out, int32_t* __restrict__ k_out, int64_t n_items, int I, int stride,
+            int J, int j_blocks, NeuronParams np) {
     // work item = (segment, 64-neuron block); one per wavefront
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int64_t item = (int64_t)blockIdx.x * (blockDim.x / kWave) + wave;
@@ -34,83 +53,337 @@ scan_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
     const int lane = threadIdx.x % kWave;
     const int j = jb * kWave + lane;
     const bool active = j < J;
-    const int jc = active ? j : J - 1;          // clamp so every lane reads valid memory
+    const unsigned jc = (unsigned)(active ? j : J - 1);      // clamp so every lane reads valid memory
 
-    const float* __restrict__ xs = sorted + (size_t)seg * I;
-    const int32_t* __restrict__ pr = perm + (size_t)seg * I;
-    const float* __restrict__ wcol = w + jc;
+    const float* __restrict__ xs = sorted + (size_t)seg * stride;
+    const int32_t* __restrict__ pr = perm + (size_t)seg * stride;
+    const int n = n_real[seg];                                // inputs with value <= MAX-0.1
 
-    // number of real inputs: first sorted position whose value exceeds MAX-0.1 (binary search)
-    int n = 0;
-    {
-        int lo = 0, hi = I;
-        while (lo < hi) {
-            const int mid = (lo + hi) >> 1;
-            if (xs[mid] > np.max_cmp) hi = mid; else lo = mid + 1;
-        }
-        n = lo;
-    }
-
-    float wsum = -np.theta, ysum = 0.0f, wa = 0.0f, ya = 0.0f;
-    bool fired = false;
+    LaneState s;
+    s.wsum = -np.theta; s.ysum = 0.0f; s.wa = 0.0f; s.ya = 0.0f; s.fired = false;
     if (np.bias) {
-        const float wb = wcol[(size_t)I * J];
-        wsum += wb;
-        ysum = np.biasvolt * wb;
-        wa = fabsf(wsum);
-        ya = wsum < 0.0f ? -ysum : ysum;
-        fired = ya > wa * np.biasvolt;
+        const float wb = (w + (size_t)I * J)[jc];
+        s.wsum += wb;
+        s.ysum = np.biasvolt * wb;
+        s.wa = fabsf(s.wsum);
+        s.ya = s.wsum < 0.0f ? -s.ysum : s.ysum;
+        s.fired = s.ya > s.wa * np.biasvolt;
     }
 
-    bool done = !active;
     int kcnt = 0;
-    for (int k0 = 0; k0 < n; k0 += CHUNK) {
-        float xv[CHUNK], wv[CHUNK];
+    if (active) {
+        // w[row, j]: the row base is wave-uniform (scalar registers), the lane adds a 32-bit byte offset
+        const unsigned joff = jc * (unsigned)sizeof(float);
+        auto weight_at = [&](int32_t row) -> float {
+            const char* rowp = reinterpret_cast<const char*>(w + (uint32_t)row * (uint32_t)J);
+            return *reinterpret_cast<const float*>(rowp + joff);
+        };
+
+        const int n_full = n & ~(CHUNK - 1);
+        float wq[CHUNK];
 #pragma unroll
-        for (int u = 0; u < CHUNK; ++u) {
-            const int kk = min(k0 + u, n - 1);
-            xv[u] = xs[kk];
-            wv[u] = wcol[(size_t)pr[kk] * J];
-        }
+        for (int u = 0; u < CHUNK; ++u) wq[u] = weight_at(pr[u]);    // row padding keeps pr[0..15] readable
+        bool open = true;
+        for (int k0 = 0; k0 < n_full && open; k0 += CHUNK) {
+            float xv[CHUNK], wc[CHUNK];
+            const int kn = (k0 + CHUNK < n_full) ? k0 + CHUNK : k0;  // next chunk, or a harmless re-read
 #pragma unroll
-        for (int u = 0; u < CHUNK; ++u) {
-            if (k0 + u < n && !done) {
-                const float x = xv[u];
-                if (fired && ya <= x * wa) {
-                    done = true;
-                } else {
-                    wsum += wv[u];
-                    ysum = __fmaf_rn(x, wv[u], ysum);
-                    wa = fabsf(wsum);
-                    ya = wsum < 0.0f ? -ysum : ysum;
-                    fired = ya > x * wa;
-                    if (WANT_K) kcnt = k0 + u + 1;
+            for (int u = 0; u < CHUNK; ++u) {
+                xv[u] = xs[k0 + u];
+                wc[u] = wq[u];
+                wq[u] = weight_at(pr[kn + u]);
+            }
+#pragma unroll
+            for (int u = 0; u < CHUNK; ++u) {
+                if (open) {
+                    open = scan_step(s, xv[u], wc[u]);
+                    if (WANT_K && open) kcnt = k0 + u + 1;
                 }
             }
         }
-        if (__all(done)) break;
-    }
+        // up to CHUNK-1 trailing steps
+        for (int k = n_full; k < n && open; ++k) {
+            open = scan_step(s, xs[k], weight_at(pr[k]));
+            if (WANT_K && open) kcnt = k + 1;
+        }
 
-    if (active) {
         float y = np.max_time, r = 0.0f;
-        if (fired) {
-            r = 1.0f / wsum;
-            y = ysum * r;
+        if (s.fired) {
+            r = 1.0f / s.wsum;
+            y = s.ysum * r;
             if (y >= np.max_time) { y = np.max_time; r = 0.0f; }
         }
         const size_t o = (size_t)seg * J + j;
         y_out[o] = y;
         rcp_out[o] = r;
-        if (WANT_K) k_out[o] = (fired && r != 0.0f) ? kcnt : -1;
+        if (WANT_K) k_out[o] = (s.fired && r != 0.0f) ? kcnt : -1;
     }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Scan with the weight slice resident in LDS.
+//
+// Walking W rows in sorted order from memory re-reads the whole matrix once per segment (8 GB of
+// cache traffic for 65 536 patches of a 3x3x64 -> 64 layer).  Here a workgroup copies the COLS
+// columns it owns -- all I(+1) rows, at most 160 KB -- into LDS once and then scans many segments
+// against it.  A wavefront covers 64/COLS segments at a time (lanes = segment x column), so narrow
+// layers (J = 10, Kc = 32) and long segments (COLS = 8 for 4608 inputs) use the same kernel.
+// Sorted values and row indices are fetched per lane (all lanes of a segment read the same
+// address) eight steps at a time, one chunk ahead of the LDS reads that need them.
+// ---------------------------------------------------------------------------------------------
+constexpr int LDS_SCAN_THREADS = 1024;
+constexpr int LDS_SCAN_BYTES = 160 * 1024;
+constexpr int LDS_SCAN_TARGET = 80 * 1024;   // two workgroups per CU when a slice this small exists
+
+struct Chunk {
+    float x[CHUNK];
+    int32_t p[CHUNK];
+};
+
+__device__ __forceinline__ void load_chunk(Chunk& c, const float* __restrict__ xs,
+                                           const int32_t* __restrict__ pr, int k) {
+    const float4 a = *reinterpret_cast<const float4*>(xs + k);
+    const float4 b = *reinterpret_cast<const float4*>(xs + k + 4);
+    const int4 pa = *reinterpret_cast<const int4*>(pr + k);
+    const int4 pb = *reinterpret_cast<const int4*>(pr + k + 4);
+    c.x[0] = a.x; c.x[1] = a.y; c.x[2] = a.z; c.x[3] = a.w;
+    c.x[4] = b.x; c.x[5] = b.y; c.x[6] = b.z; c.x[7] = b.w;
+    c.p[0] = pa.x; c.p[1] = pa.y; c.p[2] = pa.z; c.p[3] = pa.w;
+    c.p[4] = pb.x; c.p[5] = pb.y; c.p[6] = pb.z; c.p[7] = pb.w;
+}
+
+// Eight scan steps for the lanes in `run`, written out by hand: the closing test of a step simply
+// removes the lane from EXEC for the rest of the block, so a step is eight vector instructions and
+// three mask operations with no branch.  Per step (x = input time, w = its weight):
+//     close  = fired & (ya <= x*|wsum|)          -> closed |= close ; EXEC &= ~close
+//     wsum  += w ; ysum = fma(x, w, ysum) ; ya = wsum < 0 ? -ysum : ysum
+//     fired  = ya > x*|wsum|                      (bits of lanes outside EXEC read 0)
+// `fired` bits of lanes that do not run in this block are carried across it unchanged.
+#define SNNTC_SCAN_STEP(U)                                                   \
+    "v_mul_f32_e64 %[t], %[x" #U "], |%[wsum]|\n"                            \
+    "v_cmp_le_f32_e32 vcc, %[ya], %[t]\n"                                    \
+    "s_and_b64 vcc, vcc, %[fired]\n"                                         \
+    "s_or_b64 %[closed], %[closed], vcc\n"                                   \
+    "s_andn2_b64 exec, exec, vcc\n"                                          \
+    "v_add_f32_e32 %[wsum], %[wsum], %[w" #U "]\n"                           \
+    "v_fmac_f32_e32 %[ysum], %[x" #U "], %[w" #U "]\n"                       \
+    "v_cmp_gt_f32_e32 vcc, 0, %[wsum]\n"                                     \
+    "v_cndmask_b32_e64 %[ya], %[ysum], -%[ysum], vcc\n"                      \
+    "v_mul_f32_e64 %[t], %[x" #U "], |%[wsum]|\n"                            \
+    "v_cmp_gt_f32_e64 %[fired], %[ya], %[t]\n"
+
+#define SNNTC_SCAN_COUNT "v_add_u32_e32 %[kcnt], 1, %[kcnt]\n"
+
+template <bool WANT_K>
+__device__ __forceinline__ void scan_chunk(float& wsum, float& ysum, float& ya, int& kcnt, uint64_t& fired,
+                                           uint64_t& closed, uint64_t run, const float (&x)[CHUNK],
+                                           const float (&w)[CHUNK]) {
+    uint64_t saved_exec, keep;
+    float t;
+    if (WANT_K) {
+        asm volatile(
+            "s_mov_b64 %[save], exec\n"
+            "s_andn2_b64 %[keep], %[fired], %[run]\n"
+            "s_mov_b64 exec, %[run]\n"
+            SNNTC_SCAN_STEP(0) SNNTC_SCAN_COUNT SNNTC_SCAN_STEP(1) SNNTC_SCAN_COUNT
+            SNNTC_SCAN_STEP(2) SNNTC_SCAN_COUNT SNNTC_SCAN_STEP(3) SNNTC_SCAN_COUNT
+            SNNTC_SCAN_STEP(4) SNNTC_SCAN_COUNT SNNTC_SCAN_STEP(5) SNNTC_SCAN_COUNT
+            SNNTC_SCAN_STEP(6) SNNTC_SCAN_COUNT SNNTC_SCAN_STEP(7) SNNTC_SCAN_COUNT
+            "s_or_b64 %[fired], %[fired], %[keep]\n"
+            "s_mov_b64 exec, %[save]\n"
+            : [wsum] "+v"(wsum), [ysum] "+v"(ysum), [ya] "+v"(ya), [kcnt] "+v"(kcnt), [fired] "+s"(fired),
+              [closed] "+s"(closed), [save] "=&s"(saved_exec), [keep] "=&s"(keep), [t] "=&v"(t)
+            : [run] "s"(run), [x0] "v"(x[0]), [x1] "v"(x[1]), [x2] "v"(x[2]), [x3] "v"(x[3]), [x4] "v"(x[4]),
+              [x5] "v"(x[5]), [x6] "v"(x[6]), [x7] "v"(x[7]), [w0] "v"(w[0]), [w1] "v"(w[1]), [w2] "v"(w[2]),
+              [w3] "v"(w[3]), [w4] "v"(w[4]), [w5] "v"(w[5]), [w6] "v"(w[6]), [w7] "v"(w[7])
+            : "vcc");
+    } else {
+        asm volatile(
+            "s_mov_b64 %[save], exec\n"
+            "s_andn2_b64 %[keep], %[fired], %[run]\n"
+            "s_mov_b64 exec, %[run]\n"
+            SNNTC_SCAN_STEP(0) SNNTC_SCAN_STEP(1) SNNTC_SCAN_STEP(2) SNNTC_SCAN_STEP(3)
+            SNNTC_SCAN_STEP(4) SNNTC_SCAN_STEP(5) SNNTC_SCAN_STEP(6) SNNTC_SCAN_STEP(7)
+            "s_or_b64 %[fired], %[fired], %[keep]\n"
+            "s_mov_b64 exec, %[save]\n"
+            : [wsum] "+v"(wsum), [ysum] "+v"(ysum), [ya] "+v"(ya), [fired] "+s"(fired), [closed] "+s"(closed),
+              [save] "=&s"(saved_exec), [keep] "=&s"(keep), [t] "=&v"(t)
+            : [run] "s"(run), [x0] "v"(x[0]), [x1] "v"(x[1]), [x2] "v"(x[2]), [x3] "v"(x[3]), [x4] "v"(x[4]),
+              [x5] "v"(x[5]), [x6] "v"(x[6]), [x7] "v"(x[7]), [w0] "v"(w[0]), [w1] "v"(w[1]), [w2] "v"(w[2]),
+              [w3] "v"(w[3]), [w4] "v"(w[4]), [w5] "v"(w[5]), [w6] "v"(w[6]), [w7] "v"(w[7])
+            : "vcc");
+    }
+}
+
+template <int COLS, bool WANT_K>
+__global__ void __launch_bounds__(LDS_SCAN_THREADS)
+scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
+                const int32_t* __restrict__ n_real, const float* __restrict__ w, float* __restrict__ y_out,
+                float* __restrict__ rcp_out, int32_t* __restrict__ k_out, int S, int I, int stride, int J,
+                int n_slices, int n_groups, NeuronParams np) {
+    extern __shared__ float wl[];                          // [I + bias][COLS]
+    constexpr int SEGS = kWave / COLS;                     // segments per wavefront
+    constexpr int WAVES = LDS_SCAN_THREADS / kWave;
+    const int slice = blockIdx.x % n_slices;
+    const int group = blockIdx.x / n_slices;
+    const int j0 = slice * COLS;
+    const int rows = I + np.bias;
+
+    for (int idx = threadIdx.x; idx < rows * COLS; idx += LDS_SCAN_THREADS) {
+        const int r = idx / COLS, c = idx - r * COLS;
+        wl[idx] = (j0 + c < J) ? w[(size_t)r * J + j0 + c] : 0.0f;
+    }
+    __syncthreads();
+
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int sub = lane / COLS, col = lane - sub * COLS;
+    const int j = j0 + col;
+    const float* __restrict__ wcol = wl + col;
+    const int last_chunk = stride - CHUNK;                 // start of the last readable chunk of a row
+
+    for (int item = group * WAVES + wave; item * SEGS < S; item += n_groups * WAVES) {
+        const int seg_raw = item * SEGS + sub;
+        const bool live = seg_raw < S && j < J;
+        const int seg = seg_raw < S ? seg_raw : S - 1;      // idle lanes shadow a valid segment
+        const float* __restrict__ xs = sorted + (size_t)seg * stride;
+        const int32_t* __restrict__ pr = perm + (size_t)seg * stride;
+        const int n = live ? n_real[seg] : 0;
+        const int n_full = n & ~(CHUNK - 1);
+
+        float wsum = -np.theta, ysum = 0.0f, ya = 0.0f;
+        bool fired0 = false;
+        if (np.bias) {
+            const float wb = wcol[I * COLS];
+            wsum += wb;
+            ysum = np.biasvolt * wb;
+            ya = wsum < 0.0f ? -ysum : ysum;
+            fired0 = ya > fabsf(wsum) * np.biasvolt;
+        }
+        uint64_t fired = __ballot(fired0);
+        uint64_t closed = 0;
+        int kcnt = 0;
+
+        // Three chunks of (x, row) are in flight: c is consumed, c+1 feeds the LDS reads, c+2 is
+        // being fetched.  The phase loop is unrolled so that buffer indices are compile-time.
+        Chunk xp[3];
+        float wv[2][CHUNK];
+        load_chunk(xp[0], xs, pr, 0);
+        load_chunk(xp[1], xs, pr, CHUNK <= last_chunk ? CHUNK : 0);
+#pragma unroll
+        for (int u = 0; u < CHUNK; ++u) wv[0][u] = wcol[xp[0].p[u] * COLS];
+
+        for (int k0 = 0;; k0 += 6 * CHUNK) {
+            bool stop = false;
+#pragma unroll
+            for (int ph = 0; ph < 6; ++ph) {
+                const int k = k0 + ph * CHUNK;
+                const uint64_t run = __ballot(k < n_full) & ~closed;
+                if (run == 0) { stop = true; break; }
+                const int kn = k + 2 * CHUNK;
+                load_chunk(xp[(ph + 2) % 3], xs, pr, kn <= last_chunk ? kn : 0);
+#pragma unroll
+                for (int u = 0; u < CHUNK; ++u) wv[(ph + 1) % 2][u] = wcol[xp[(ph + 1) % 3].p[u] * COLS];
+                scan_chunk<WANT_K>(wsum, ysum, ya, kcnt, fired, closed, run, xp[ph % 3].x, wv[ph % 2]);
+            }
+            if (stop) break;
+        }
+
+        // per-lane epilogue: up to CHUNK-1 trailing inputs, then the output
+        if (live) {
+            LaneState s;
+            s.wsum = wsum; s.ysum = ysum; s.wa = fabsf(wsum); s.ya = ya;
+            const bool was_closed = (closed >> lane) & 1;
+            s.fired = was_closed || ((fired >> lane) & 1);
+            bool open = !was_closed;
+            for (int k = n_full; k < n && open; ++k) {
+                open = scan_step(s, xs[k], wcol[pr[k] * COLS]);
+                if (WANT_K && open) ++kcnt;
+            }
+            float y = np.max_time, r = 0.0f;
+            if (s.fired) {
+                r = 1.0f / s.wsum;
+                y = s.ysum * r;
+                if (y >= np.max_time) { y = np.max_time; r = 0.0f; }
+            }
+            const size_t o = (size_t)seg * J + j;
+            y_out[o] = y;
+            rcp_out[o] = r;
+            if (WANT_K) k_out[o] = (s.fired && r != 0.0f) ? kcnt : -1;
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256)
+unpad_rows_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
+                  float* __restrict__ sorted_out, int32_t* __restrict__ perm_out, int64_t n, int I, int stride) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n) return;
+    const int64_t row = t / I;
+    const int col = (int)(t - row * I);
+    const size_t src = (size_t)row * stride + col;
+    if (sorted_out) sorted_out[t] = sorted[src];
+    if (perm_out) perm_out[t] = perm[src];
 }
 
 }  // namespace
 
-int launch_scan(const float* sorted, const int32_t* perm, const float* w, float* y, float* rcp,
-                int32_t* causal_k, int64_t S, int64_t I, int64_t J, const NeuronParams& np,
-                hipStream_t stream) {
+template <int COLS>
+int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_real, const float* w, float* y,
+                    float* rcp, int32_t* causal_k, int64_t S, int64_t I, int64_t stride, int64_t J,
+                    const NeuronParams& np, size_t lds_bytes, hipStream_t stream) {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        SNNTC_HIP_CHECK(hipGetDevice(&dev));
+        SNNTC_HIP_CHECK(hipGetDeviceProperties(&prop, dev));
+        cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    }
+    constexpr int SEGS = kWave / COLS, WAVES = LDS_SCAN_THREADS / kWave;
+    const int n_slices = (int)((J + COLS - 1) / COLS);
+    const int64_t items = (S + SEGS - 1) / SEGS;
+    // one resident workgroup per CU: split the segments so that slices x groups covers the chip
+    const int wgs_per_cu = lds_bytes * 2 <= (size_t)LDS_SCAN_BYTES ? 2 : 1;
+    int64_t n_groups = ((int64_t)cus * wgs_per_cu + n_slices - 1) / n_slices;
+    const int64_t max_groups = (items + WAVES - 1) / WAVES;
+    if (n_groups > max_groups) n_groups = max_groups;
+    if (n_groups < 1) n_groups = 1;
+    auto kern_k = scan_lds_kernel<COLS, true>;
+    auto kern = scan_lds_kernel<COLS, false>;
+    SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(causal_k ? kern_k : kern),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+    dim3 grid((unsigned)(n_slices * n_groups)), block(LDS_SCAN_THREADS);
+    {
+        KernelTimerScope timer_("scan", stream);
+        if (causal_k)
+            hipLaunchKernelGGL(kern_k, grid, block, lds_bytes, stream, sorted, perm, n_real, w, y, rcp, causal_k,
+                               (int)S, (int)I, (int)stride, (int)J, n_slices, (int)n_groups, np);
+        else
+            hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, sorted, perm, n_real, w, y, rcp, causal_k,
+                               (int)S, (int)I, (int)stride, (int)J, n_slices, (int)n_groups, np);
+    }
+    SNNTC_HIP_CHECK(hipGetLastError());
+    return SNNTC_OK;
+}
+
+int launch_scan(const float* sorted, const int32_t* perm, const int32_t* n_real, const float* w, float* y,
+                float* rcp, int32_t* causal_k, int64_t S, int64_t I, int64_t stride, int64_t J,
+                const NeuronParams& np, hipStream_t stream) {
     if (S <= 0 || J <= 0) return SNNTC_OK;
+    // widest column slice (8..64) whose I+bias rows fit in LDS; none fits -> stream W from memory
+    const size_t rows = (size_t)I + np.bias;
+    int cols = 64;
+    while (cols > 8 && (rows * cols * sizeof(float) > (size_t)LDS_SCAN_TARGET || cols / 2 >= J)) cols >>= 1;
+    const size_t lds_bytes = rows * cols * sizeof(float);
+    if (lds_bytes <= (size_t)LDS_SCAN_BYTES) {
+        switch (cols) {
+            case 64: return launch_scan_lds<64>(sorted, perm, n_real, w, y, rcp, causal_k, S, I, stride, J, np, lds_bytes, stream);
+            case 32: return launch_scan_lds<32>(sorted, perm, n_real, w, y, rcp, causal_k, S, I, stride, J, np, lds_bytes, stream);
+            case 16: return launch_scan_lds<16>(sorted, perm, n_real, w, y, rcp, causal_k, S, I, stride, J, np, lds_bytes, stream);
+            default: return launch_scan_lds<8>(sorted, perm, n_real, w, y, rcp, causal_k, S, I, stride, J, np, lds_bytes, stream);
+        }
+    }
     const int j_blocks = (int)((J + kWave - 1) / kWave);
     const int64_t n_items = S * j_blocks;
     const int waves_per_block = 4;
@@ -118,13 +391,26 @@ int launch_scan(const float* sorted, const int32_t* perm, const float* w, float*
     if (blocks > 0x7fffffffLL) return fail(SNNTC_ERR_TOO_LARGE, "scan: grid too large");
     dim3 grid((unsigned)blocks), block(waves_per_block * kWave);
     {
-        KernelTimerScope timer_("scan", stream);
+        KernelTimerScope timer_("scan_stream", stream);
         if (causal_k)
-            hipLaunchKernelGGL(scan_kernel<true>, grid, block, 0, stream, sorted, perm, w, y, rcp, causal_k,
-                               n_items, (int)S, (int)I, (int)J, j_blocks, np);
+            hipLaunchKernelGGL(scan_kernel<true>, grid, block, 0, stream, sorted, perm, n_real, w, y, rcp,
+                               causal_k, n_items, (int)I, (int)stride, (int)J, j_blocks, np);
         else
-            hipLaunchKernelGGL(scan_kernel<false>, grid, block, 0, stream, sorted, perm, w, y, rcp, causal_k,
-                               n_items, (int)S, (int)I, (int)J, j_blocks, np);
+            hipLaunchKernelGGL(scan_kernel<false>, grid, block, 0, stream, sorted, perm, n_real, w, y, rcp,
+                               causal_k, n_items, (int)I, (int)stride, (int)J, j_blocks, np);
+    }
+    SNNTC_HIP_CHECK(hipGetLastError());
+    return SNNTC_OK;
+}
+
+int launch_unpad_rows(const float* sorted, const int32_t* perm, float* sorted_out, int32_t* perm_out,
+                      int64_t S, int64_t I, int64_t stride, hipStream_t stream) {
+    const int64_t n = S * I;
+    if (n <= 0 || (!sorted_out && !perm_out)) return SNNTC_OK;
+    {
+        KernelTimerScope timer_("unpad_rows", stream);
+        hipLaunchKernelGGL(unpad_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, sorted,
+                           perm, sorted_out, perm_out, n, (int)I, (int)stride);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;

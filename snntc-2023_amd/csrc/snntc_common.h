@@ -59,13 +59,24 @@ struct ConvGeom {
 
 // ---- launchers (each enqueues on `stream` and returns a status) --------------------------------
 
-// Segmented stable ascending sort: sorted[S,I] and perm[S,I].
-int launch_sort(const SegmentSource& src, int64_t S, float* sorted, int32_t* perm, hipStream_t stream);
+// Row stride of the sorted / perm scratch arrays: segments are padded to a multiple of 16 entries
+// so the scan can fetch them in aligned groups without bounds checks.
+inline int64_t padded_stride(int64_t I) { return (I + 15) / 16 * 16; }
 
-// Causal-set scan over sorted segments: y[S,J], rcp[S,J], optional causal_k[S,J].
-int launch_scan(const float* sorted, const int32_t* perm, const float* w, float* y, float* rcp,
-                int32_t* causal_k, int64_t S, int64_t I, int64_t J, const NeuronParams& np,
-                hipStream_t stream);
+// Segmented stable ascending sort: sorted[S,out_stride] and perm[S,out_stride] (entries past the
+// segment length hold +inf / 0), n_real[S] = number of values <= max_cmp (may be NULL).
+int launch_sort(const SegmentSource& src, int64_t S, float* sorted, int32_t* perm, int32_t* n_real,
+                int out_stride, float max_cmp, hipStream_t stream);
+
+// Copies the first I entries of every padded row into dense [S,I] arrays (either may be NULL).
+int launch_unpad_rows(const float* sorted, const int32_t* perm, float* sorted_out, int32_t* perm_out,
+                      int64_t S, int64_t I, int64_t stride, hipStream_t stream);
+
+// Causal-set scan over sorted segments (rows of length `stride`, n_real inputs each):
+// y[S,J], rcp[S,J], optional causal_k[S,J].
+int launch_scan(const float* sorted, const int32_t* perm, const int32_t* n_real, const float* w, float* y,
+                float* rcp, int32_t* causal_k, int64_t S, int64_t I, int64_t stride, int64_t J,
+                const NeuronParams& np, hipStream_t stream);
 
 // upm = valid ? grad*rcp : 0 ; ym = valid ? y : -inf   (valid: y <= MAX-0.1), n elements each.
 int launch_prep_upstream(const float* grad, const float* y, const float* rcp, float* upm, float* ym,

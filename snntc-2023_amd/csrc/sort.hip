@@ -30,11 +30,13 @@ __device__ __forceinline__ float key_to_float(uint32_t k) {
 
 template <int EPT, int G, int BLOCK>
 __global__ void __launch_bounds__(BLOCK)
-sort_segments_kernel(SegmentSource src, float* __restrict__ sorted, int32_t* __restrict__ perm, int S) {
+sort_segments_kernel(SegmentSource src, float* __restrict__ sorted, int32_t* __restrict__ perm,
+                     int32_t* __restrict__ n_real, int S, int out_stride, float max_cmp) {
     constexpr int NPAD = EPT * G;
     constexpr int SEGS = BLOCK / G;
     constexpr bool CROSS_WAVE = G > kWave;
     __shared__ u64 xchg[CROSS_WAVE ? NPAD : 1];
+    __shared__ int wave_count[CROSS_WAVE ? G / kWave : 1];
 
     const int tseg = threadIdx.x % G;
     const int seg = blockIdx.x * SEGS + threadIdx.x / G;
@@ -126,30 +128,53 @@ sort_segments_kernel(SegmentSource src, float* __restrict__ sorted, int32_t* __r
         }
     }
 
-    // ---- store ------------------------------------------------------------------------------------
+    // ---- store: rows are out_stride long; positions past the segment get (+inf, row 0) ------------
+    int below = 0;                      // own elements that take part in the scan (value <= MAX-0.1)
     if (live) {
-        float* so = sorted + (size_t)seg * I;
-        int32_t* po = perm + (size_t)seg * I;
+        float* so = sorted + (size_t)seg * out_stride;
+        int32_t* po = perm + (size_t)seg * out_stride;
 #pragma unroll
         for (int r = 0; r < EPT; ++r) {
             const int e = tseg * EPT + r;
             if (e < I) {
-                so[e] = key_to_float((uint32_t)(v[r] >> 32));
+                const float f = key_to_float((uint32_t)(v[r] >> 32));
+                so[e] = f;
                 po[e] = (int32_t)(uint32_t)v[r];
+                below += (f <= max_cmp) ? 1 : 0;
+            } else if (e < out_stride) {
+                so[e] = INFINITY;
+                po[e] = 0;
             }
+        }
+    }
+    // ---- number of scan inputs per segment: sum of `below` over the segment's G threads -----------
+    if (n_real != nullptr) {
+#pragma unroll
+        for (int d = 1; d < (G < kWave ? G : kWave); d <<= 1) below += __shfl_xor(below, d, kWave);
+        if (CROSS_WAVE) {
+            if ((threadIdx.x % kWave) == 0) wave_count[threadIdx.x / kWave] = below;
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                int total = 0;
+                for (int wv = 0; wv < G / kWave; ++wv) total += wave_count[wv];
+                n_real[seg] = total;
+            }
+        } else if (live && tseg == 0) {
+            n_real[seg] = below;
         }
     }
 }
 
 template <int EPT, int G>
-int launch_sort_t(const SegmentSource& src, int64_t S, float* sorted, int32_t* perm, hipStream_t stream) {
+int launch_sort_t(const SegmentSource& src, int64_t S, float* sorted, int32_t* perm, int32_t* n_real,
+                  int out_stride, float max_cmp, hipStream_t stream) {
     constexpr int BLOCK = G > 256 ? G : 256;
     constexpr int SEGS = BLOCK / G;
     const int64_t blocks = (S + SEGS - 1) / SEGS;
     if (blocks > 0x7fffffffLL) return fail(SNNTC_ERR_TOO_LARGE, "sort: too many segments (%lld)", (long long)S);
     { KernelTimerScope timer_("sort_segments", stream);
     hipLaunchKernelGGL((sort_segments_kernel<EPT, G, BLOCK>), dim3((unsigned)blocks), dim3(BLOCK), 0, stream,
-                       src, sorted, perm, (int)S);
+                       src, sorted, perm, n_real, (int)S, out_stride, max_cmp);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
@@ -157,21 +182,22 @@ int launch_sort_t(const SegmentSource& src, int64_t S, float* sorted, int32_t* p
 
 }  // namespace
 
-int launch_sort(const SegmentSource& src, int64_t S, float* sorted, int32_t* perm, hipStream_t stream) {
+int launch_sort(const SegmentSource& src, int64_t S, float* sorted, int32_t* perm, int32_t* n_real,
+                int out_stride, float max_cmp, hipStream_t stream) {
     if (S <= 0 || src.I <= 0) return SNNTC_OK;
     const int I = src.I;
     if (I > kMaxSegment)
         return fail(SNNTC_ERR_UNSUPPORTED, "segment length %d exceeds the largest supported sort (%d)", I,
                     kMaxSegment);
-    if (I <= 32)   return launch_sort_t<2, 16>(src, S, sorted, perm, stream);
-    if (I <= 64)   return launch_sort_t<2, 32>(src, S, sorted, perm, stream);
-    if (I <= 128)  return launch_sort_t<2, 64>(src, S, sorted, perm, stream);
-    if (I <= 256)  return launch_sort_t<4, 64>(src, S, sorted, perm, stream);
-    if (I <= 512)  return launch_sort_t<8, 64>(src, S, sorted, perm, stream);
-    if (I <= 1024) return launch_sort_t<16, 64>(src, S, sorted, perm, stream);
-    if (I <= 2048) return launch_sort_t<8, 256>(src, S, sorted, perm, stream);
-    if (I <= 4096) return launch_sort_t<8, 512>(src, S, sorted, perm, stream);
-    return launch_sort_t<8, 1024>(src, S, sorted, perm, stream);
+    if (I <= 32)   return launch_sort_t<2, 16>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
+    if (I <= 64)   return launch_sort_t<2, 32>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
+    if (I <= 128)  return launch_sort_t<2, 64>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
+    if (I <= 256)  return launch_sort_t<4, 64>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
+    if (I <= 512)  return launch_sort_t<8, 64>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
+    if (I <= 1024) return launch_sort_t<16, 64>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
+    if (I <= 2048) return launch_sort_t<8, 256>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
+    if (I <= 4096) return launch_sort_t<8, 512>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
+    return launch_sort_t<8, 1024>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
 }
 
 }  // namespace snntc
