@@ -58,6 +58,7 @@ __global__ void __launch_bounds__(256) fill_zero_kernel(float* __restrict__ p, i
 // and are summed through LDS in a fixed order.
 // ---------------------------------------------------------------------------------------------
 constexpr int DX_RB = 4;
+constexpr int DX_UNROLL = 8;
 
 __global__ void __launch_bounds__(256)
 fc_grad_input_kernel(const float* __restrict__ x, const float* __restrict__ wt,
@@ -67,26 +68,45 @@ fc_grad_input_kernel(const float* __restrict__ x, const float* __restrict__ wt,
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int i = blockIdx.y * kWave + lane;
-    const int ic = min(i, I - 1);
+    const unsigned ic = (unsigned)min(i, I - 1);
     const int b0 = blockIdx.x * DX_RB;
 
     float xr[DX_RB], acc[DX_RB];
-    int brow[DX_RB];
+    const float* __restrict__ yrow[DX_RB];
+    const float* __restrict__ urow[DX_RB];
 #pragma unroll
     for (int r = 0; r < DX_RB; ++r) {
-        brow[r] = min(b0 + r, B - 1);
-        xr[r] = x[(size_t)brow[r] * I + ic];
+        const int brow = min(b0 + r, B - 1);
+        xr[r] = x[(size_t)brow * I + ic];
+        yrow[r] = ym + (size_t)brow * J;
+        urow[r] = upm + (size_t)brow * J;
         acc[r] = 0.0f;
     }
     const int jq = (J + 3) / 4;
     const int j_lo = wave * jq, j_hi = min(J, j_lo + jq);
-    for (int j = j_lo; j < j_hi; ++j) {
-        const float wv = wt[(size_t)j * wt_stride + ic];
+    const float* __restrict__ wcol = wt + ic;
+    int j = j_lo;
+    // DX_UNROLL columns at a time: their weights are requested together, the y / up values of the
+    // block's samples are wave-uniform and arrive through the scalar path.
+    for (; j + DX_UNROLL <= j_hi; j += DX_UNROLL) {
+        float wv[DX_UNROLL];
+#pragma unroll
+        for (int u = 0; u < DX_UNROLL; ++u) wv[u] = wcol[(size_t)(j + u) * wt_stride];
 #pragma unroll
         for (int r = 0; r < DX_RB; ++r) {
-            const float yv = ym[(size_t)brow[r] * J + j];
-            const float uv = upm[(size_t)brow[r] * J + j];
-            acc[r] = __fmaf_rn(xr[r] <= yv ? uv : 0.0f, wv, acc[r]);
+#pragma unroll
+            for (int u = 0; u < DX_UNROLL; ++u) {
+                const float t = xr[r] <= yrow[r][j + u] ? wv[u] : 0.0f;
+                acc[r] = __fmaf_rn(urow[r][j + u], t, acc[r]);
+            }
+        }
+    }
+    for (; j < j_hi; ++j) {
+        const float wv = wcol[(size_t)j * wt_stride];
+#pragma unroll
+        for (int r = 0; r < DX_RB; ++r) {
+            const float t = xr[r] <= yrow[r][j] ? wv : 0.0f;
+            acc[r] = __fmaf_rn(urow[r][j], t, acc[r]);
         }
     }
     if (wave > 0) {
@@ -111,6 +131,24 @@ fc_grad_input_kernel(const float* __restrict__ x, const float* __restrict__ wt,
 // added in slice order by reduce_partials_kernel.
 // ---------------------------------------------------------------------------------------------
 constexpr int DW_RI = 8;
+constexpr int DW_UNROLL = 4;
+
+// Source offset of weight row e relative to the segment base (dense: the column; conv: kh/kw/c).
+__device__ __forceinline__ int row_offset(const SegmentSource& src, int e) {
+    if (!src.conv) return e;
+    const int span = src.Kw * src.C;
+    const int kh = e / span;
+    return kh * src.W * src.C + (e - kh * span);
+}
+
+// Base of segment s inside the source tensor.
+__device__ __forceinline__ const float* segment_base(const SegmentSource& src, int s) {
+    if (!src.conv) return src.base + (size_t)s * src.I;
+    const int per_img = src.Nh * src.Nw;
+    const int a = s / per_img, r2 = s - a * per_img;
+    const int nh = r2 / src.Nw, nw = r2 - nh * src.Nw;
+    return src.base + ((size_t)(a * src.H + nh * src.Sh) * src.W + (size_t)nw * src.Sw) * src.C;
+}
 
 __global__ void __launch_bounds__(256)
 grad_weight_kernel(SegmentSource src, const float* __restrict__ upm, const float* __restrict__ ym,
@@ -119,26 +157,9 @@ grad_weight_kernel(SegmentSource src, const float* __restrict__ upm, const float
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int j = blockIdx.x * kWave + lane;
-    const int jc = min(j, J - 1);
+    const unsigned jc = (unsigned)min(j, J - 1);
     const int i0 = blockIdx.y * DW_RI;
     const int I = src.I;
-
-    // per-row source offsets relative to the segment base (dense: the column; conv: kh/kw/c)
-    int off[DW_RI];
-    bool is_bias[DW_RI];
-#pragma unroll
-    for (int r = 0; r < DW_RI; ++r) {
-        const int i = min(i0 + r, rows - 1);
-        is_bias[r] = i >= I;
-        const int e = min(i, I - 1);
-        if (src.conv) {
-            const int span = src.Kw * src.C;
-            const int kh = e / span;
-            off[r] = kh * src.W * src.C + (e - kh * span);
-        } else {
-            off[r] = e;
-        }
-    }
 
     const int s_begin = blockIdx.z * seg_per_slice;
     const int s_end = min(S, s_begin + seg_per_slice);
@@ -149,30 +170,54 @@ grad_weight_kernel(SegmentSource src, const float* __restrict__ upm, const float
     float acc[DW_RI];
 #pragma unroll
     for (int r = 0; r < DW_RI; ++r) acc[r] = 0.0f;
+    const float* __restrict__ ycol = ym + jc;
+    const float* __restrict__ ucol = upm + jc;
 
-    // walk (a, nh, nw) incrementally for conv sources
-    int a = 0, nh = 0, nw = 0;
-    if (src.conv && s_lo < s_hi) {
-        const int per_img = src.Nh * src.Nw;
-        a = s_lo / per_img;
-        const int r2 = s_lo - a * per_img;
-        nh = r2 / src.Nw;
-        nw = r2 - nh * src.Nw;
-    }
-    for (int s = s_lo; s < s_hi; ++s) {
-        const float* xb;
-        if (src.conv) {
-            xb = src.base + ((size_t)(a * src.H + nh * src.Sh) * src.W + (size_t)nw * src.Sw) * src.C;
-            if (++nw == src.Nw) { nw = 0; if (++nh == src.Nh) { nh = 0; ++a; } }
-        } else {
-            xb = src.base + (size_t)s * I;
+    // The RI weight rows of this block are contiguous in the source (always for dense rows, for
+    // patches when the rows share one (kh, kw)): their x values come as one scalar fetch.
+    const bool contiguous = i0 + DW_RI <= I && (!src.conv || (i0 % src.C) + DW_RI <= src.C);
+    if (contiguous) {
+        const int off0 = row_offset(src, i0);
+        int s = s_lo;
+        for (; s + DW_UNROLL <= s_hi; s += DW_UNROLL) {
+            float yv[DW_UNROLL], uv[DW_UNROLL];
+            const float* xb[DW_UNROLL];
+#pragma unroll
+            for (int u = 0; u < DW_UNROLL; ++u) {
+                yv[u] = ycol[(size_t)(s + u) * J];
+                uv[u] = ucol[(size_t)(s + u) * J];
+                xb[u] = segment_base(src, s + u) + off0;
+            }
+#pragma unroll
+            for (int u = 0; u < DW_UNROLL; ++u) {
+#pragma unroll
+                for (int r = 0; r < DW_RI; ++r)
+                    acc[r] = __fmaf_rn(fminf(xb[u][r] - yv[u], 0.0f), uv[u], acc[r]);
+            }
         }
-        const float yv = ym[(size_t)s * J + jc];
-        const float uv = upm[(size_t)s * J + jc];
+        for (; s < s_hi; ++s) {
+            const float yv = ycol[(size_t)s * J], uv = ucol[(size_t)s * J];
+            const float* xb = segment_base(src, s) + off0;
+#pragma unroll
+            for (int r = 0; r < DW_RI; ++r) acc[r] = __fmaf_rn(fminf(xb[r] - yv, 0.0f), uv, acc[r]);
+        }
+    } else {
+        int off[DW_RI];
+        bool is_bias[DW_RI];
 #pragma unroll
         for (int r = 0; r < DW_RI; ++r) {
-            const float xv = is_bias[r] ? biasvolt : xb[off[r]];
-            acc[r] = __fmaf_rn(fminf(xv - yv, 0.0f), uv, acc[r]);
+            const int i = min(i0 + r, rows - 1);
+            is_bias[r] = i >= I;
+            off[r] = row_offset(src, min(i, I - 1));
+        }
+        for (int s = s_lo; s < s_hi; ++s) {
+            const float yv = ycol[(size_t)s * J], uv = ucol[(size_t)s * J];
+            const float* xb = segment_base(src, s);
+#pragma unroll
+            for (int r = 0; r < DW_RI; ++r) {
+                const float xv = is_bias[r] ? biasvolt : xb[off[r]];
+                acc[r] = __fmaf_rn(fminf(xv - yv, 0.0f), uv, acc[r]);
+            }
         }
     }
     if (wave > 0) {
@@ -294,6 +339,7 @@ int launch_fc_grad_input(const float* x, const float* wt, const float* upm, cons
 // at least 64 segments per slice, at most 256 slices.
 int weight_grad_splits(int64_t S, int64_t rows, int64_t J) {
     const int64_t base_blocks = ((J + kWave - 1) / kWave) * ((rows + DW_RI - 1) / DW_RI);
+    if (base_blocks >= 1024) return 1;
     int64_t want = (2048 + base_blocks - 1) / (base_blocks > 0 ? base_blocks : 1);
     int64_t cap = S / 64;
     if (want > cap) want = cap;
