@@ -148,17 +148,27 @@ int forward_chain(const SegmentSource& src, const FcFwdWs& ws, const float* w, f
     return launch_scan(ws.sorted, ws.perm, ws.n_real, w, out, out + S * J, causal_k, S, I, ws.stride, J, np, st);
 }
 
-struct BwdWs { float* upm; float* ym; float* wt; float* partial; int nsplit; size_t bytes; };
-BwdWs bwd_ws(void* ws, int64_t S, int64_t rows, int64_t J) {
+// Backward scratch.  `rows` is the weight row count including a possible bias row; the partial-sum
+// area is sized for the worst case of 256 slices only when slicing can happen at all.
+struct BwdWs { float* upm; float* ym; float* wt; float* partial; int max_split; size_t bytes; };
+BwdWs bwd_ws(void* ws, int64_t S, int64_t rows, int64_t J, int64_t min_base_blocks) {
     Carver c(ws);
     BwdWs r;
     r.upm = c.take<float>(S * J);
     r.ym = c.take<float>(S * J);
     r.wt = c.take<float>(rows * J);
-    r.nsplit = weight_grad_splits(S, rows, J);
-    r.partial = c.take<float>(r.nsplit > 1 ? (int64_t)r.nsplit * rows * J : 0);
+    r.max_split = weight_grad_splits(S, min_base_blocks);
+    r.partial = c.take<float>(r.max_split > 1 ? (int64_t)r.max_split * rows * J : 0);
     r.bytes = c.used;
     return r;
+}
+
+// Smallest block count the weight-gradient launch of a conv layer can have (it decides how far the
+// patch range may be sliced): the wide kernel covers 32 rows per block, the generic one 8.
+int64_t cv_weight_base_blocks(const ConvGeom& g) {
+    const int64_t generic = grad_weight_blocks(g.P + 1, g.Kc);
+    const int64_t wide = cv_grad_weight_wide_supported(g) ? cv_grad_weight_wide_blocks(g) : generic;
+    return wide < generic ? wide : generic;
 }
 
 int fc_forward_impl(const float* x, const float* w, const float* params, float* out, float* sorted_z,
@@ -299,7 +309,7 @@ int snntc_fc_forward_workspace_bytes(int64_t B, int64_t I, int64_t J, size_t* by
 int snntc_fc_backward_workspace_bytes(int64_t B, int64_t I, int64_t J, size_t* bytes) {
     if (!bytes || B < 0 || I < 0 || J < 0)
         return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_fc_backward_workspace_bytes: bad argument");
-    *bytes = bwd_ws(nullptr, B, I + 1, J).bytes;
+    *bytes = bwd_ws(nullptr, B, I + 1, J, grad_weight_blocks(I, J)).bytes;
     return SNNTC_OK;
 }
 
@@ -334,7 +344,7 @@ int snntc_fc_backward(const float* grad, const float* x, const float* w, const f
         return launch_fill_zero(dw, w_rows * J, st);
     }
     if (!grad || !x || !w || !oldout) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_fc_backward: NULL tensor pointer");
-    BwdWs ws = bwd_ws(workspace, B, I + 1, J);
+    BwdWs ws = bwd_ws(workspace, B, I + 1, J, grad_weight_blocks(I, J));
     rc = check_workspace(workspace, workspace_bytes, ws.bytes);
     if (rc) return rc;
     const NeuronParams np = neuron_params(params_host[0], params_host[2], params_host[5]);
@@ -346,9 +356,11 @@ int snntc_fc_backward(const float* grad, const float* x, const float* w, const f
     if (rc) return rc;
     SegmentSource src{};
     src.base = x; src.conv = 0; src.I = (int)I;
-    int nsplit = weight_grad_splits(B, w_rows, J);
-    if (nsplit > ws.nsplit) nsplit = ws.nsplit;
-    return launch_grad_weight(src, ws.upm, ws.ym, dw, ws.partial, nsplit, B, J, np, st);
+    int nsplit = weight_grad_splits(B, grad_weight_blocks(w_rows, J));
+    if (nsplit > ws.max_split) nsplit = ws.max_split;
+    rc = launch_grad_weight_rows(src, ws.upm, ws.ym, nsplit > 1 ? ws.partial : dw, nsplit, B, J, 0, np, st);
+    if (rc) return rc;
+    return launch_reduce_partials(ws.partial, dw, w_rows * J, nsplit, st);
 }
 
 int snntc_cv_output_dims(int64_t H, int64_t W, const float* params_host, int64_t* Nh, int64_t* Nw) {
@@ -376,7 +388,7 @@ int snntc_cv_backward_workspace_bytes(int64_t B, int64_t H, int64_t W, int64_t C
     int rc = cv_geom(B, H, W, C, Kc, 0, params_host, false, "snntc_cv_backward_workspace_bytes", &g);
     if (rc) return rc;
     if (!bytes) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_cv_backward_workspace_bytes: bytes is NULL");
-    *bytes = bwd_ws(nullptr, g.S, g.P + 1, Kc).bytes;
+    *bytes = bwd_ws(nullptr, g.S, g.P + 1, Kc, cv_weight_base_blocks(g)).bytes;
     return SNNTC_OK;
 }
 
@@ -413,19 +425,32 @@ int snntc_cv_backward(const float* grad, const float* xpad, const float* w, cons
         return launch_fill_zero(dw, w_rows * Kc, st);
     }
     if (!grad || !xpad || !w || !oldout) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_cv_backward: NULL tensor pointer");
-    BwdWs ws = bwd_ws(workspace, g.S, g.P + 1, Kc);
+    BwdWs ws = bwd_ws(workspace, g.S, g.P + 1, Kc, cv_weight_base_blocks(g));
     rc = check_workspace(workspace, workspace_bytes, ws.bytes);
     if (rc) return rc;
     const NeuronParams np = neuron_params(params_host[0], params_host[4], params_host[11]);
     rc = launch_prep_upstream(grad, oldout, oldout + g.S * Kc, ws.upm, ws.ym, g.S * Kc, np, st);
     if (rc) return rc;
-    rc = launch_transpose(w, ws.wt, g.P, Kc, st);       // wt[Kc, P]
+    if (cv_grad_input_chan_supported(g)) {
+        rc = launch_cv_grad_input_chan(xpad, w, ws.upm, ws.ym, dxpad, g, np, st);
+    } else {
+        rc = launch_transpose(w, ws.wt, g.P, Kc, st);   // wt[Kc, P]
+        if (rc) return rc;
+        rc = launch_cv_grad_input(xpad, ws.wt, ws.upm, ws.ym, dxpad, g, g.P, st);
+    }
     if (rc) return rc;
-    rc = launch_cv_grad_input(xpad, ws.wt, ws.upm, ws.ym, dxpad, g, g.P, st);
+    const bool wide = cv_grad_weight_wide_supported(g);
+    int nsplit = weight_grad_splits(g.S, wide ? cv_grad_weight_wide_blocks(g) : grad_weight_blocks(w_rows, Kc));
+    if (nsplit > ws.max_split) nsplit = ws.max_split;
+    float* dst = nsplit > 1 ? ws.partial : dw;
+    const SegmentSource src = conv_source(xpad, g);
+    if (wide) {
+        rc = launch_cv_grad_weight_wide(xpad, ws.upm, ws.ym, dst, nsplit, g, w_rows, np, st);
+    } else {
+        rc = launch_grad_weight_rows(src, ws.upm, ws.ym, dst, nsplit, g.S, Kc, 0, np, st);
+    }
     if (rc) return rc;
-    int nsplit = weight_grad_splits(g.S, w_rows, Kc);
-    if (nsplit > ws.nsplit) nsplit = ws.nsplit;
-    return launch_grad_weight(conv_source(xpad, g), ws.upm, ws.ym, dw, ws.partial, nsplit, g.S, Kc, np, st);
+    return launch_reduce_partials(ws.partial, dw, w_rows * Kc, nsplit, st);
 }
 
 }  // extern "C"

@@ -1,0 +1,225 @@
+// Backward kernels specialised for conv layers whose channel count is a multiple of 32.
+//
+// Same contract as grad.hip (snntc/snncvgrad_kernels.cu.cc:15-161): with up = grad*1/S masked by
+// y <= MAX-0.1 (arrays upm / ym), patch s = (a, nh, nw), element i = (kh*Kw + kw)*C + c,
+//   dXpad[a,h,w,c] = sum over patches covering (h,w) and over kc of [x <= ym[s,kc]] upm[s,kc] W[i,kc]
+//   dW[i,kc]       = sum over patches of min(x_si - ym[s,kc], 0) * upm[s,kc]
+// Both kernels put the channel (dX) or the output channel (dW) on the lanes, so everything that
+// depends only on the patch is wave-uniform and is fetched through the scalar path.
+#include "snntc_common.h"
+
+namespace snntc {
+namespace {
+
+// ---------------------------------------------------------------------------------------------
+// dX.  A wavefront owns TILE consecutive pixels of one image row and 64 (or 32) channels; lane =
+// channel.  For every kernel tap (kh, kw) the lane keeps its weight row W[(kh,kw,c), 0..KCB) in
+// registers and sweeps the tile: the patch under the tap is the same for all lanes, so its ym /
+// upm rows are scalar operands.  Gather form: no atomics, fixed summation order.
+// ---------------------------------------------------------------------------------------------
+constexpr int DX_TILE = 4;
+
+template <int KCB>
+__global__ void __launch_bounds__(256)
+cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restrict__ w,
+                          const float* __restrict__ upm, const float* __restrict__ ym,
+                          float* __restrict__ dxpad, int H, int W, int C, int Kc, int Kh, int Kw, int Sh, int Sw,
+                          int Nh, int Nw, int tiles_w, int c_blocks, int64_t n_items, float max_cmp) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int64_t item = (int64_t)blockIdx.x * (blockDim.x / kWave) + wave;
+    if (item >= n_items) return;
+    const int lane = threadIdx.x % kWave;
+    const int cb = (int)(item % c_blocks);
+    int64_t rest = item / c_blocks;
+    const int tw = (int)(rest % tiles_w); rest /= tiles_w;
+    const int h = (int)(rest % H);
+    const int a = (int)(rest / H);
+    const int w0 = tw * DX_TILE;
+    const int c = cb * kWave + lane;
+    const bool lane_ok = c < C;
+    const unsigned cc = (unsigned)(lane_ok ? c : C - 1);
+
+    float xv[DX_TILE], acc[DX_TILE];
+    bool any_real = false;
+    const float* __restrict__ xrow = xpad + ((size_t)(a * H + h) * W) * C + cc;
+#pragma unroll
+    for (int t = 0; t < DX_TILE; ++t) {
+        const int wx = min(w0 + t, W - 1);
+        xv[t] = xrow[(size_t)wx * C];
+        acc[t] = 0.0f;
+        any_real |= xv[t] <= max_cmp;
+    }
+    // padded pixels (x > MAX-0.1) can never satisfy x <= ym: skip tiles that hold nothing else
+    if (__any(any_real)) {
+        for (int kh = 0; kh < Kh; ++kh) {
+            const int hh = h - kh;
+            if (hh < 0 || hh % Sh != 0) continue;
+            const int nh = hh / Sh;
+            if (nh >= Nh) continue;
+            for (int kw = 0; kw < Kw; ++kw) {
+                const float* __restrict__ wrow = w + ((size_t)(kh * Kw + kw) * C + cc) * Kc;
+                for (int kc0 = 0; kc0 < Kc; kc0 += KCB) {
+                    float wreg[KCB];
+#pragma unroll
+                    for (int q = 0; q < KCB; q += 4) {
+                        const float4 v4 = *reinterpret_cast<const float4*>(wrow + kc0 + q);
+                        wreg[q] = v4.x; wreg[q + 1] = v4.y; wreg[q + 2] = v4.z; wreg[q + 3] = v4.w;
+                    }
+#pragma unroll
+                    for (int t = 0; t < DX_TILE; ++t) {
+                        const int ww = w0 + t - kw;
+                        if (w0 + t >= W || ww < 0 || ww % Sw != 0) continue;
+                        const int nw = ww / Sw;
+                        if (nw >= Nw) continue;
+                        const size_t so = ((size_t)(a * Nh + nh) * Nw + nw) * Kc + kc0;
+                        const float* __restrict__ yrow = ym + so;
+                        const float* __restrict__ urow = upm + so;
+                        // 16 output channels at a time: 32 scalar operands live, not 2*KCB
+#pragma unroll
+                        for (int q0 = 0; q0 < KCB; q0 += 16) {
+#pragma unroll
+                            for (int q = q0; q < q0 + 16; ++q) {
+                                const float tq = xv[t] <= yrow[q] ? wreg[q] : 0.0f;
+                                acc[t] = __fmaf_rn(urow[q], tq, acc[t]);
+                            }
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
+                }
+            }
+        }
+    }
+    if (lane_ok) {
+        float* __restrict__ orow = dxpad + ((size_t)(a * H + h) * W) * C + c;
+#pragma unroll
+        for (int t = 0; t < DX_TILE; ++t)
+            if (w0 + t < W) orow[(size_t)(w0 + t) * C] = acc[t];
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// dW.  Lane = output channel kc; a block owns DWW_RI consecutive weight rows that share one tap
+// (kh, kw), i.e. DWW_RI consecutive input channels, so the x values of a patch are one contiguous
+// scalar fetch.  The patch range is cut into gridDim.z slices (partial sums are added in slice
+// order afterwards) and each slice over the four wavefronts of the block.
+// ---------------------------------------------------------------------------------------------
+constexpr int DWW_RI = 32;
+
+__global__ void __launch_bounds__(256)
+cv_grad_weight_wide_kernel(const float* __restrict__ xpad, const float* __restrict__ upm,
+                           const float* __restrict__ ym, float* __restrict__ dst, int S, int Kc, int rows,
+                           int seg_per_slice, int H, int W, int C, int Kw, int Sh, int Sw, int Nh, int Nw,
+                           int bias_row, float biasvolt) {
+    __shared__ float red[3][DWW_RI + 1][kWave];
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int j = blockIdx.x * kWave + lane;
+    const unsigned jc = (unsigned)min(j, Kc - 1);
+    const int i0 = blockIdx.y * DWW_RI;                 // first weight row of the block
+    const int tap = i0 / C, c0 = i0 - tap * C;          // tap = kh*Kw + kw
+    const int kh = tap / Kw, kw = tap - kh * Kw;
+
+    const int s_begin = blockIdx.z * seg_per_slice;
+    const int s_end = min(S, s_begin + seg_per_slice);
+    const int per_wave = (s_end - s_begin + 3) / 4;
+    const int s_lo = s_begin + wave * per_wave;
+    const int s_hi = min(s_end, s_lo + per_wave);
+
+    float acc[DWW_RI];
+#pragma unroll
+    for (int r = 0; r < DWW_RI; ++r) acc[r] = 0.0f;
+    // the block of rows 0..31 also carries the bias row (x = biasvolt for every patch)
+    const bool with_bias = bias_row >= 0 && blockIdx.y == 0;
+    float acc_bias = 0.0f;
+
+    if (s_lo < s_hi) {
+        const int per_img = Nh * Nw;
+        int a = s_lo / per_img;
+        int r2 = s_lo - a * per_img;
+        int nh = r2 / Nw, nw = r2 - nh * Nw;
+        const float* __restrict__ ycol = ym + jc;
+        const float* __restrict__ ucol = upm + jc;
+        for (int s = s_lo; s < s_hi; ++s) {
+            const float* __restrict__ xb =
+                xpad + ((size_t)(a * H + nh * Sh + kh) * W + (size_t)(nw * Sw + kw)) * C + c0;
+            const float yv = ycol[(size_t)s * Kc];
+            const float uv = ucol[(size_t)s * Kc];
+#pragma unroll
+            for (int r = 0; r < DWW_RI; ++r) acc[r] = __fmaf_rn(fminf(xb[r] - yv, 0.0f), uv, acc[r]);
+            if (with_bias) acc_bias = __fmaf_rn(fminf(biasvolt - yv, 0.0f), uv, acc_bias);
+            if (++nw == Nw) { nw = 0; if (++nh == Nh) { nh = 0; ++a; } }
+        }
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int r = 0; r < DWW_RI; ++r) red[wave - 1][r][lane] = acc[r];
+        red[wave - 1][DWW_RI][lane] = acc_bias;
+    }
+    __syncthreads();
+    if (wave == 0 && j < Kc) {
+        float* out = dst + (size_t)blockIdx.z * rows * Kc;
+#pragma unroll
+        for (int r = 0; r < DWW_RI; ++r)
+            out[(size_t)(i0 + r) * Kc + j] = ((acc[r] + red[0][r][lane]) + red[1][r][lane]) + red[2][r][lane];
+        if (with_bias)
+            out[(size_t)bias_row * Kc + j] =
+                ((acc_bias + red[0][DWW_RI][lane]) + red[1][DWW_RI][lane]) + red[2][DWW_RI][lane];
+    }
+}
+
+}  // namespace
+
+bool cv_grad_input_chan_supported(const ConvGeom& g) {
+    return g.C >= 32 && g.Kc % 16 == 0;
+}
+
+int launch_cv_grad_input_chan(const float* xpad, const float* w, const float* upm, const float* ym,
+                              float* dxpad, const ConvGeom& g, const NeuronParams& np, hipStream_t stream) {
+    const int tiles_w = (int)((g.W + DX_TILE - 1) / DX_TILE);
+    const int c_blocks = (int)((g.C + kWave - 1) / kWave);
+    const int64_t n_items = g.B * g.H * tiles_w * c_blocks;
+    const int64_t blocks = (n_items + 3) / 4;
+    if (blocks > 0x7fffffffLL) return fail(SNNTC_ERR_TOO_LARGE, "conv backward: grid too large");
+    dim3 grid((unsigned)blocks), block(256);
+    {
+        KernelTimerScope timer_("cv_grad_input", stream);
+        if (g.Kc % 64 == 0)
+            hipLaunchKernelGGL(cv_grad_input_chan_kernel<64>, grid, block, 0, stream, xpad, w, upm, ym, dxpad,
+                               (int)g.H, (int)g.W, (int)g.C, (int)g.Kc, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw,
+                               (int)g.Nh, (int)g.Nw, tiles_w, c_blocks, n_items, np.max_cmp);
+        else if (g.Kc % 32 == 0)
+            hipLaunchKernelGGL(cv_grad_input_chan_kernel<32>, grid, block, 0, stream, xpad, w, upm, ym, dxpad,
+                               (int)g.H, (int)g.W, (int)g.C, (int)g.Kc, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw,
+                               (int)g.Nh, (int)g.Nw, tiles_w, c_blocks, n_items, np.max_cmp);
+        else
+            hipLaunchKernelGGL(cv_grad_input_chan_kernel<16>, grid, block, 0, stream, xpad, w, upm, ym, dxpad,
+                               (int)g.H, (int)g.W, (int)g.C, (int)g.Kc, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw,
+                               (int)g.Nh, (int)g.Nw, tiles_w, c_blocks, n_items, np.max_cmp);
+    }
+    SNNTC_HIP_CHECK(hipGetLastError());
+    return SNNTC_OK;
+}
+
+bool cv_grad_weight_wide_supported(const ConvGeom& g) { return g.C % DWW_RI == 0; }
+
+int cv_grad_weight_wide_blocks(const ConvGeom& g) {
+    return (int)(((g.Kc + kWave - 1) / kWave) * (g.P / DWW_RI));
+}
+
+// All rows of dW, bias row included (or of every partial-sum slice when nsplit > 1).
+int launch_cv_grad_weight_wide(const float* xpad, const float* upm, const float* ym, float* dst, int nsplit,
+                               const ConvGeom& g, int64_t rows, const NeuronParams& np, hipStream_t stream) {
+    const int seg_per_slice = (int)((g.S + nsplit - 1) / nsplit);
+    dim3 grid((unsigned)((g.Kc + kWave - 1) / kWave), (unsigned)(g.P / DWW_RI), (unsigned)nsplit);
+    if (grid.y > 65535u) return fail(SNNTC_ERR_TOO_LARGE, "weight gradient: too many weight rows");
+    {
+        KernelTimerScope timer_("grad_weight", stream);
+        hipLaunchKernelGGL(cv_grad_weight_wide_kernel, grid, dim3(256), 0, stream, xpad, upm, ym, dst, (int)g.S,
+                           (int)g.Kc, (int)rows, seg_per_slice, (int)g.H, (int)g.W, (int)g.C, (int)g.Kw, (int)g.Sh,
+                           (int)g.Sw, (int)g.Nh, (int)g.Nw, np.bias ? (int)g.P : -1, np.biasvolt);
+    }
+    SNNTC_HIP_CHECK(hipGetLastError());
+    return SNNTC_OK;
+}
+
+}  // namespace snntc

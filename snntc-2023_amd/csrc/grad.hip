@@ -152,13 +152,14 @@ __device__ __forceinline__ const float* segment_base(const SegmentSource& src, i
 
 __global__ void __launch_bounds__(256)
 grad_weight_kernel(SegmentSource src, const float* __restrict__ upm, const float* __restrict__ ym,
-                   float* __restrict__ dst, int S, int J, int rows, int seg_per_slice, float biasvolt) {
+                   float* __restrict__ dst, int S, int J, int rows, int row_start, int seg_per_slice,
+                   float biasvolt) {
     __shared__ float red[3][DW_RI][kWave];
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int j = blockIdx.x * kWave + lane;
     const unsigned jc = (unsigned)min(j, J - 1);
-    const int i0 = blockIdx.y * DW_RI;
+    const int i0 = row_start + blockIdx.y * DW_RI;
     const int I = src.I;
 
     const int s_begin = blockIdx.z * seg_per_slice;
@@ -239,9 +240,17 @@ __global__ void __launch_bounds__(256)
 reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ out, int64_t n, int nsplit) {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= n) return;
-    float acc = 0.0f;
-    for (int z = 0; z < nsplit; ++z) acc += partial[(size_t)z * n + t];
-    out[t] = acc;
+    // slices are added in ascending order, four independent chains to keep the loads in flight
+    float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+    int z = 0;
+    for (; z + 4 <= nsplit; z += 4) {
+        a0 += partial[(size_t)z * n + t];
+        a1 += partial[(size_t)(z + 1) * n + t];
+        a2 += partial[(size_t)(z + 2) * n + t];
+        a3 += partial[(size_t)(z + 3) * n + t];
+    }
+    for (; z < nsplit; ++z) a0 += partial[(size_t)z * n + t];
+    out[t] = (a0 + a1) + (a2 + a3);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -335,12 +344,12 @@ int launch_fc_grad_input(const float* x, const float* wt, const float* upm, cons
     return SNNTC_OK;
 }
 
-// Number of slices the segment range is cut into for dW: enough blocks to fill the chip,
-// at least 64 segments per slice, at most 256 slices.
-int weight_grad_splits(int64_t S, int64_t rows, int64_t J) {
-    const int64_t base_blocks = ((J + kWave - 1) / kWave) * ((rows + DW_RI - 1) / DW_RI);
+// Number of slices the segment range is cut into for dW: none when the (row-block x column-block)
+// grid alone fills the chip; otherwise enough for ~2048 blocks, at least 64 segments per slice, at
+// most 256 slices.
+int weight_grad_splits(int64_t S, int64_t base_blocks) {
     if (base_blocks >= 1024) return 1;
-    int64_t want = (2048 + base_blocks - 1) / (base_blocks > 0 ? base_blocks : 1);
+    int64_t want = (1536 + base_blocks - 1) / (base_blocks > 0 ? base_blocks : 1);
     int64_t cap = S / 64;
     if (want > cap) want = cap;
     if (want > 256) want = 256;
@@ -348,30 +357,38 @@ int weight_grad_splits(int64_t S, int64_t rows, int64_t J) {
     return (int)want;
 }
 
-int launch_grad_weight(const SegmentSource& src, const float* upm, const float* ym, float* dw,
-                       float* partial, int nsplit, int64_t S, int64_t J, const NeuronParams& np,
-                       hipStream_t stream) {
+int grad_weight_blocks(int64_t rows, int64_t J) {
+    return (int)(((J + kWave - 1) / kWave) * ((rows + DW_RI - 1) / DW_RI));
+}
+
+// Rows [row_start, rows) of dW, or of every partial-sum slice when nsplit > 1 (dst = slices).
+int launch_grad_weight_rows(const SegmentSource& src, const float* upm, const float* ym, float* dst,
+                            int nsplit, int64_t S, int64_t J, int64_t row_start, const NeuronParams& np,
+                            hipStream_t stream) {
     const int64_t rows = (int64_t)src.I + np.bias;
-    if (rows <= 0 || J <= 0) return SNNTC_OK;
-    if (S <= 0) return launch_fill_zero(dw, rows * J, stream);
+    if (rows <= row_start || J <= 0 || S <= 0) return SNNTC_OK;
     if (nsplit < 1) nsplit = 1;
     const int seg_per_slice = (int)((S + nsplit - 1) / nsplit);
-    dim3 grid((unsigned)((J + kWave - 1) / kWave), (unsigned)((rows + DW_RI - 1) / DW_RI), (unsigned)nsplit);
+    dim3 grid((unsigned)((J + kWave - 1) / kWave), (unsigned)((rows - row_start + DW_RI - 1) / DW_RI),
+              (unsigned)nsplit);
     if (grid.y > 65535u) return fail(SNNTC_ERR_TOO_LARGE, "weight gradient: too many weight rows");
-    float* dst = nsplit > 1 ? partial : dw;
-    { KernelTimerScope timer_("grad_weight", stream);
-    hipLaunchKernelGGL(grad_weight_kernel, grid, dim3(256), 0, stream, src, upm, ym, dst, (int)S, (int)J,
-                       (int)rows, seg_per_slice, np.biasvolt);
+    {
+        KernelTimerScope timer_(row_start ? "grad_weight_tail" : "grad_weight", stream);
+        hipLaunchKernelGGL(grad_weight_kernel, grid, dim3(256), 0, stream, src, upm, ym, dst, (int)S, (int)J,
+                           (int)rows, (int)row_start, seg_per_slice, np.biasvolt);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
-    if (nsplit > 1) {
-        const int64_t n = rows * J;
-        { KernelTimerScope timer_("reduce_partials", stream);
+    return SNNTC_OK;
+}
+
+int launch_reduce_partials(const float* partial, float* dw, int64_t n, int nsplit, hipStream_t stream) {
+    if (n <= 0 || nsplit <= 1) return SNNTC_OK;
+    {
+        KernelTimerScope timer_("reduce_partials", stream);
         hipLaunchKernelGGL(reduce_partials_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream, partial, dw,
                            n, nsplit);
-        }
-        SNNTC_HIP_CHECK(hipGetLastError());
     }
+    SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
 }
 

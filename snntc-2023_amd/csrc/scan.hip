@@ -174,44 +174,50 @@ __device__ __forceinline__ void load_chunk(Chunk& c, const float* __restrict__ x
 
 #define SNNTC_SCAN_COUNT "v_add_u32_e32 %[kcnt], 1, %[kcnt]\n"
 
-template <bool WANT_K>
+#define SNNTC_SCAN_PROLOGUE                         \
+    "s_mov_b64 %[save], exec\n"                     \
+    "s_andn2_b64 %[keep], %[fired], %[run]\n"       \
+    "s_mov_b64 exec, %[run]\n"
+#define SNNTC_SCAN_EPILOGUE                         \
+    "s_or_b64 %[fired], %[fired], %[keep]\n"        \
+    "s_mov_b64 exec, %[save]\n"
+#define SNNTC_SCAN_STATE                                                                               \
+    [wsum] "+v"(wsum), [ysum] "+v"(ysum), [ya] "+v"(ya), [kcnt] "+v"(kcnt), [fired] "+s"(fired),       \
+        [closed] "+s"(closed), [save] "=&s"(saved_exec), [keep] "=&s"(keep), [t] "=&v"(t)
+#define SNNTC_SCAN_INPUTS(XC, X)                                                                       \
+    [run] "s"(run), [x0] XC(X[0]), [x1] XC(X[1]), [x2] XC(X[2]), [x3] XC(X[3]), [x4] XC(X[4]),          \
+        [x5] XC(X[5]), [x6] XC(X[6]), [x7] XC(X[7]), [w0] "v"(w[0]), [w1] "v"(w[1]), [w2] "v"(w[2]),    \
+        [w3] "v"(w[3]), [w4] "v"(w[4]), [w5] "v"(w[5]), [w6] "v"(w[6]), [w7] "v"(w[7])
+#define SNNTC_SCAN_BODY_K                                                                              \
+    SNNTC_SCAN_PROLOGUE SNNTC_SCAN_STEP(0) SNNTC_SCAN_COUNT SNNTC_SCAN_STEP(1) SNNTC_SCAN_COUNT         \
+        SNNTC_SCAN_STEP(2) SNNTC_SCAN_COUNT SNNTC_SCAN_STEP(3) SNNTC_SCAN_COUNT SNNTC_SCAN_STEP(4)      \
+            SNNTC_SCAN_COUNT SNNTC_SCAN_STEP(5) SNNTC_SCAN_COUNT SNNTC_SCAN_STEP(6) SNNTC_SCAN_COUNT    \
+                SNNTC_SCAN_STEP(7) SNNTC_SCAN_COUNT SNNTC_SCAN_EPILOGUE
+#define SNNTC_SCAN_BODY                                                                                \
+    SNNTC_SCAN_PROLOGUE SNNTC_SCAN_STEP(0) SNNTC_SCAN_STEP(1) SNNTC_SCAN_STEP(2) SNNTC_SCAN_STEP(3)     \
+        SNNTC_SCAN_STEP(4) SNNTC_SCAN_STEP(5) SNNTC_SCAN_STEP(6) SNNTC_SCAN_STEP(7) SNNTC_SCAN_EPILOGUE
+
+// UNIFORM_X: the eight input times are the same for every lane (one segment per wavefront) and are
+// handed over in scalar registers.
+template <bool WANT_K, bool UNIFORM_X>
 __device__ __forceinline__ void scan_chunk(float& wsum, float& ysum, float& ya, int& kcnt, uint64_t& fired,
                                            uint64_t& closed, uint64_t run, const float (&x)[CHUNK],
                                            const float (&w)[CHUNK]) {
     uint64_t saved_exec, keep;
     float t;
-    if (WANT_K) {
-        asm volatile(
-            "s_mov_b64 %[save], exec\n"
-            "s_andn2_b64 %[keep], %[fired], %[run]\n"
-            "s_mov_b64 exec, %[run]\n"
-            SNNTC_SCAN_STEP(0) SNNTC_SCAN_COUNT SNNTC_SCAN_STEP(1) SNNTC_SCAN_COUNT
-            SNNTC_SCAN_STEP(2) SNNTC_SCAN_COUNT SNNTC_SCAN_STEP(3) SNNTC_SCAN_COUNT
-            SNNTC_SCAN_STEP(4) SNNTC_SCAN_COUNT SNNTC_SCAN_STEP(5) SNNTC_SCAN_COUNT
-            SNNTC_SCAN_STEP(6) SNNTC_SCAN_COUNT SNNTC_SCAN_STEP(7) SNNTC_SCAN_COUNT
-            "s_or_b64 %[fired], %[fired], %[keep]\n"
-            "s_mov_b64 exec, %[save]\n"
-            : [wsum] "+v"(wsum), [ysum] "+v"(ysum), [ya] "+v"(ya), [kcnt] "+v"(kcnt), [fired] "+s"(fired),
-              [closed] "+s"(closed), [save] "=&s"(saved_exec), [keep] "=&s"(keep), [t] "=&v"(t)
-            : [run] "s"(run), [x0] "v"(x[0]), [x1] "v"(x[1]), [x2] "v"(x[2]), [x3] "v"(x[3]), [x4] "v"(x[4]),
-              [x5] "v"(x[5]), [x6] "v"(x[6]), [x7] "v"(x[7]), [w0] "v"(w[0]), [w1] "v"(w[1]), [w2] "v"(w[2]),
-              [w3] "v"(w[3]), [w4] "v"(w[4]), [w5] "v"(w[5]), [w6] "v"(w[6]), [w7] "v"(w[7])
-            : "vcc");
+    if (UNIFORM_X) {
+        int xs[CHUNK];
+#pragma unroll
+        for (int u = 0; u < CHUNK; ++u) xs[u] = __builtin_amdgcn_readfirstlane(__float_as_int(x[u]));
+        if (WANT_K)
+            asm volatile(SNNTC_SCAN_BODY_K : SNNTC_SCAN_STATE : SNNTC_SCAN_INPUTS("s", xs) : "vcc");
+        else
+            asm volatile(SNNTC_SCAN_BODY : SNNTC_SCAN_STATE : SNNTC_SCAN_INPUTS("s", xs) : "vcc");
     } else {
-        asm volatile(
-            "s_mov_b64 %[save], exec\n"
-            "s_andn2_b64 %[keep], %[fired], %[run]\n"
-            "s_mov_b64 exec, %[run]\n"
-            SNNTC_SCAN_STEP(0) SNNTC_SCAN_STEP(1) SNNTC_SCAN_STEP(2) SNNTC_SCAN_STEP(3)
-            SNNTC_SCAN_STEP(4) SNNTC_SCAN_STEP(5) SNNTC_SCAN_STEP(6) SNNTC_SCAN_STEP(7)
-            "s_or_b64 %[fired], %[fired], %[keep]\n"
-            "s_mov_b64 exec, %[save]\n"
-            : [wsum] "+v"(wsum), [ysum] "+v"(ysum), [ya] "+v"(ya), [fired] "+s"(fired), [closed] "+s"(closed),
-              [save] "=&s"(saved_exec), [keep] "=&s"(keep), [t] "=&v"(t)
-            : [run] "s"(run), [x0] "v"(x[0]), [x1] "v"(x[1]), [x2] "v"(x[2]), [x3] "v"(x[3]), [x4] "v"(x[4]),
-              [x5] "v"(x[5]), [x6] "v"(x[6]), [x7] "v"(x[7]), [w0] "v"(w[0]), [w1] "v"(w[1]), [w2] "v"(w[2]),
-              [w3] "v"(w[3]), [w4] "v"(w[4]), [w5] "v"(w[5]), [w6] "v"(w[6]), [w7] "v"(w[7])
-            : "vcc");
+        if (WANT_K)
+            asm volatile(SNNTC_SCAN_BODY_K : SNNTC_SCAN_STATE : SNNTC_SCAN_INPUTS("v", x) : "vcc");
+        else
+            asm volatile(SNNTC_SCAN_BODY : SNNTC_SCAN_STATE : SNNTC_SCAN_INPUTS("v", x) : "vcc");
     }
 }
 
@@ -284,7 +290,7 @@ scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ pe
                 load_chunk(xp[(ph + 2) % 3], xs, pr, kn <= last_chunk ? kn : 0);
 #pragma unroll
                 for (int u = 0; u < CHUNK; ++u) wv[(ph + 1) % 2][u] = wcol[xp[(ph + 1) % 3].p[u] * COLS];
-                scan_chunk<WANT_K>(wsum, ysum, ya, kcnt, fired, closed, run, xp[ph % 3].x, wv[ph % 2]);
+                scan_chunk<WANT_K, COLS == kWave>(wsum, ysum, ya, kcnt, fired, closed, run, xp[ph % 3].x, wv[ph % 2]);
             }
             if (stop) break;
         }

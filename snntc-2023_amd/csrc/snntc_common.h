@@ -88,11 +88,23 @@ int launch_transpose(const float* w, float* wt, int64_t rows, int64_t cols, hipS
 int launch_fc_grad_input(const float* x, const float* wt, const float* upm, const float* ym, float* dx,
                          int64_t B, int64_t I, int64_t J, int64_t wt_stride, hipStream_t stream);
 
-// dW for dense rows or implicit patches; `partial` is scratch for the split reduction.
-int weight_grad_splits(int64_t S, int64_t rows, int64_t J);
-int launch_grad_weight(const SegmentSource& src, const float* upm, const float* ym, float* dw,
-                       float* partial, int nsplit, int64_t S, int64_t J, const NeuronParams& np,
-                       hipStream_t stream);
+// dW for dense rows or implicit patches.  The segment range may be cut into `nsplit` slices whose
+// partial sums (scratch `dst`, nsplit x rows x J) are added in slice order by launch_reduce_partials.
+int weight_grad_splits(int64_t S, int64_t base_blocks);
+int grad_weight_blocks(int64_t rows, int64_t J);
+int launch_grad_weight_rows(const SegmentSource& src, const float* upm, const float* ym, float* dst,
+                            int nsplit, int64_t S, int64_t J, int64_t row_start, const NeuronParams& np,
+                            hipStream_t stream);
+int launch_reduce_partials(const float* partial, float* dw, int64_t n, int nsplit, hipStream_t stream);
+
+// Conv layers with many channels: lane = channel (dX) / wide row blocks (dW), see cv_grad.hip.
+bool cv_grad_input_chan_supported(const ConvGeom& g);
+int launch_cv_grad_input_chan(const float* xpad, const float* w, const float* upm, const float* ym,
+                              float* dxpad, const ConvGeom& g, const NeuronParams& np, hipStream_t stream);
+bool cv_grad_weight_wide_supported(const ConvGeom& g);
+int cv_grad_weight_wide_blocks(const ConvGeom& g);
+int launch_cv_grad_weight_wide(const float* xpad, const float* upm, const float* ym, float* dst, int nsplit,
+                               const ConvGeom& g, int64_t rows, const NeuronParams& np, hipStream_t stream);
 
 int launch_cv_grad_input(const float* xpad, const float* wt, const float* upm, const float* ym,
                          float* dxpad, const ConvGeom& g, int64_t wt_stride, hipStream_t stream);
