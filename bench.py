@@ -199,6 +199,61 @@ WORKLOADS = {"mlp": MlpTrainStep, "dense": DenseLayerStep, "conv": ConvLayerStep
 
 
 # ------------------------------------------------------------------------------------------------
+# HIP graph of one step
+# ------------------------------------------------------------------------------------------------
+def capture_step(torch, wl):
+    """Captures wl.step() into a HIP graph (all launches of a step replayed with one call) and checks
+    that replays reproduce eager steps bit for bit from the same starting weights.  Returns the graph,
+    or None (with the reason) when capture or the check fails; the caller then times eager steps."""
+    params = getattr(wl, "params", [])
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                wl.step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        start = [p.detach().clone() for p in params]
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = wl.step()
+        torch.cuda.synchronize()
+
+        def restore():
+            with torch.no_grad():
+                for p, s0 in zip(params, start):
+                    p.copy_(s0)
+
+        def snapshot(res):
+            vals = [p.detach().clone() for p in params]
+            if isinstance(res, torch.Tensor):
+                vals.append(res.detach().clone())
+            elif isinstance(res, (tuple, list)):
+                vals += [r.detach().clone() for r in res if isinstance(r, torch.Tensor)]
+            return vals
+
+        restore()
+        eager = []
+        for _ in range(3):
+            eager.append(snapshot(wl.step()))
+        restore()
+        for i in range(3):
+            graph.replay()
+            torch.cuda.synchronize()
+            got = snapshot(out)
+            if len(got) != len(eager[i]) or not all(torch.equal(a, b) for a, b in zip(got, eager[i])):
+                restore()
+                return None, f"replay {i} differs from the eager step"
+            _ = sum(float(v.sum()) for v in got[:1])      # eager work and a sync between replays
+        restore()
+        return graph, None
+    except Exception as e:  # capture not possible on this stack: fall back to eager timing
+        torch.cuda.synchronize()
+        return None, f"{type(e).__name__}: {e}"
+
+
+# ------------------------------------------------------------------------------------------------
 # roofline accounting: algorithmic flops / bytes per kernel, summed over the layers of one step
 # ------------------------------------------------------------------------------------------------
 def account(torch, snn, layers):
@@ -325,6 +380,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="mlp")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="time eager steps instead of HIP-graph replays")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -339,15 +395,28 @@ def main():
     torch.cuda.set_device(dev)
     wl = WORKLOADS[args.workload](torch, snn, dev)
 
+    graph, graph_note = (None, "disabled by --no-graph") if args.no_graph else capture_step(torch, wl)
+    run_step = graph.replay if graph is not None else wl.step
+
     for _ in range(args.warmup):
+        run_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run_step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+
+    # the same steps launched eagerly, for reference
+    for _ in range(3):
         wl.step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
         wl.step()
     torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    ms_per_step = dt / args.steps * 1e3
+    eager_ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
 
     # second pass over the same steps with the library's per-kernel HIP-event timing switched on
     _lib.profile_enable(True)
@@ -386,7 +455,9 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": wl.name, "batch": wl.batch, "device": torch.cuda.get_device_name(0)},
+        "config": {"workload": wl.name, "batch": wl.batch, "device": torch.cuda.get_device_name(0),
+                   "launch": "hip graph replay" if graph is not None else "eager", "graph_note": graph_note},
+        "eager_ms_per_step": eager_ms_per_step,
         "roofline": roof,
         "kernels": kernels,
         "library_kernel_us_per_step": sum(v["us_per_step"] for v in kernels.values()),

@@ -104,7 +104,8 @@ SNNTC_API int snntc_fc_forward_ex(const float* x, const float* w, const float* p
                         void* workspace, size_t workspace_bytes, void* stream);
 
 /* grad[grad_rows,J] (only rows [0,B) are read), oldout[2B,J] = the forward output.
- * dx[B,I], dw[w_rows,J], dparams[6] (device, may be NULL; written with zeros).
+ * dx[B,I], dw[w_rows,J], dparams[6] (device; written with zeros).  Any of the three outputs may be
+ * NULL: that gradient is then not computed (the reference always computes all of them).
  * Errors: grad_rows != 2B -> DIM_MISMATCH (snntc/snnfcgrad_kernels.cc:119-120); sizes as above. */
 SNNTC_API int snntc_fc_backward(const float* grad, const float* x, const float* w, const float* params_host,
                       const float* oldout, float* dx, float* dw, float* dparams,
@@ -140,7 +141,8 @@ SNNTC_API int snntc_cv_forward_ex(const float* xpad, const float* w, const float
                         void* workspace, size_t workspace_bytes, void* stream);
 
 /* grad[grad_rows,Nh,Nw,Kc] (rows [0,B) read), oldout[2B,Nh,Nw,Kc].
- * dxpad[B,H,W,C] (gradient w.r.t. the padded input), dw[w_rows,Kc], dparams[12] (may be NULL).
+ * dxpad[B,H,W,C] (gradient w.r.t. the padded input), dw[w_rows,Kc], dparams[12]; any may be NULL
+ * (not computed).
  * Errors: grad_rows != 2B -> DIM_MISMATCH; sizes as in the forward op. */
 SNNTC_API int snntc_cv_backward(const float* grad, const float* xpad, const float* w, const float* params_host,
                       const float* oldout, float* dxpad, float* dw, float* dparams,

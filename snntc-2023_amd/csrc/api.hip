@@ -338,10 +338,10 @@ int snntc_fc_backward(const float* grad, const float* x, const float* w, const f
                     (long long)grad_rows, (long long)B);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (dparams) { rc = launch_fill_zero(dparams, 6, st); if (rc) return rc; }
-    if (!dx || !dw) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_fc_backward: NULL output pointer");
+    if (!dx && !dw) return SNNTC_OK;                     // a NULL gradient output is simply not computed
     if (B == 0 || J == 0) {
-        rc = launch_fill_zero(dx, B * I, st); if (rc) return rc;
-        return launch_fill_zero(dw, w_rows * J, st);
+        if (dx) { rc = launch_fill_zero(dx, B * I, st); if (rc) return rc; }
+        return dw ? launch_fill_zero(dw, w_rows * J, st) : SNNTC_OK;
     }
     if (!grad || !x || !w || !oldout) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_fc_backward: NULL tensor pointer");
     BwdWs ws = bwd_ws(workspace, B, I + 1, J, grad_weight_blocks(I, J));
@@ -350,10 +350,13 @@ int snntc_fc_backward(const float* grad, const float* x, const float* w, const f
     const NeuronParams np = neuron_params(params_host[0], params_host[2], params_host[5]);
     rc = launch_prep_upstream(grad, oldout, oldout + B * J, ws.upm, ws.ym, B * J, np, st);
     if (rc) return rc;
-    rc = launch_transpose(w, ws.wt, I, J, st);          // wt[J, I]: bias row not needed for dX
-    if (rc) return rc;
-    rc = launch_fc_grad_input(x, ws.wt, ws.upm, ws.ym, dx, B, I, J, I, st);
-    if (rc) return rc;
+    if (dx) {
+        rc = launch_transpose(w, ws.wt, I, J, st);      // wt[J, I]: bias row not needed for dX
+        if (rc) return rc;
+        rc = launch_fc_grad_input(x, ws.wt, ws.upm, ws.ym, dx, B, I, J, I, st);
+        if (rc) return rc;
+    }
+    if (!dw) return SNNTC_OK;
     SegmentSource src{};
     src.base = x; src.conv = 0; src.I = (int)I;
     int nsplit = weight_grad_splits(B, grad_weight_blocks(w_rows, J));
@@ -419,10 +422,10 @@ int snntc_cv_backward(const float* grad, const float* xpad, const float* w, cons
                     (long long)grad_rows, (long long)B);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (dparams) { rc = launch_fill_zero(dparams, 12, st); if (rc) return rc; }
-    if (!dxpad || !dw) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_cv_backward: NULL output pointer");
+    if (!dxpad && !dw) return SNNTC_OK;                  // a NULL gradient output is simply not computed
     if (g.S == 0 || Kc == 0) {
-        rc = launch_fill_zero(dxpad, B * H * W * C, st); if (rc) return rc;
-        return launch_fill_zero(dw, w_rows * Kc, st);
+        if (dxpad) { rc = launch_fill_zero(dxpad, B * H * W * C, st); if (rc) return rc; }
+        return dw ? launch_fill_zero(dw, w_rows * Kc, st) : SNNTC_OK;
     }
     if (!grad || !xpad || !w || !oldout) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_cv_backward: NULL tensor pointer");
     BwdWs ws = bwd_ws(workspace, g.S, g.P + 1, Kc, cv_weight_base_blocks(g));
@@ -431,14 +434,17 @@ int snntc_cv_backward(const float* grad, const float* xpad, const float* w, cons
     const NeuronParams np = neuron_params(params_host[0], params_host[4], params_host[11]);
     rc = launch_prep_upstream(grad, oldout, oldout + g.S * Kc, ws.upm, ws.ym, g.S * Kc, np, st);
     if (rc) return rc;
-    if (cv_grad_input_chan_supported(g)) {
-        rc = launch_cv_grad_input_chan(xpad, w, ws.upm, ws.ym, dxpad, g, np, st);
-    } else {
-        rc = launch_transpose(w, ws.wt, g.P, Kc, st);   // wt[Kc, P]
+    if (dxpad) {
+        if (cv_grad_input_chan_supported(g)) {
+            rc = launch_cv_grad_input_chan(xpad, w, ws.upm, ws.ym, dxpad, g, np, st);
+        } else {
+            rc = launch_transpose(w, ws.wt, g.P, Kc, st);   // wt[Kc, P]
+            if (rc) return rc;
+            rc = launch_cv_grad_input(xpad, ws.wt, ws.upm, ws.ym, dxpad, g, g.P, st);
+        }
         if (rc) return rc;
-        rc = launch_cv_grad_input(xpad, ws.wt, ws.upm, ws.ym, dxpad, g, g.P, st);
     }
-    if (rc) return rc;
+    if (!dw) return SNNTC_OK;
     const bool wide = cv_grad_weight_wide_supported(g);
     int nsplit = weight_grad_splits(g.S, wide ? cv_grad_weight_wide_blocks(g) : grad_weight_blocks(w_rows, Kc));
     if (nsplit > ws.max_split) nsplit = ws.max_split;

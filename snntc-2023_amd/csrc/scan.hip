@@ -357,8 +357,16 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     if (n_groups < 1) n_groups = 1;
     auto kern_k = scan_lds_kernel<COLS, true>;
     auto kern = scan_lds_kernel<COLS, false>;
-    SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(causal_k ? kern_k : kern),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+    // raise the dynamic-LDS limit of both instantiations once (not per launch: the call is not
+    // allowed while a stream is being captured into a graph)
+    static bool lds_limit_raised = false;
+    if (!lds_limit_raised) {
+        SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern_k),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS_SCAN_BYTES));
+        SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS_SCAN_BYTES));
+        lds_limit_raised = true;
+    }
     dim3 grid((unsigned)(n_slices * n_groups)), block(LDS_SCAN_THREADS);
     {
         KernelTimerScope timer_("scan", stream);

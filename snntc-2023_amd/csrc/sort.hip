@@ -194,6 +194,8 @@ int launch_sort(const SegmentSource& src, int64_t S, float* sorted, int32_t* per
     if (I <= 128)  return launch_sort_t<2, 64>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
     if (I <= 256)  return launch_sort_t<4, 64>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
     if (I <= 512)  return launch_sort_t<8, 64>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
+    // few long segments (a dense batch): four wavefronts per segment instead of one fill the chip
+    if (I <= 1024 && I > 512 && S < 2048) return launch_sort_t<4, 256>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
     if (I <= 1024) return launch_sort_t<16, 64>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
     if (I <= 2048) return launch_sort_t<8, 256>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
     if (I <= 4096) return launch_sort_t<8, 512>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);

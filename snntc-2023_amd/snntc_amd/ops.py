@@ -85,8 +85,10 @@ def snnfc(X, W, Params, return_aux=False):
     return out
 
 
-def snnfc_grad(grad, X, W, Params, Y):
-    """Dense backward.  grad[2B,J], Y[2B,J] = forward output -> (dX[B,I], dW like W, dParams[6])."""
+def snnfc_grad(grad, X, W, Params, Y, want_dparams=True, want_dx=True, want_dw=True):
+    """Dense backward.  grad[2B,J], Y[2B,J] = forward output -> (dX[B,I], dW like W, dParams[6]).
+    dParams is all zeros (Params is a constant).  A want_* flag set to False skips that gradient
+    (None is returned in its place)."""
     lib = _lib.load()
     grad = _dev_f32(grad, "grad", 2)
     X = _dev_f32(X, "X", 2)
@@ -102,9 +104,9 @@ def snnfc_grad(grad, X, W, Params, Y):
         need = ctypes.c_size_t()
         _lib.check(lib.snntc_fc_backward_workspace_bytes(B, I, J, ctypes.byref(need)))
         ws = _workspace(X.device, need.value)
-        dX = torch.empty_like(X)
-        dW = torch.empty_like(W)
-        dP = torch.empty(6, dtype=torch.float32, device=X.device)
+        dX = torch.empty_like(X) if want_dx else None
+        dW = torch.empty_like(W) if want_dw else None
+        dP = torch.empty(6, dtype=torch.float32, device=X.device) if want_dparams else None
         _lib.check(lib.snntc_fc_backward(_ptr(grad), _ptr(X), _ptr(W), pp, _ptr(Y), _ptr(dX), _ptr(dW), _ptr(dP),
                                          B, I, J, w_rows, grad.shape[0], _ptr(ws), ws.numel(), _stream(X.device)))
     return dX, dW, dP
@@ -146,8 +148,8 @@ def snncv(X, W, Params, return_aux=False):
     return out
 
 
-def snncv_grad(grad, X, W, Params, Y):
-    """Conv backward -> (dXpad like X, dW like W, dParams[12])."""
+def snncv_grad(grad, X, W, Params, Y, want_dparams=True, want_dx=True, want_dw=True):
+    """Conv backward -> (dXpad like X, dW like W, dParams[12] of zeros, or None if not wanted)."""
     lib = _lib.load()
     grad = _dev_f32(grad, "grad", 4)
     X = _dev_f32(X, "X", 4)
@@ -163,9 +165,9 @@ def snncv_grad(grad, X, W, Params, Y):
         need = ctypes.c_size_t()
         _lib.check(lib.snntc_cv_backward_workspace_bytes(B, H, Wd, C, Kc, pp, ctypes.byref(need)))
         ws = _workspace(X.device, need.value)
-        dX = torch.empty_like(X)
-        dW = torch.empty_like(W)
-        dP = torch.empty(12, dtype=torch.float32, device=X.device)
+        dX = torch.empty_like(X) if want_dx else None
+        dW = torch.empty_like(W) if want_dw else None
+        dP = torch.empty(12, dtype=torch.float32, device=X.device) if want_dparams else None
         _lib.check(lib.snntc_cv_backward(_ptr(grad), _ptr(X), _ptr(W), pp, _ptr(Y), _ptr(dX), _ptr(dW), _ptr(dP),
                                          B, H, Wd, C, Kc, w_rows, grad.shape[0], _ptr(ws), ws.numel(),
                                          _stream(X.device)))
@@ -186,7 +188,8 @@ class SnnFc(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad):
         X, W, Y = ctx.saved_tensors
-        dX, dW, _ = snnfc_grad(grad.contiguous(), X, W, ctx.params, Y)
+        dX, dW, _ = snnfc_grad(grad.contiguous(), X, W, ctx.params, Y, want_dparams=False,
+                               want_dx=ctx.needs_input_grad[0], want_dw=ctx.needs_input_grad[1])
         return dX, dW, None
 
 
@@ -203,5 +206,6 @@ class SnnCv(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad):
         X, W, Y = ctx.saved_tensors
-        dX, dW, _ = snncv_grad(grad.contiguous(), X, W, ctx.params, Y)
+        dX, dW, _ = snncv_grad(grad.contiguous(), X, W, ctx.params, Y, want_dparams=False,
+                               want_dx=ctx.needs_input_grad[0], want_dw=ctx.needs_input_grad[1])
         return dX, dW, None
