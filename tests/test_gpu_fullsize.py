@@ -1,0 +1,113 @@
+"""Parity at the BASELINE configurations' full sizes, where the oracle is too slow to run whole:
+size-independent properties on the complete GPU result plus exact oracle comparison on a slice that
+is independent of the rest (single images / samples)."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import conv_case, dense_case
+from oracle import capi
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def t(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def check_forward_properties(x_seg, w, out, sz, perm, ck, bias, max_time=1e5):
+    """x_seg[S,I] (device) are the segments; all arguments torch tensors on the GPU."""
+    S, I = x_seg.shape
+    J = w.shape[1]
+    # sorted ascending, perm is a permutation that reproduces the sort, ties in index order
+    assert torch.all(sz[:, 1:] >= sz[:, :-1])
+    assert torch.equal(torch.gather(x_seg, 1, perm.long()), sz)
+    assert torch.equal(torch.sort(perm, dim=1).values, torch.arange(I, device=DEV, dtype=perm.dtype).expand(S, I))
+    tie = sz[:, 1:] == sz[:, :-1]
+    assert torch.all(perm[:, 1:][tie] > perm[:, :-1][tie])
+    y, r = out[:S].reshape(S, J), out[S:].reshape(S, J)
+    fired = ck >= 0
+    assert torch.all(y[~fired] == max_time) and torch.all(r[~fired] == 0)
+    assert torch.all(r[fired] != 0) and torch.all(y[fired] < max_time)
+    # the spike lies after the last causal input and not after the next one (1 ulp of slack for
+    # y = ysum * (1/wsum) versus the division-free test the kernel decides with)
+    k = ck.clamp(min=0).long()
+    last = torch.where(k > 0, torch.gather(sz, 1, (k - 1).clamp(min=0)), torch.ones_like(y) if bias else torch.zeros_like(y))
+    nxt = torch.where(k < I, torch.gather(sz, 1, k.clamp(max=I - 1)), torch.full_like(y, max_time))
+    slack = 4e-7 * y.abs()
+    assert torch.all((y + slack >= last)[fired])
+    assert torch.all((y - slack <= nxt)[fired])
+
+
+def test_dense_north_star_layer_full_batch():
+    """B=256, 784 -> 800 with bias (BASELINE config 2, layer 1)."""
+    import snntc_amd as snn
+    x, w, p, g = dense_case(10, 256, 784, 800, True, "baseline")
+    X, W, G = t(x), t(w), t(g)
+    out, sz, perm, ck = snn.snnfc(X, W, p, return_aux=True)
+    check_forward_properties(X, W, out, sz, perm, ck, True)
+    # samples are independent: the first 8 and the last 8 must equal the oracle exactly
+    for sl in (slice(0, 8), slice(248, 256)):
+        ref, rk, _, rperm = capi.fc_forward_dev(x[sl], w, p, want_aux=True)
+        n = sl.stop - sl.start
+        got = torch.cat((out[sl], out[256 + sl.start:256 + sl.stop])).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+        assert np.array_equal(ck[sl].cpu().numpy(), rk) and np.array_equal(perm[sl].cpu().numpy(), rperm)
+    # backward: linear in the upstream gradient, dX independent per sample, dW additive over samples
+    dx, dw, _ = snn.snnfc_grad(G, X, W, p, out)
+    dx2, dw2, _ = snn.snnfc_grad(2 * G, X, W, p, out)
+    assert torch.equal(dx2, 2 * dx) and torch.equal(dw2, 2 * dw)           # scaling by 2 is exact in fp32
+    half = 128
+    oa = torch.cat((out[:half], out[256:256 + half])); ob = torch.cat((out[half:256], out[256 + half:]))
+    ga = torch.cat((G[:half], G[256:256 + half])); gb = torch.cat((G[half:256], G[256 + half:]))
+    dxa, dwa, _ = snn.snnfc_grad(ga, X[:half], W, p, oa)
+    dxb, dwb, _ = snn.snnfc_grad(gb, X[half:], W, p, ob)
+    assert torch.equal(torch.cat((dxa, dxb)), dx)
+    # two summation orders of the same fp32 terms: compare on the scale of the summed magnitudes
+    oabs = out.clone(); oabs[256:] = oabs[256:].abs()
+    _, dw_mag, _ = snn.snnfc_grad(G.abs(), X, W, p, oabs)               # = -sum |x - y| |up|
+    assert torch.all((dwa + dwb - dw).abs() <= 1e-5 * dw.abs() + 1e-6 * dw_mag.abs().clamp(min=1.0))
+    rdx, _, _ = capi.fc_backward_dev(np.concatenate((g[:8], g[256:264])), x[:8], w, p,
+                                     np.concatenate((out[:8].cpu().numpy(), out[256:264].cpu().numpy())), wide=True)
+    assert np.all(np.abs(dx[:8].cpu().numpy() - rdx) <= 1e-5 * np.abs(rdx) + 1e-5)
+
+
+def test_conv_north_star_layer_full_batch():
+    """B=64, 32x32x64 -> 64, 3x3 SAME with bias (BASELINE config 3): 65 536 patches of 576."""
+    import snntc_amd as snn
+    B = 64
+    _, xpad, w, p, g = conv_case(11, B, 32, 32, 64, 64, 3, 3, 1, 1, True, True, "baseline")
+    X, W, G = t(xpad), t(w), t(g)
+    out, sz, perm, ck = snn.snncv(X, W, p, return_aux=True)
+    # patches as the op sees them (built with torch.unfold on the device, independent of the kernels)
+    patches = X.unfold(1, 3, 1).unfold(2, 3, 1)                       # [B,Nh,Nw,C,kh,kw]
+    patches = patches.permute(0, 1, 2, 4, 5, 3).reshape(B * 32 * 32, 576)
+    check_forward_properties(patches, W, out.reshape(2 * B * 1024, 64), sz, perm, ck, True)
+    # images are independent: first and last image against the oracle, exactly
+    for b in (0, B - 1):
+        ref, rk, _, rperm = capi.cv_forward_dev(xpad[b:b + 1], w, p, want_aux=True)
+        got = torch.stack((out[b], out[B + b])).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+        assert np.array_equal(ck[b * 1024:(b + 1) * 1024].cpu().numpy(), rk)
+        assert np.array_equal(perm[b * 1024:(b + 1) * 1024].cpu().numpy(), rperm)
+    dx, dw, _ = snn.snncv_grad(G, X, W, p, out)
+    dx2, dw2, _ = snn.snncv_grad(2 * G, X, W, p, out)
+    assert torch.equal(dx2, 2 * dx) and torch.equal(dw2, 2 * dw)
+    assert torch.all(dx[X > 99999.0] == 0)                             # padding receives no gradient
+    # one image: dX exact slice of the batch result, and against the oracle
+    o1 = torch.stack((out[0], out[B])); g1 = torch.stack((G[0], G[B]))
+    dx1, dw1, _ = snn.snncv_grad(g1, X[:1], W, p, o1)
+    assert torch.equal(dx1[0], dx[0])
+    rdx, rdw, _ = capi.cv_backward_dev(g1.cpu().numpy(), xpad[:1], w, p, o1.cpu().numpy(), wide=True)
+    assert np.all(np.abs(dx1.cpu().numpy() - rdx) <= 1e-5 * np.abs(rdx) + 1e-5)
+    assert np.all(np.abs(dw1.cpu().numpy() - rdw) <= 1e-5 * np.abs(rdw) + 1e-4)
+    # dW of the batch = sum of per-image dW (computed by the same kernels on single images)
+    acc = torch.zeros_like(dw, dtype=torch.float64)
+    for b in range(0, B, 8):
+        ob = torch.cat((out[b:b + 8], out[B + b:B + b + 8])); gb = torch.cat((G[b:b + 8], G[B + b:B + b + 8]))
+        _, dwb, _ = snn.snncv_grad(gb, X[b:b + 8], W, p, ob)
+        acc += dwb.double()
+    oabs = out.clone(); oabs[B:] = oabs[B:].abs()
+    _, dw_mag, _ = snn.snncv_grad(G.abs(), X, W, p, oabs)               # = -sum |x - y| |up|
+    assert torch.all((acc - dw.double()).abs() <= 1e-5 * acc.abs() + 1e-6 * dw_mag.abs().double().clamp(min=1.0))
