@@ -125,14 +125,21 @@ int fc_check(int64_t B, int64_t I, int64_t J, int64_t w_rows, const float* param
     return SNNTC_OK;
 }
 
-struct FcFwdWs { float* sorted; int32_t* perm; int32_t* n_real; int64_t stride; size_t bytes; };
-FcFwdWs fc_fwd_ws(void* ws, int64_t S, int64_t I) {
+// Forward scratch.  n_pix / pix_c > 0 adds the per-pixel sorted channels the conv merge path needs.
+struct FcFwdWs {
+    float* sorted; int32_t* perm; int32_t* n_real; float* pix_z; int32_t* pix_c;
+    int64_t stride, pix_stride; size_t bytes;
+};
+FcFwdWs fc_fwd_ws(void* ws, int64_t S, int64_t I, int64_t n_pix = 0, int64_t pix_c = 0) {
     Carver c(ws);
     FcFwdWs r;
     r.stride = padded_stride(I);
+    r.pix_stride = padded_stride(pix_c);
     r.sorted = c.take<float>(S * r.stride);
     r.perm = c.take<int32_t>(S * r.stride);
     r.n_real = c.take<int32_t>(S);
+    r.pix_z = c.take<float>(n_pix * r.pix_stride);
+    r.pix_c = c.take<int32_t>(n_pix * r.pix_stride);
     r.bytes = c.used;
     return r;
 }
@@ -241,12 +248,26 @@ int cv_forward_impl(const float* xpad, const float* w, const float* params, floa
     if (rc) return rc;
     if (g.S == 0 || Kc == 0) return SNNTC_OK;
     if (!xpad || !w || !out) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_cv_forward: NULL tensor pointer");
-    FcFwdWs ws = fc_fwd_ws(workspace, g.S, g.P);
+    const bool merge = merge_sort_supported(g);
+    FcFwdWs ws = fc_fwd_ws(workspace, g.S, g.P, merge ? B * H * W : 0, merge ? C : 0);
     rc = check_workspace(workspace, workspace_bytes, ws.bytes);
     if (rc) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const NeuronParams np = neuron_params(params[0], params[4], params[11]);
-    return forward_chain(conv_source(xpad, g), ws, w, out, sorted_z, perm, causal_k, g.S, g.P, Kc, np, st);
+    if (!merge)
+        return forward_chain(conv_source(xpad, g), ws, w, out, sorted_z, perm, causal_k, g.S, g.P, Kc, np, st);
+    // sort every pixel's channels once, then assemble the patches by rank merging
+    SegmentSource pixels{};
+    pixels.base = xpad; pixels.conv = 0; pixels.I = (int)C;
+    rc = launch_sort(pixels, B * H * W, ws.pix_z, ws.pix_c, nullptr, (int)ws.pix_stride, np.max_cmp, st);
+    if (rc) return rc;
+    rc = launch_merge_patches(ws.pix_z, ws.pix_c, ws.pix_stride, ws.sorted, ws.perm, ws.n_real, g, ws.stride,
+                              np.max_cmp, st);
+    if (rc) return rc;
+    rc = launch_unpad_rows(ws.sorted, ws.perm, sorted_z, perm, g.S, g.P, ws.stride, st);
+    if (rc) return rc;
+    return launch_scan(ws.sorted, ws.perm, ws.n_real, w, out, out + g.S * Kc, causal_k, g.S, g.P, ws.stride, Kc, np,
+                       st);
 }
 
 }  // namespace
@@ -381,7 +402,8 @@ int snntc_cv_forward_workspace_bytes(int64_t B, int64_t H, int64_t W, int64_t C,
     int rc = cv_geom(B, H, W, C, Kc, 0, params_host, false, "snntc_cv_forward_workspace_bytes", &g);
     if (rc) return rc;
     if (!bytes) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_cv_forward_workspace_bytes: bytes is NULL");
-    *bytes = fc_fwd_ws(nullptr, g.S, g.P).bytes;
+    const bool merge = merge_sort_supported(g);
+    *bytes = fc_fwd_ws(nullptr, g.S, g.P, merge ? B * H * W : 0, merge ? C : 0).bytes;
     return SNNTC_OK;
 }
 

@@ -68,6 +68,12 @@ inline int64_t padded_stride(int64_t I) { return (I + 15) / 16 * 16; }
 int launch_sort(const SegmentSource& src, int64_t S, float* sorted, int32_t* perm, int32_t* n_real,
                 int out_stride, float max_cmp, hipStream_t stream);
 
+// Conv patch sort by merging pre-sorted pixels (merge.hip): pix_z / pix_c are the [B*H*W, Cs] outputs
+// of launch_sort on the image's pixels.
+bool merge_sort_supported(const ConvGeom& g);
+int launch_merge_patches(const float* pix_z, const int32_t* pix_c, int64_t Cs, float* sorted, int32_t* perm,
+                         int32_t* n_real, const ConvGeom& g, int64_t stride, float max_cmp, hipStream_t stream);
+
 // Copies the first I entries of every padded row into dense [S,I] arrays (either may be NULL).
 int launch_unpad_rows(const float* sorted, const int32_t* perm, float* sorted_out, int32_t* perm_out,
                       int64_t S, int64_t I, int64_t stride, hipStream_t stream);

@@ -92,6 +92,9 @@ CONV_CASES = [
     (5, 2, 9, 9, 4, 70, 5, 6, 2, 3, True, False, "reftest"),
     (6, 1, 8, 8, 128, 128, 3, 3, 1, 1, True, True, "baseline"),     # P = 1152
     (7, 1, 4, 4, 512, 96, 3, 3, 1, 1, True, True, "baseline"),      # P = 4608
+    (8, 2, 10, 9, 48, 20, 3, 2, 2, 1, True, True, "reftest"),       # channels not a power of two
+    (9, 2, 9, 9, 32, 16, 3, 3, 2, 2, True, False, "baseline"),      # stride 2 with 32 channels
+    (10, 1, 12, 7, 40, 8, 2, 3, 1, 2, False, True, "reftest"),      # VALID, ragged kernel and stride
 ]
 
 
@@ -120,3 +123,25 @@ def test_conv_forward_backward(seed, B, H, W, C, Kc, Kh, Kw, Sh, Sw, same, bias,
     check_grad(dx, rdx, adx, "dXpad")
     check_grad(dw, rdw, adw, "dW")
     assert np.all(dp == 0)
+
+
+@pytest.mark.parametrize("C,Kh,Kw,Sh,Sw", [(32, 3, 3, 1, 1), (64, 3, 3, 1, 1), (3, 3, 3, 1, 1), (40, 2, 3, 1, 2)])
+def test_conv_sort_with_heavy_ties(C, Kh, Kw, Sh, Sw):
+    """Quantised inputs: most values repeat inside a patch (and SAME padding adds runs of 1e5), so
+    the permutation is decided by the stable tie rule (kh, kw, c) almost everywhere."""
+    import snntc_amd as snn
+    from oracle.closed_form import same_pad
+    rng = np.random.default_rng(C + Kh)
+    B, H, W, Kc = 2, 7, 9, 16
+    x = (1.0 + rng.integers(0, 6, (B, H, W, C)) / 4.0).astype(np.float32)
+    (tp, bt), (lf, rt) = same_pad(H, Kh, Sh), same_pad(W, Kw, Sw)
+    xpad = np.ascontiguousarray(np.pad(x, ((0, 0), (tp, bt), (lf, rt), (0, 0)), constant_values=np.float32(1e5)))
+    w = (rng.standard_normal((Kh * Kw * C + 1, Kc)) * 0.3 + 0.05).astype(np.float32)
+    p = capi.cv_params(Kh, Kw, Sh, Sw, same=True, biasvolt=1.0)
+    ref_out, ref_k, ref_sorted, ref_perm = capi.cv_forward_dev(xpad, w, p, want_aux=True)
+    out, sz, perm, ck = snn.snncv(t(xpad), t(w), p, return_aux=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(perm.cpu().numpy(), ref_perm), "permutation differs"
+    assert np.array_equal(sz.cpu().numpy(), ref_sorted)
+    assert np.array_equal(ck.cpu().numpy(), ref_k)
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), ref_out.view(np.uint32))
