@@ -221,7 +221,57 @@ __device__ __forceinline__ void scan_chunk(float& wsum, float& ysum, float& ya, 
     }
 }
 
-template <int COLS, bool WANT_K>
+// The same eight steps with every decision kept on the vector side: instead of a fired mask the
+// lane carries a gate value yg = fired ? ya : +inf, the closing test `yg > x*|wsum|` writes EXEC
+// directly and the new gate is a select.  One more vector instruction per step, but no
+// vector -> scalar -> EXEC round trips, so a step of a lone wavefront takes far fewer cycles: used
+// when a launch has too few wavefronts per SIMD to hide that latency.
+#define SNNTC_VSCAN_STEP(U)                                                  \
+    "v_mul_f32_e64 %[t], %[x" #U "], |%[wsum]|\n"                            \
+    "v_cmpx_gt_f32_e32 vcc, %[yg], %[t]\n"                                   \
+    "v_add_f32_e32 %[wsum], %[wsum], %[w" #U "]\n"                           \
+    "v_fmac_f32_e32 %[ysum], %[x" #U "], %[w" #U "]\n"                       \
+    "v_cmp_gt_f32_e32 vcc, 0, %[wsum]\n"                                     \
+    "v_cndmask_b32_e64 %[ya], %[ysum], -%[ysum], vcc\n"                      \
+    "v_mul_f32_e64 %[t], %[x" #U "], |%[wsum]|\n"                            \
+    "v_cmp_gt_f32_e32 vcc, %[ya], %[t]\n"                                    \
+    "v_cndmask_b32_e32 %[yg], %[inf], %[ya], vcc\n"
+#define SNNTC_VSCAN_PROLOGUE                        \
+    "s_mov_b64 %[save], exec\n"                     \
+    "s_mov_b64 exec, %[run]\n"
+#define SNNTC_VSCAN_EPILOGUE                         \
+    "s_andn2_b64 %[gone], %[run], exec\n"            \
+    "s_or_b64 %[closed], %[closed], %[gone]\n"       \
+    "s_mov_b64 exec, %[save]\n"
+#define SNNTC_VSCAN_STATE                                                                              \
+    [wsum] "+v"(wsum), [ysum] "+v"(ysum), [ya] "+v"(ya), [yg] "+v"(yg), [kcnt] "+v"(kcnt),             \
+        [closed] "+s"(closed), [save] "=&s"(saved_exec), [gone] "=&s"(gone), [t] "=&v"(t)
+#define SNNTC_VSCAN_INPUTS                                                                             \
+    [run] "s"(run), [inf] "v"(inf), [x0] "v"(x[0]), [x1] "v"(x[1]), [x2] "v"(x[2]), [x3] "v"(x[3]),     \
+        [x4] "v"(x[4]), [x5] "v"(x[5]), [x6] "v"(x[6]), [x7] "v"(x[7]), [w0] "v"(w[0]), [w1] "v"(w[1]), \
+        [w2] "v"(w[2]), [w3] "v"(w[3]), [w4] "v"(w[4]), [w5] "v"(w[5]), [w6] "v"(w[6]), [w7] "v"(w[7])
+
+template <bool WANT_K>
+__device__ __forceinline__ void scan_chunk_vector(float& wsum, float& ysum, float& ya, float& yg, int& kcnt,
+                                                  uint64_t& closed, uint64_t run, const float (&x)[CHUNK],
+                                                  const float (&w)[CHUNK]) {
+    uint64_t saved_exec, gone;
+    float t;
+    const float inf = INFINITY;
+    if (WANT_K)
+        asm volatile(SNNTC_VSCAN_PROLOGUE SNNTC_VSCAN_STEP(0) SNNTC_SCAN_COUNT SNNTC_VSCAN_STEP(1) SNNTC_SCAN_COUNT
+                     SNNTC_VSCAN_STEP(2) SNNTC_SCAN_COUNT SNNTC_VSCAN_STEP(3) SNNTC_SCAN_COUNT SNNTC_VSCAN_STEP(4)
+                     SNNTC_SCAN_COUNT SNNTC_VSCAN_STEP(5) SNNTC_SCAN_COUNT SNNTC_VSCAN_STEP(6) SNNTC_SCAN_COUNT
+                     SNNTC_VSCAN_STEP(7) SNNTC_SCAN_COUNT SNNTC_VSCAN_EPILOGUE
+                     : SNNTC_VSCAN_STATE : SNNTC_VSCAN_INPUTS : "vcc");
+    else
+        asm volatile(SNNTC_VSCAN_PROLOGUE SNNTC_VSCAN_STEP(0) SNNTC_VSCAN_STEP(1) SNNTC_VSCAN_STEP(2)
+                     SNNTC_VSCAN_STEP(3) SNNTC_VSCAN_STEP(4) SNNTC_VSCAN_STEP(5) SNNTC_VSCAN_STEP(6)
+                     SNNTC_VSCAN_STEP(7) SNNTC_VSCAN_EPILOGUE
+                     : SNNTC_VSCAN_STATE : SNNTC_VSCAN_INPUTS : "vcc");
+}
+
+template <int COLS, bool WANT_K, bool LOW_LATENCY>
 __global__ void __launch_bounds__(LDS_SCAN_THREADS)
 scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
                 const int32_t* __restrict__ n_real, const float* __restrict__ w, float* __restrict__ y_out,
@@ -269,6 +319,7 @@ scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ pe
         uint64_t fired = __ballot(fired0);
         uint64_t closed = 0;
         int kcnt = 0;
+        float yg = fired0 ? ya : INFINITY;                  // gate value of the vector-only step
 
         // Three chunks of (x, row) are in flight: c is consumed, c+1 feeds the LDS reads, c+2 is
         // being fetched.  The phase loop is unrolled so that buffer indices are compile-time.
@@ -290,7 +341,11 @@ scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ pe
                 load_chunk(xp[(ph + 2) % 3], xs, pr, kn <= last_chunk ? kn : 0);
 #pragma unroll
                 for (int u = 0; u < CHUNK; ++u) wv[(ph + 1) % 2][u] = wcol[xp[(ph + 1) % 3].p[u] * COLS];
-                scan_chunk<WANT_K, COLS == kWave>(wsum, ysum, ya, kcnt, fired, closed, run, xp[ph % 3].x, wv[ph % 2]);
+                if (LOW_LATENCY)
+                    scan_chunk_vector<WANT_K>(wsum, ysum, ya, yg, kcnt, closed, run, xp[ph % 3].x, wv[ph % 2]);
+                else
+                    scan_chunk<WANT_K, COLS == kWave>(wsum, ysum, ya, kcnt, fired, closed, run, xp[ph % 3].x,
+                                                      wv[ph % 2]);
             }
             if (stop) break;
         }
@@ -300,7 +355,7 @@ scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ pe
             LaneState s;
             s.wsum = wsum; s.ysum = ysum; s.wa = fabsf(wsum); s.ya = ya;
             const bool was_closed = (closed >> lane) & 1;
-            s.fired = was_closed || ((fired >> lane) & 1);
+            s.fired = was_closed || (LOW_LATENCY ? yg < INFINITY : (bool)((fired >> lane) & 1));
             bool open = !was_closed;
             for (int k = n_full; k < n && open; ++k) {
                 open = scan_step(s, xs[k], wcol[pr[k] * COLS]);
@@ -355,17 +410,21 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     const int64_t max_groups = (items + WAVES - 1) / WAVES;
     if (n_groups > max_groups) n_groups = max_groups;
     if (n_groups < 1) n_groups = 1;
-    auto kern_k = scan_lds_kernel<COLS, true>;
-    auto kern = scan_lds_kernel<COLS, false>;
+    // few resident wavefronts per SIMD cannot hide the scalar round trips of the regular step
+    const int64_t waves = (int64_t)n_slices * n_groups * WAVES;
+    const int64_t busy_waves = items * n_slices < waves ? items * n_slices : waves;
+    const bool low_latency = busy_waves <= (int64_t)cus * 4 * 5;
+    auto kern_k = low_latency ? scan_lds_kernel<COLS, true, true> : scan_lds_kernel<COLS, true, false>;
+    auto kern = low_latency ? scan_lds_kernel<COLS, false, true> : scan_lds_kernel<COLS, false, false>;
     // raise the dynamic-LDS limit of both instantiations once (not per launch: the call is not
     // allowed while a stream is being captured into a graph)
-    static bool lds_limit_raised = false;
-    if (!lds_limit_raised) {
+    static bool lds_limit_raised[2] = {false, false};
+    if (!lds_limit_raised[low_latency]) {
         SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern_k),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, LDS_SCAN_BYTES));
         SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, LDS_SCAN_BYTES));
-        lds_limit_raised = true;
+        lds_limit_raised[low_latency] = true;
     }
     dim3 grid((unsigned)(n_slices * n_groups)), block(LDS_SCAN_THREADS);
     {
