@@ -140,8 +140,24 @@ struct Chunk {
     int32_t p[CHUNK];
 };
 
-__device__ __forceinline__ void load_chunk(Chunk& c, const float* __restrict__ xs,
-                                           const int32_t* __restrict__ pr, int k) {
+// Rows are read through buffer descriptors: a scalar descriptor (first row of the work item), a
+// scalar chunk offset and a per-lane byte offset that never changes during a scan.  No per-lane
+// address arithmetic is left, so issuing the next loads never has to wait for those in flight.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+struct RowSource {
+    __amdgpu_buffer_rsrc_t xs, pr;
+};
+
+__device__ __forceinline__ RowSource make_row_source(const float* xs0, const int32_t* pr0, int bytes) {
+    RowSource r;
+    r.xs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(xs0), 0, bytes, 0x00020000);
+    r.pr = __builtin_amdgcn_make_buffer_rsrc(const_cast<int32_t*>(pr0), 0, bytes, 0x00020000);
+    return r;
+}
+
+__device__ __forceinline__ void load_chunk_flat(Chunk& c, const float* __restrict__ xs,
+                                                const int32_t* __restrict__ pr, int k) {
     const float4 a = *reinterpret_cast<const float4*>(xs + k);
     const float4 b = *reinterpret_cast<const float4*>(xs + k + 4);
     const int4 pa = *reinterpret_cast<const int4*>(pr + k);
@@ -150,6 +166,18 @@ __device__ __forceinline__ void load_chunk(Chunk& c, const float* __restrict__ x
     c.x[4] = b.x; c.x[5] = b.y; c.x[6] = b.z; c.x[7] = b.w;
     c.p[0] = pa.x; c.p[1] = pa.y; c.p[2] = pa.z; c.p[3] = pa.w;
     c.p[4] = pb.x; c.p[5] = pb.y; c.p[6] = pb.z; c.p[7] = pb.w;
+}
+
+__device__ __forceinline__ void load_chunk(Chunk& c, const RowSource& src, int lane_bytes, int k) {
+    const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(src.xs, lane_bytes, k * 4, 0);
+    const u32x4 b = __builtin_amdgcn_raw_buffer_load_b128(src.xs, lane_bytes + 16, k * 4, 0);
+    const u32x4 pa = __builtin_amdgcn_raw_buffer_load_b128(src.pr, lane_bytes, k * 4, 0);
+    const u32x4 pb = __builtin_amdgcn_raw_buffer_load_b128(src.pr, lane_bytes + 16, k * 4, 0);
+    c.x[0] = __uint_as_float(a.x); c.x[1] = __uint_as_float(a.y); c.x[2] = __uint_as_float(a.z);
+    c.x[3] = __uint_as_float(a.w); c.x[4] = __uint_as_float(b.x); c.x[5] = __uint_as_float(b.y);
+    c.x[6] = __uint_as_float(b.z); c.x[7] = __uint_as_float(b.w);
+    c.p[0] = (int)pa.x; c.p[1] = (int)pa.y; c.p[2] = (int)pa.z; c.p[3] = (int)pa.w;
+    c.p[4] = (int)pb.x; c.p[5] = (int)pb.y; c.p[6] = (int)pb.z; c.p[7] = (int)pb.w;
 }
 
 // Eight scan steps for the lanes in `run`, written out by hand: the closing test of a step simply
@@ -271,23 +299,61 @@ __device__ __forceinline__ void scan_chunk_vector(float& wsum, float& ysum, floa
                      : SNNTC_VSCAN_STATE : SNNTC_VSCAN_INPUTS : "vcc");
 }
 
+// LOW_LATENCY is the instantiation for launches with at most a couple of wavefronts per SIMD, where
+// nothing hides a stall: workgroups of at most four wavefronts (so that the work spreads over the
+// chip), seven chunks of (x, row) in flight instead of two, and the vector-only step block.
+constexpr int LOW_LATENCY_THREADS = 256;
+
 template <int COLS, bool WANT_K, bool LOW_LATENCY>
-__global__ void __launch_bounds__(LDS_SCAN_THREADS)
+__global__ void __launch_bounds__(LOW_LATENCY ? LOW_LATENCY_THREADS : LDS_SCAN_THREADS)
 scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
                 const int32_t* __restrict__ n_real, const float* __restrict__ w, float* __restrict__ y_out,
                 float* __restrict__ rcp_out, int32_t* __restrict__ k_out, int S, int I, int stride, int J,
                 int n_slices, int n_groups, NeuronParams np) {
     extern __shared__ float wl[];                          // [I + bias][COLS]
     constexpr int SEGS = kWave / COLS;                     // segments per wavefront
-    constexpr int WAVES = LDS_SCAN_THREADS / kWave;
+    const int WAVES = blockDim.x / kWave;                  // 1..16, chosen by the launcher
     const int slice = blockIdx.x % n_slices;
     const int group = blockIdx.x / n_slices;
     const int j0 = slice * COLS;
     const int rows = I + np.bias;
 
-    for (int idx = threadIdx.x; idx < rows * COLS; idx += LDS_SCAN_THREADS) {
-        const int r = idx / COLS, c = idx - r * COLS;
-        wl[idx] = (j0 + c < J) ? w[(size_t)r * J + j0 + c] : 0.0f;
+    // copy the column slice of W; loads are issued in batches so that a small workgroup does not
+    // pay one memory latency per element
+    const int n_fill = rows * COLS;
+    if ((J & 3) == 0) {
+        constexpr int C4 = COLS / 4, FILL = 4;
+        for (int base = threadIdx.x; base < rows * C4; base += FILL * blockDim.x) {
+            float4 v[FILL];
+#pragma unroll
+            for (int u = 0; u < FILL; ++u) {
+                const int idx = base + u * blockDim.x;
+                const int r = idx / C4, c = (idx - r * C4) * 4;
+                v[u] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                if (idx < rows * C4 && j0 + c < J) v[u] = *reinterpret_cast<const float4*>(w + (size_t)r * J + j0 + c);
+            }
+#pragma unroll
+            for (int u = 0; u < FILL; ++u) {
+                const int idx = base + u * blockDim.x;
+                if (idx < rows * C4) reinterpret_cast<float4*>(wl)[idx] = v[u];
+            }
+        }
+    } else {
+        constexpr int FILL = 16;
+        for (int base = threadIdx.x; base < n_fill; base += FILL * blockDim.x) {
+            float v[FILL];
+#pragma unroll
+            for (int u = 0; u < FILL; ++u) {
+                const int idx = base + u * blockDim.x;
+                const int r = idx / COLS, c = idx - r * COLS;
+                v[u] = (idx < n_fill && j0 + c < J) ? w[(size_t)r * J + j0 + c] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < FILL; ++u) {
+                const int idx = base + u * blockDim.x;
+                if (idx < n_fill) wl[idx] = v[u];
+            }
+        }
     }
     __syncthreads();
 
@@ -304,6 +370,11 @@ scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ pe
         const int seg = seg_raw < S ? seg_raw : S - 1;      // idle lanes shadow a valid segment
         const float* __restrict__ xs = sorted + (size_t)seg * stride;
         const int32_t* __restrict__ pr = perm + (size_t)seg * stride;
+        const int seg0 = __builtin_amdgcn_readfirstlane(item * SEGS);
+        const int n_segs = S - seg0 < SEGS ? S - seg0 : SEGS;
+        const RowSource rows_of_item = make_row_source(sorted + (size_t)seg0 * stride, perm + (size_t)seg0 * stride,
+                                                       n_segs * stride * (int)sizeof(float));
+        const int lane_bytes = (seg - seg0) * stride * (int)sizeof(float);
         const int n = live ? n_real[seg] : 0;
         const int n_full = n & ~(CHUNK - 1);
 
@@ -321,33 +392,45 @@ scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ pe
         int kcnt = 0;
         float yg = fired0 ? ya : INFINITY;                  // gate value of the vector-only step
 
-        // Three chunks of (x, row) are in flight: c is consumed, c+1 feeds the LDS reads, c+2 is
-        // being fetched.  The phase loop is unrolled so that buffer indices are compile-time.
-        Chunk xp[3];
+        // NBUF chunks of (x, row) are held: c is consumed, c+1 feeds the LDS reads, up to c+NBUF-1
+        // are being fetched.  The phase loop is unrolled so that buffer indices are compile-time.
+        constexpr int NBUF = LOW_LATENCY ? 8 : 3, AHEAD = NBUF - 1;
+        constexpr int PHASES = (NBUF % 2 == 0) ? NBUF : 2 * NBUF;
+        Chunk xp[NBUF];
         float wv[2][CHUNK];
-        load_chunk(xp[0], xs, pr, 0);
-        load_chunk(xp[1], xs, pr, CHUNK <= last_chunk ? CHUNK : 0);
+#pragma unroll
+        for (int b = 0; b < AHEAD; ++b) {
+            const int kb = b * CHUNK <= last_chunk ? b * CHUNK : 0;
+            if (LOW_LATENCY) load_chunk(xp[b], rows_of_item, lane_bytes, kb);
+            else load_chunk_flat(xp[b], xs, pr, kb);
+        }
 #pragma unroll
         for (int u = 0; u < CHUNK; ++u) wv[0][u] = wcol[xp[0].p[u] * COLS];
 
-        for (int k0 = 0;; k0 += 6 * CHUNK) {
+        // LOW_LATENCY: the body is one straight block per PHASES chunks (no exit between phases: a
+        // phase whose lanes are all done runs with an empty EXEC), which lets the compiler keep
+        // all seven chunks in flight; the regular instantiation leaves as soon as nothing runs.
+        for (int k0 = 0;; k0 += PHASES * CHUNK) {
             bool stop = false;
 #pragma unroll
-            for (int ph = 0; ph < 6; ++ph) {
+            for (int ph = 0; ph < PHASES; ++ph) {
+                if (LOW_LATENCY) __builtin_amdgcn_sched_barrier(0);   // keep each phase's loads and reads in it
                 const int k = k0 + ph * CHUNK;
                 const uint64_t run = __ballot(k < n_full) & ~closed;
-                if (run == 0) { stop = true; break; }
-                const int kn = k + 2 * CHUNK;
-                load_chunk(xp[(ph + 2) % 3], xs, pr, kn <= last_chunk ? kn : 0);
+                if (!LOW_LATENCY && run == 0) { stop = true; break; }
+                const int kn = k + AHEAD * CHUNK;
+                const int kf = kn <= last_chunk ? kn : 0;
+                if (LOW_LATENCY) load_chunk(xp[(ph + AHEAD) % NBUF], rows_of_item, lane_bytes, kf);
+                else load_chunk_flat(xp[(ph + AHEAD) % NBUF], xs, pr, kf);
 #pragma unroll
-                for (int u = 0; u < CHUNK; ++u) wv[(ph + 1) % 2][u] = wcol[xp[(ph + 1) % 3].p[u] * COLS];
+                for (int u = 0; u < CHUNK; ++u) wv[(ph + 1) % 2][u] = wcol[xp[(ph + 1) % NBUF].p[u] * COLS];
                 if (LOW_LATENCY)
-                    scan_chunk_vector<WANT_K>(wsum, ysum, ya, yg, kcnt, closed, run, xp[ph % 3].x, wv[ph % 2]);
+                    scan_chunk_vector<WANT_K>(wsum, ysum, ya, yg, kcnt, closed, run, xp[ph % NBUF].x, wv[ph % 2]);
                 else
-                    scan_chunk<WANT_K, COLS == kWave>(wsum, ysum, ya, kcnt, fired, closed, run, xp[ph % 3].x,
+                    scan_chunk<WANT_K, COLS == kWave>(wsum, ysum, ya, kcnt, fired, closed, run, xp[ph % NBUF].x,
                                                       wv[ph % 2]);
             }
-            if (stop) break;
+            if (stop || (__ballot(k0 + PHASES * CHUNK < n_full) & ~closed) == 0) break;
         }
 
         // per-lane epilogue: up to CHUNK-1 trailing inputs, then the output
@@ -401,19 +484,22 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
         SNNTC_HIP_CHECK(hipGetDeviceProperties(&prop, dev));
         cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
     }
-    constexpr int SEGS = kWave / COLS, WAVES = LDS_SCAN_THREADS / kWave;
+    constexpr int SEGS = kWave / COLS;
     const int n_slices = (int)((J + COLS - 1) / COLS);
     const int64_t items = (S + SEGS - 1) / SEGS;
-    // one resident workgroup per CU: split the segments so that slices x groups covers the chip
+    // A launch that cannot put more than two wavefronts on every SIMD runs the low-latency
+    // instantiation, in workgroups small enough (4, 2 or 1 wavefronts) to reach every CU: the same
+    // work packed into a few full workgroups would leave most of the chip idle.
+    const bool low_latency = items * n_slices <= (int64_t)cus * 4 * 2;
+    int WAVES = (low_latency ? LOW_LATENCY_THREADS : LDS_SCAN_THREADS) / kWave;
+    if (low_latency)
+        while (WAVES > 1 && (int64_t)n_slices * ((items + WAVES - 1) / WAVES) < cus) WAVES >>= 1;
+    // resident workgroups per CU: split the segments so that slices x groups covers the chip
     const int wgs_per_cu = lds_bytes * 2 <= (size_t)LDS_SCAN_BYTES ? 2 : 1;
     int64_t n_groups = ((int64_t)cus * wgs_per_cu + n_slices - 1) / n_slices;
     const int64_t max_groups = (items + WAVES - 1) / WAVES;
     if (n_groups > max_groups) n_groups = max_groups;
     if (n_groups < 1) n_groups = 1;
-    // few resident wavefronts per SIMD cannot hide the scalar round trips of the regular step
-    const int64_t waves = (int64_t)n_slices * n_groups * WAVES;
-    const int64_t busy_waves = items * n_slices < waves ? items * n_slices : waves;
-    const bool low_latency = busy_waves <= (int64_t)cus * 4 * 5;
     auto kern_k = low_latency ? scan_lds_kernel<COLS, true, true> : scan_lds_kernel<COLS, true, false>;
     auto kern = low_latency ? scan_lds_kernel<COLS, false, true> : scan_lds_kernel<COLS, false, false>;
     // raise the dynamic-LDS limit of both instantiations once (not per launch: the call is not
@@ -426,7 +512,7 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
                                             hipFuncAttributeMaxDynamicSharedMemorySize, LDS_SCAN_BYTES));
         lds_limit_raised[low_latency] = true;
     }
-    dim3 grid((unsigned)(n_slices * n_groups)), block(LDS_SCAN_THREADS);
+    dim3 grid((unsigned)(n_slices * n_groups)), block((unsigned)(WAVES * kWave));
     {
         KernelTimerScope timer_("scan", stream);
         if (causal_k)
