@@ -90,8 +90,7 @@ class MlpTrainStep(Workload):
         loss = self.snn.loss_func(self.forward(), self.onehot)
         grads = torch.autograd.grad(loss, self.params)
         with torch.no_grad():
-            for p, g in zip(self.params, grads):
-                p.add_(g, alpha=-self.lr)
+            torch._foreach_add_(self.params, list(grads), alpha=-self.lr)     # SGD, one multi-tensor kernel
         return loss
 
     def layers(self):
@@ -185,8 +184,7 @@ class CifarTrainStep(Workload):
         loss = self.snn.loss_func(self.forward(), self.onehot)
         grads = torch.autograd.grad(loss, self.params)
         with torch.no_grad():
-            for p, g in zip(self.params, grads):
-                p.add_(g, alpha=-self.lr)
+            torch._foreach_add_(self.params, list(grads), alpha=-self.lr)     # SGD, one multi-tensor kernel
         return loss
 
     def layers(self):

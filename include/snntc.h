@@ -103,7 +103,8 @@ SNNTC_API int snntc_fc_forward_ex(const float* x, const float* w, const float* p
                         int64_t B, int64_t I, int64_t J, int64_t w_rows,
                         void* workspace, size_t workspace_bytes, void* stream);
 
-/* grad[grad_rows,J] (only rows [0,B) are read), oldout[2B,J] = the forward output.
+/* grad[grad_rows,J] (only rows [0,B) are read, so a buffer holding just those rows may be passed with
+ * grad_rows still declared as 2B), oldout[2B,J] = the forward output.
  * dx[B,I], dw[w_rows,J], dparams[6] (device; written with zeros).  Any of the three outputs may be
  * NULL: that gradient is then not computed (the reference always computes all of them).
  * Errors: grad_rows != 2B -> DIM_MISMATCH (snntc/snnfcgrad_kernels.cc:119-120); sizes as above. */

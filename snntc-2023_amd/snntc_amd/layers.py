@@ -12,7 +12,7 @@ import numpy as np
 import torch
 import torch.nn.functional as F
 
-from .ops import SnnCv, SnnFc
+from .ops import SnnCvTimes, SnnFcTimes
 
 # Mirrors the reference's module-level switch (SNN_TC_Modules.py:11): when True the layers keep
 # the largest batch and element count they have seen in ``maxD`` (every tensor must stay below
@@ -94,8 +94,7 @@ class SNN_dense(torch.nn.Module, _CostsMixin):
         if Check_Dim:
             self.maxD[0] = max(self.maxD[0], int(B))
             self.maxD[1] = max(self.maxD[1], int(B) * int(X.shape[1]))
-        Y = SnnFc.apply(X, self.weight, self.Params)
-        return Y[:B]
+        return SnnFcTimes.apply(X, self.weight, self.Params)      # Y[:B] of the [2B,J] op output
 
 
 class SNN_conv(torch.nn.Module, _CostsMixin):
@@ -146,8 +145,7 @@ class SNN_conv(torch.nn.Module, _CostsMixin):
         if Check_Dim:
             self.maxD[0] = max(self.maxD[0], int(B))
             self.maxD[1] = max(self.maxD[1], int(X.numel()))
-        Y = SnnCv.apply(X.contiguous(), self.weight, self.Params)
-        return Y[:B]
+        return SnnCvTimes.apply(X.contiguous(), self.weight, self.Params)   # Y[:B] of the op output
 
 
 class SNN_LRN(torch.nn.Module):

@@ -85,7 +85,7 @@ def snnfc(X, W, Params, return_aux=False):
     return out
 
 
-def snnfc_grad(grad, X, W, Params, Y, want_dparams=True, want_dx=True, want_dw=True):
+def snnfc_grad(grad, X, W, Params, Y, want_dparams=True, want_dx=True, want_dw=True, first_half_grad=False):
     """Dense backward.  grad[2B,J], Y[2B,J] = forward output -> (dX[B,I], dW like W, dParams[6]).
     dParams is all zeros (Params is a constant).  A want_* flag set to False skips that gradient
     (None is returned in its place)."""
@@ -107,8 +107,10 @@ def snnfc_grad(grad, X, W, Params, Y, want_dparams=True, want_dx=True, want_dw=T
         dX = torch.empty_like(X) if want_dx else None
         dW = torch.empty_like(W) if want_dw else None
         dP = torch.empty(6, dtype=torch.float32, device=X.device) if want_dparams else None
+        # the op only ever reads rows [0,B) of grad, so a caller that holds just those rows passes them as is
+        grad_rows = 2 * B if (first_half_grad and grad.shape[0] == B) else grad.shape[0]
         _lib.check(lib.snntc_fc_backward(_ptr(grad), _ptr(X), _ptr(W), pp, _ptr(Y), _ptr(dX), _ptr(dW), _ptr(dP),
-                                         B, I, J, w_rows, grad.shape[0], _ptr(ws), ws.numel(), _stream(X.device)))
+                                         B, I, J, w_rows, grad_rows, _ptr(ws), ws.numel(), _stream(X.device)))
     return dX, dW, dP
 
 
@@ -148,7 +150,7 @@ def snncv(X, W, Params, return_aux=False):
     return out
 
 
-def snncv_grad(grad, X, W, Params, Y, want_dparams=True, want_dx=True, want_dw=True):
+def snncv_grad(grad, X, W, Params, Y, want_dparams=True, want_dx=True, want_dw=True, first_half_grad=False):
     """Conv backward -> (dXpad like X, dW like W, dParams[12] of zeros, or None if not wanted)."""
     lib = _lib.load()
     grad = _dev_f32(grad, "grad", 4)
@@ -169,8 +171,9 @@ def snncv_grad(grad, X, W, Params, Y, want_dparams=True, want_dx=True, want_dw=T
         dW = torch.empty_like(W) if want_dw else None
         dP = torch.empty(12, dtype=torch.float32, device=X.device) if want_dparams else None
         _lib.check(lib.snntc_cv_backward(_ptr(grad), _ptr(X), _ptr(W), pp, _ptr(Y), _ptr(dX), _ptr(dW), _ptr(dP),
-                                         B, H, Wd, C, Kc, w_rows, grad.shape[0], _ptr(ws), ws.numel(),
-                                         _stream(X.device)))
+                                         B, H, Wd, C, Kc, w_rows,
+                                         2 * B if (first_half_grad and grad.shape[0] == B) else grad.shape[0],
+                                         _ptr(ws), ws.numel(), _stream(X.device)))
     return dX, dW, dP
 
 
@@ -208,4 +211,44 @@ class SnnCv(torch.autograd.Function):
         X, W, Y = ctx.saved_tensors
         dX, dW, _ = snncv_grad(grad.contiguous(), X, W, ctx.params, Y, want_dparams=False,
                                want_dx=ctx.needs_input_grad[0], want_dw=ctx.needs_input_grad[1])
+        return dX, dW, None
+
+
+class SnnFcTimes(torch.autograd.Function):
+    """What SNN_dense.call returns (SNN_TC_Modules.py:73-75): the spike times Y[:B] of snnfc.  The full
+    [2B,J] output is kept for the backward op, which then takes the [B,J] upstream gradient directly --
+    slicing the output of SnnFc instead costs a zero fill and a copy of [2B,J] per backward pass."""
+
+    @staticmethod
+    def forward(ctx, X, W, Params):
+        Y = snnfc(X, W, Params)
+        ctx.save_for_backward(X, W, Y)
+        ctx.params = np.array(Params, dtype=np.float32, copy=True)
+        return Y[:X.shape[0]]
+
+    @staticmethod
+    def backward(ctx, grad):
+        X, W, Y = ctx.saved_tensors
+        dX, dW, _ = snnfc_grad(grad.contiguous(), X, W, ctx.params, Y, want_dparams=False,
+                               want_dx=ctx.needs_input_grad[0], want_dw=ctx.needs_input_grad[1],
+                               first_half_grad=True)
+        return dX, dW, None
+
+
+class SnnCvTimes(torch.autograd.Function):
+    """Spike times Y[:B] of snncv, as SNN_conv.call returns them (SNN_TC_Modules.py:168-170)."""
+
+    @staticmethod
+    def forward(ctx, X, W, Params):
+        Y = snncv(X, W, Params)
+        ctx.save_for_backward(X, W, Y)
+        ctx.params = np.array(Params, dtype=np.float32, copy=True)
+        return Y[:X.shape[0]]
+
+    @staticmethod
+    def backward(ctx, grad):
+        X, W, Y = ctx.saved_tensors
+        dX, dW, _ = snncv_grad(grad.contiguous(), X, W, ctx.params, Y, want_dparams=False,
+                               want_dx=ctx.needs_input_grad[0], want_dw=ctx.needs_input_grad[1],
+                               first_half_grad=True)
         return dX, dW, None

@@ -145,3 +145,36 @@ def test_conv_sort_with_heavy_ties(C, Kh, Kw, Sh, Sw):
     assert np.array_equal(sz.cpu().numpy(), ref_sorted)
     assert np.array_equal(ck.cpu().numpy(), ref_k)
     assert np.array_equal(out.cpu().numpy().view(np.uint32), ref_out.view(np.uint32))
+
+
+def test_layer_autograd_matches_op_level_chain():
+    """SNN_dense / SNN_conv hand the [B,...] upstream gradient to the backward op directly; the result
+    must equal slicing the full op output under autograd (zero-extended gradient), bit for bit."""
+    import snntc_amd as snn
+    x, w, p, g = dense_case(11, 24, 120, 50, True, "baseline")
+    B = x.shape[0]
+    layer = snn.SNN_dense(x.shape[1], w.shape[1], weight=w.copy()).to(DEV)
+    X1 = t(x).requires_grad_(True)
+    y1 = layer(X1)
+    (y1 * t(g[:B])).sum().backward()
+    X2 = t(x).requires_grad_(True)
+    W2 = t(w).requires_grad_(True)
+    y2 = snn.SnnFc.apply(X2, W2, layer.Params)[:B]
+    (y2 * t(g[:B])).sum().backward()
+    assert torch.equal(y1, y2)
+    assert torch.equal(X1.grad, X2.grad) and torch.equal(layer.weight.grad, W2.grad)
+
+    xraw, xpad, w, p, g = conv_case(12, 2, 9, 9, 32, 16, 3, 3, 1, 1, True, True, "baseline")
+    B = xraw.shape[0]
+    conv = snn.SNN_conv(32, 16, 3, 1, 'SAME', weight=w.copy()).to(DEV)
+    X1 = t(xraw).requires_grad_(True)
+    y1 = conv(X1)
+    (y1 * t(g[:B])).sum().backward()
+    X2 = t(xpad).requires_grad_(True)
+    W2 = t(w).requires_grad_(True)
+    y2 = snn.SnnCv.apply(X2, W2, conv.Params)[:B]
+    (y2 * t(g[:B])).sum().backward()
+    assert torch.equal(y1, y2)
+    assert torch.equal(conv.weight.grad, W2.grad)
+    # dX of the layer is the padded gradient cropped back to the unpadded image
+    assert torch.equal(X1.grad, X2.grad[:, 1:-1, 1:-1, :])
