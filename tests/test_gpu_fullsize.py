@@ -111,3 +111,54 @@ def test_conv_north_star_layer_full_batch():
     oabs = out.clone(); oabs[B:] = oabs[B:].abs()
     _, dw_mag, _ = snn.snncv_grad(G.abs(), X, W, p, oabs)               # = -sum |x - y| |up|
     assert torch.all((acc - dw.double()).abs() <= 1e-5 * acc.abs() + 1e-6 * dw_mag.abs().double().clamp(min=1.0))
+
+
+# Layers of BASELINE configs 4 (CIFAR-10 net, B=128) and 5 (ResNet-18-shaped net, B=32) at full size.
+LAYER_SHAPES = [
+    # name,                    B,   H,   W,   C,  Kc, K, S
+    ("cifar conv 3->32 @32",   128, 32,  32,  3,   32,  3, 1),
+    ("cifar conv 32->32 @32",  128, 32,  32,  32,  32,  3, 1),
+    ("cifar conv 32->64 @16",  128, 16,  16,  32,  64,  3, 1),
+    ("cifar conv 64->128 @8",  128, 8,   8,   64,  128, 3, 1),
+    ("resnet stem 7x7/2",      32,  224, 224, 3,   64,  7, 2),
+    ("resnet 64->64 @56",      32,  56,  56,  64,  64,  3, 1),
+    ("resnet 64->128 @28",     32,  28,  28,  64,  128, 3, 1),
+    ("resnet 128->128 @28",    32,  28,  28,  128, 128, 3, 1),
+    ("resnet 256->256 @14",    32,  14,  14,  256, 256, 3, 1),
+    ("resnet 512->512 @7",     32,  7,   7,   512, 512, 3, 1),
+]
+
+
+@pytest.mark.parametrize("name,B,H,W,C,Kc,K,S", LAYER_SHAPES, ids=[s[0] for s in LAYER_SHAPES])
+def test_conv_layer_shapes_of_the_baseline_networks(name, B, H, W, C, Kc, K, S):
+    import snntc_amd as snn
+    _, xpad, w, p, g = conv_case(20 + C + K, B, H, W, C, Kc, K, K, S, S, True, True, "baseline")
+    X, Wt, G = t(xpad), t(w), t(g)
+    out, sz, perm, ck = snn.snncv(X, Wt, p, return_aux=True)
+    Nh, Nw = out.shape[1], out.shape[2]
+    n_img = Nh * Nw
+    patches = X.unfold(1, K, S).unfold(2, K, S).permute(0, 1, 2, 4, 5, 3).reshape(B * n_img, K * K * C)
+    check_forward_properties(patches, Wt, out.reshape(2 * B * n_img, Kc), sz, perm, ck, True)
+    del patches
+    for b in (0, B - 1):                                   # images are independent: exact against the oracle
+        ref, rk, _, rperm = capi.cv_forward_dev(xpad[b:b + 1], w, p, want_aux=True)
+        got = torch.stack((out[b], out[B + b])).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+        assert np.array_equal(ck[b * n_img:(b + 1) * n_img].cpu().numpy(), rk)
+        assert np.array_equal(perm[b * n_img:(b + 1) * n_img].cpu().numpy(), rperm)
+    del sz, perm, ck
+    dx, dw, _ = snn.snncv_grad(G, X, Wt, p, out)
+    dx2, dw2, _ = snn.snncv_grad(2 * G, X, Wt, p, out)
+    assert torch.equal(dx2, 2 * dx) and torch.equal(dw2, 2 * dw)
+    assert torch.all(dx[X > 99999.0] == 0)
+    b = B - 1                                              # last image alone: same dX, oracle dX / dW
+    o1 = torch.stack((out[b], out[B + b])); g1 = torch.stack((G[b], G[B + b]))
+    dx1, dw1, _ = snn.snncv_grad(g1, X[b:b + 1], Wt, p, o1)
+    assert torch.equal(dx1[0], dx[b])
+    rdx, rdw, _ = capi.cv_backward_dev(g1.cpu().numpy(), xpad[b:b + 1], w, p, o1.cpu().numpy(), wide=True)
+    o1a = o1.clone(); o1a[1] = o1a[1].abs()
+    mdx, mdw, _ = snn.snncv_grad(g1.abs(), X[b:b + 1], Wt.abs(), p, o1a)      # sums of |summands|
+    tol_dx = 1e-5 * np.abs(rdx) + 1e-6 * np.maximum(1.0, np.abs(mdx.cpu().numpy()))
+    tol_dw = 1e-5 * np.abs(rdw) + 1e-6 * np.maximum(1.0, np.abs(mdw.cpu().numpy()))
+    assert np.all(np.abs(dx1.cpu().numpy() - rdx) <= tol_dx)
+    assert np.all(np.abs(dw1.cpu().numpy() - rdw) <= tol_dw)
