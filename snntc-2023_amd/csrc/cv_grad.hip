@@ -14,10 +14,12 @@ namespace {
 // ---------------------------------------------------------------------------------------------
 // dX.  A wavefront owns TILE consecutive pixels of one image row and 64 (or 32) channels; lane =
 // channel.  For every kernel tap (kh, kw) the lane keeps its weight row W[(kh,kw,c), 0..KCB) in
-// registers and sweeps the tile: the patch under the tap is the same for all lanes, so its ym /
-// upm rows are scalar operands.  Gather form: no atomics, fixed summation order.
+// registers and sweeps the tile: the patch under the tap is the same for all lanes.  The ym / upm
+// rows of the TILE + Kw - 1 patches one kernel row can touch are staged in a wavefront-private
+// piece of LDS (lane = output channel while staging) and read back as broadcasts, four output
+// channels per read.  Gather form: no atomics, fixed summation order.
 // ---------------------------------------------------------------------------------------------
-constexpr int DX_TILE = 4;
+constexpr int DX_TILE = 8;
 
 template <int KCB>
 __global__ void __launch_bounds__(256)
@@ -25,6 +27,7 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
                           const float* __restrict__ upm, const float* __restrict__ ym,
                           float* __restrict__ dxpad, int H, int W, int C, int Kc, int Kh, int Kw, int Sh, int Sw,
                           int Nh, int Nw, int tiles_w, int c_blocks, int64_t n_items, float max_cmp) {
+    extern __shared__ float staged[];                    // per wavefront: [2][TILE + Kw - 1][KCB]
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int64_t item = (int64_t)blockIdx.x * (blockDim.x / kWave) + wave;
     if (item >= n_items) return;
@@ -38,6 +41,9 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
     const int c = cb * kWave + lane;
     const bool lane_ok = c < C;
     const unsigned cc = (unsigned)(lane_ok ? c : C - 1);
+    const int n_slots = DX_TILE + Kw - 1;                // slot d holds the patch whose left column is w0-Kw+1+d
+    float* __restrict__ ys = staged + (size_t)wave * 2 * n_slots * KCB;
+    float* __restrict__ us = ys + n_slots * KCB;
 
     float xv[DX_TILE], acc[DX_TILE];
     bool any_real = false;
@@ -56,33 +62,43 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
             if (hh < 0 || hh % Sh != 0) continue;
             const int nh = hh / Sh;
             if (nh >= Nh) continue;
-            for (int kw = 0; kw < Kw; ++kw) {
-                const float* __restrict__ wrow = w + ((size_t)(kh * Kw + kw) * C + cc) * Kc;
-                for (int kc0 = 0; kc0 < Kc; kc0 += KCB) {
+            const size_t row0 = (size_t)(a * Nh + nh) * Nw;
+            for (int kc0 = 0; kc0 < Kc; kc0 += KCB) {
+                // stage the patch row: slots whose patch does not exist are never read
+                __builtin_amdgcn_wave_barrier();
+                for (int d = 0; d < n_slots; ++d) {
+                    const int ww = w0 - Kw + 1 + d;
+                    if (ww < 0 || ww % Sw != 0 || ww / Sw >= Nw) continue;
+                    if (lane < KCB) {
+                        const size_t so = (row0 + ww / Sw) * Kc + kc0 + lane;
+                        ys[d * KCB + lane] = ym[so];
+                        us[d * KCB + lane] = upm[so];
+                    }
+                }
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                for (int kw = 0; kw < Kw; ++kw) {
+                    const float* __restrict__ wrow = w + ((size_t)(kh * Kw + kw) * C + cc) * Kc + kc0;
                     float wreg[KCB];
 #pragma unroll
                     for (int q = 0; q < KCB; q += 4) {
-                        const float4 v4 = *reinterpret_cast<const float4*>(wrow + kc0 + q);
+                        const float4 v4 = *reinterpret_cast<const float4*>(wrow + q);
                         wreg[q] = v4.x; wreg[q + 1] = v4.y; wreg[q + 2] = v4.z; wreg[q + 3] = v4.w;
                     }
 #pragma unroll
                     for (int t = 0; t < DX_TILE; ++t) {
                         const int ww = w0 + t - kw;
-                        if (w0 + t >= W || ww < 0 || ww % Sw != 0) continue;
-                        const int nw = ww / Sw;
-                        if (nw >= Nw) continue;
-                        const size_t so = ((size_t)(a * Nh + nh) * Nw + nw) * Kc + kc0;
-                        const float* __restrict__ yrow = ym + so;
-                        const float* __restrict__ urow = upm + so;
-                        // 16 output channels at a time: 32 scalar operands live, not 2*KCB
+                        if (w0 + t >= W || ww < 0 || ww % Sw != 0 || ww / Sw >= Nw) continue;
+                        const float* __restrict__ yrow = ys + (t - kw + Kw - 1) * KCB;
+                        const float* __restrict__ urow = us + (t - kw + Kw - 1) * KCB;
 #pragma unroll
-                        for (int q0 = 0; q0 < KCB; q0 += 16) {
-#pragma unroll
-                            for (int q = q0; q < q0 + 16; ++q) {
-                                const float tq = xv[t] <= yrow[q] ? wreg[q] : 0.0f;
-                                acc[t] = __fmaf_rn(urow[q], tq, acc[t]);
-                            }
-                            __builtin_amdgcn_sched_barrier(0);
+                        for (int q = 0; q < KCB; q += 4) {
+                            const float4 y4 = *reinterpret_cast<const float4*>(yrow + q);
+                            const float4 u4 = *reinterpret_cast<const float4*>(urow + q);
+                            acc[t] = __fmaf_rn(u4.x, xv[t] <= y4.x ? wreg[q] : 0.0f, acc[t]);
+                            acc[t] = __fmaf_rn(u4.y, xv[t] <= y4.y ? wreg[q + 1] : 0.0f, acc[t]);
+                            acc[t] = __fmaf_rn(u4.z, xv[t] <= y4.z ? wreg[q + 2] : 0.0f, acc[t]);
+                            acc[t] = __fmaf_rn(u4.w, xv[t] <= y4.w ? wreg[q + 3] : 0.0f, acc[t]);
                         }
                     }
                 }
@@ -170,7 +186,8 @@ cv_grad_weight_wide_kernel(const float* __restrict__ xpad, const float* __restri
 }  // namespace
 
 bool cv_grad_input_chan_supported(const ConvGeom& g) {
-    return g.C >= 32 && g.Kc % 16 == 0;
+    // the staging buffer (four wavefronts, TILE + Kw - 1 patches) has to fit the default 64 KB of LDS
+    return g.C >= 32 && g.Kc % 16 == 0 && (DX_TILE + g.Kw - 1) * 64 * 8 * 4 <= 64 * 1024;
 }
 
 int launch_cv_grad_input_chan(const float* xpad, const float* w, const float* upm, const float* ym,
@@ -181,18 +198,20 @@ int launch_cv_grad_input_chan(const float* xpad, const float* w, const float* up
     const int64_t blocks = (n_items + 3) / 4;
     if (blocks > 0x7fffffffLL) return fail(SNNTC_ERR_TOO_LARGE, "conv backward: grid too large");
     dim3 grid((unsigned)blocks), block(256);
+    const int kcb = g.Kc % 64 == 0 ? 64 : (g.Kc % 32 == 0 ? 32 : 16);
+    const size_t lds = (size_t)4 * 2 * (DX_TILE + g.Kw - 1) * kcb * sizeof(float);
     {
         KernelTimerScope timer_("cv_grad_input", stream);
         if (g.Kc % 64 == 0)
-            hipLaunchKernelGGL(cv_grad_input_chan_kernel<64>, grid, block, 0, stream, xpad, w, upm, ym, dxpad,
+            hipLaunchKernelGGL(cv_grad_input_chan_kernel<64>, grid, block, lds, stream, xpad, w, upm, ym, dxpad,
                                (int)g.H, (int)g.W, (int)g.C, (int)g.Kc, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw,
                                (int)g.Nh, (int)g.Nw, tiles_w, c_blocks, n_items, np.max_cmp);
         else if (g.Kc % 32 == 0)
-            hipLaunchKernelGGL(cv_grad_input_chan_kernel<32>, grid, block, 0, stream, xpad, w, upm, ym, dxpad,
+            hipLaunchKernelGGL(cv_grad_input_chan_kernel<32>, grid, block, lds, stream, xpad, w, upm, ym, dxpad,
                                (int)g.H, (int)g.W, (int)g.C, (int)g.Kc, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw,
                                (int)g.Nh, (int)g.Nw, tiles_w, c_blocks, n_items, np.max_cmp);
         else
-            hipLaunchKernelGGL(cv_grad_input_chan_kernel<16>, grid, block, 0, stream, xpad, w, upm, ym, dxpad,
+            hipLaunchKernelGGL(cv_grad_input_chan_kernel<16>, grid, block, lds, stream, xpad, w, upm, ym, dxpad,
                                (int)g.H, (int)g.W, (int)g.C, (int)g.Kc, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw,
                                (int)g.Nh, (int)g.Nw, tiles_w, c_blocks, n_items, np.max_cmp);
     }
