@@ -334,25 +334,29 @@ def cpu_baseline(workload_key, seed=0):
         h = np.exp(1.0 - rng.random((B, sizes[0]))).astype(np.float32)
         ws = [_w_init(rng, sizes[i], sizes[i + 1]) for i in range(len(sizes) - 1)]
         p = capi.fc_params(1.0)
+        reps = 10 if workload_key == "mlp" else 20          # about 12 s of host work
+        x0 = h
         t0 = time.perf_counter()
-        acts, outs = [], []
-        for w in ws:
-            acts.append(h)
-            out = capi.fc_forward_host(h, w, p)
-            outs.append(out)
-            h = np.ascontiguousarray(out[:B])
-        g = np.zeros_like(outs[-1]); g[:B] = rng.standard_normal((B, sizes[-1]))
-        for w, a, out in zip(reversed(ws), reversed(acts), reversed(outs)):
-            dx, dw, _ = capi.fc_backward_host(g, a, w, p, out)
-            w -= np.float32(1e-4) * dw
-            g = np.zeros((2 * B, a.shape[1]), np.float32); g[:B] = dx
-        what = "the same dense layer stack"
+        for _ in range(reps):
+            h = x0
+            acts, outs = [], []
+            for w in ws:
+                acts.append(h)
+                out = capi.fc_forward_host(h, w, p)
+                outs.append(out)
+                h = np.ascontiguousarray(out[:B])
+            g = np.zeros_like(outs[-1]); g[:B] = rng.standard_normal((B, sizes[-1]))
+            for w, a, out in zip(reversed(ws), reversed(acts), reversed(outs)):
+                dx, dw, _ = capi.fc_backward_host(g, a, w, p, out)
+                w -= np.float32(1e-4) * dw
+                g = np.zeros((2 * B, a.shape[1]), np.float32); g[:B] = dx
+        what = f"the same dense layer stack, {reps} steps"
     else:
         if workload_key == "conv":
-            specs, dense, B = [(32, 64, 64)], (), 8
+            specs, dense, B = [(32, 64, 64)], (), 32
         else:  # cifar: conv layers (hw, C, Kc); pooling and loss are left out of the CPU sample
             specs = [(32, 3, 32), (32, 32, 32), (16, 32, 64), (16, 64, 64), (8, 64, 128)]
-            dense, B = ((2048, 512), (512, 10)), 4
+            dense, B = ((2048, 512), (512, 10)), 32
         for hw, C, Kc in specs:
             x = np.exp(rng.random((B, hw, hw, C))).astype(np.float32)
             xpad = np.pad(x, ((0, 0), (1, 1), (1, 1), (0, 0)), constant_values=np.float32(1e5))
@@ -371,7 +375,8 @@ def cpu_baseline(workload_key, seed=0):
             capi.fc_backward_host(g, xx, w, p, out)
         what = "the same conv/dense layers (pooling and loss left out)"
     dt = time.perf_counter() - t0
-    return {"value": B / dt, "unit": "samples/s", "cores": 1, "kind": "port",
+    n_samples = B * (reps if workload_key in ("mlp", "dense") else 1)
+    return {"value": n_samples / dt, "unit": "samples/s", "cores": 1, "kind": "port",
             "sample": f"B={B} through {what}, fwd+bwd, reference host functors restated in C (gcc -O3), 1 thread",
             "seconds": dt, "host_cpus": os.cpu_count()}
 
@@ -385,6 +390,9 @@ def main():
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="mlp")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time eager steps instead of HIP-graph replays")
+    ap.add_argument("--calibration-copies", type=int, default=0,
+                    help="first do this many plain 256 MiB device copies: a kernel of known traffic to scale "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings of the same run by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -397,6 +405,13 @@ def main():
         sys.exit("bench.py needs a ROCm GPU")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.calibration_copies > 0:
+        src = torch.empty(256 * 1024 * 1024 // 4, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(args.calibration_copies):
+            dst.copy_(src)                               # 256 MiB read + 256 MiB written per copy
+        torch.cuda.synchronize()
+        del src, dst
     wl = WORKLOADS[args.workload](torch, snn, dev)
 
     graph, graph_note = (None, "disabled by --no-graph") if args.no_graph else capture_step(torch, wl)
