@@ -151,6 +151,16 @@ SNNTC_API int snntc_cv_backward(const float* grad, const float* xpad, const floa
                       int64_t grad_rows, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Loss of the example networks, loss_func (SNN_TC_Modules.py:286-288): categorical cross-entropy of
+ * label[B,J] (one-hot, or any non-negative weights) against softmax(-times[B,J]).
+ *   sample_loss[B]  per-sample loss  -sum_j label_j * log softmax(-times)_j        (may be NULL)
+ *   dtimes[B,J]     gradient of the batch MEAN of sample_loss w.r.t. times         (may be NULL)
+ * The batch mean itself is left to the caller (mean of sample_loss).  No workspace.
+ * ------------------------------------------------------------------------------------------- */
+SNNTC_API int snntc_softmax_time_loss(const float* times, const float* label, float* sample_loss, float* dtimes,
+                            int64_t B, int64_t J, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * Per-kernel timing (no counterpart in the reference, which only times whole scripts with
  * time.time()).  While enabled, every kernel the library launches is bracketed by a pair of HIP
  * events on its launch stream; this is the only process-wide state the library keeps and it is

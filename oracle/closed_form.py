@@ -165,3 +165,16 @@ def fd_grads(g, x, w, params, h=1e-6, probes=64, seed=0):
         w[r, c] = w0 + h; lp = loss(); w[r, c] = w0 - h; lm = loss(); w[r, c] = w0
         out_w.append(((r, c), (lp - lm) / (2 * h)))
     return out_x, out_w
+
+
+def softmax_time_loss(times, label):
+    """float64 statement of loss_func (SNN_TC_Modules.py:286-288): per-sample cross-entropy of `label`
+    against softmax(-times), and the gradient of the batch mean with respect to `times`."""
+    t = np.asarray(times, np.float64); y = np.asarray(label, np.float64)
+    l = -t
+    l = l - l.max(axis=1, keepdims=True)
+    lse = np.log(np.exp(l).sum(axis=1, keepdims=True))
+    logp = l - lse
+    sample = -(y * logp).sum(axis=1)
+    grad = (y - np.exp(logp) * y.sum(axis=1, keepdims=True)) / t.shape[0]
+    return sample, grad

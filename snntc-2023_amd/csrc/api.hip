@@ -294,6 +294,16 @@ const char* snntc_status_string(int status) {
     }
 }
 
+int snntc_softmax_time_loss(const float* times, const float* label, float* sample_loss, float* dtimes, int64_t B,
+                            int64_t J, void* stream) {
+    if (B < 0 || J < 0) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_softmax_time_loss: negative size");
+    if (B > INT32_MAX || J > INT32_MAX || B * J > INT32_MAX)
+        return fail(SNNTC_ERR_TOO_LARGE, "snntc_softmax_time_loss: more than INT32_MAX elements");
+    if (B > 0 && J > 0 && (!times || !label || (!sample_loss && !dtimes)))
+        return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_softmax_time_loss: null pointer");
+    return launch_softmax_time_loss(times, label, sample_loss, dtimes, B, J, static_cast<hipStream_t>(stream));
+}
+
 int snntc_profile_enable(int on) {
     std::lock_guard<std::mutex> lock(g_prof_mutex);
     prof_drain();

@@ -116,5 +116,7 @@ int launch_cv_grad_input(const float* xpad, const float* wt, const float* upm, c
                          float* dxpad, const ConvGeom& g, int64_t wt_stride, hipStream_t stream);
 
 int launch_fill_zero(float* p, int64_t n, hipStream_t stream);
+int launch_softmax_time_loss(const float* times, const float* label, float* sample_loss, float* dtimes,
+                             int64_t B, int64_t J, hipStream_t stream);
 
 }  // namespace snntc

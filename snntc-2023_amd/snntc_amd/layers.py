@@ -12,7 +12,7 @@ import numpy as np
 import torch
 import torch.nn.functional as F
 
-from .ops import SnnCvTimes, SnnFcTimes
+from .ops import SnnCvTimes, SnnFcTimes, SoftmaxTimeLoss
 
 # Mirrors the reference's module-level switch (SNN_TC_Modules.py:11): when True the layers keep
 # the largest batch and element count they have seen in ``maxD`` (every tensor must stay below
@@ -204,5 +204,8 @@ class SNN_avgpool2d(_Pool2d):
 def loss_func(logit=None, label=None):
     """Mean categorical cross-entropy of one-hot ``label`` against softmax(-logit): the earliest
     output spike is the predicted class (SNN_TC_Modules.py:286-288)."""
-    logp = F.log_softmax(-logit, dim=-1)
+    if (logit.is_cuda and logit.dim() == 2 and logit.dtype == torch.float32 and label.dtype == torch.float32
+            and not label.requires_grad):
+        return SoftmaxTimeLoss.apply(logit, label)           # one fused kernel for loss and gradient
+    logp = F.log_softmax(-logit, dim=-1)                      # host tensors / other layouts: the formula itself
     return torch.mean(-torch.sum(label * logp, dim=-1))

@@ -252,3 +252,40 @@ class SnnCvTimes(torch.autograd.Function):
                                want_dx=ctx.needs_input_grad[0], want_dw=ctx.needs_input_grad[1],
                                first_half_grad=True)
         return dX, dW, None
+
+
+def softmax_time_loss(times, label, want_loss=True, want_grad=True):
+    """Per-sample cross-entropy of label[B,J] against softmax(-times[B,J]) and the gradient of its batch
+    mean with respect to times, in one kernel (loss_func, SNN_TC_Modules.py:286-288).
+    Returns (sample_loss[B] or None, dtimes[B,J] or None)."""
+    lib = _lib.load()
+    times = _dev_f32(times, "times", 2)
+    label = _dev_f32(label, "label", 2)
+    if tuple(times.shape) != tuple(label.shape):
+        raise ValueError(f"loss: times {tuple(times.shape)} and label {tuple(label.shape)} differ in shape")
+    B, J = times.shape
+    with torch.cuda.device(times.device):
+        loss = torch.empty(B, dtype=torch.float32, device=times.device) if want_loss else None
+        grad = torch.empty_like(times) if want_grad else None
+        _lib.check(lib.snntc_softmax_time_loss(_ptr(times), _ptr(label), _ptr(loss), _ptr(grad), B, J,
+                                               _stream(times.device)))
+    return loss, grad
+
+
+class SoftmaxTimeLoss(torch.autograd.Function):
+    """mean_b CE(label_b, softmax(-times_b)); the gradient is produced by the forward kernel."""
+
+    @staticmethod
+    def forward(ctx, times, label):
+        loss, grad = softmax_time_loss(times, label, want_grad=times.requires_grad)
+        if grad is not None:
+            ctx.save_for_backward(grad)
+        ctx.has_grad = grad is not None
+        return loss.mean()
+
+    @staticmethod
+    def backward(ctx, upstream):
+        if not ctx.has_grad:
+            return None, None
+        (grad,) = ctx.saved_tensors
+        return grad * upstream, None

@@ -128,3 +128,12 @@ def test_python_ops_map_status_to_exceptions():
     rc = lib.snntc_fc_forward(FAKE, FAKE, _fp(p0), FAKE, 4, 10, 5, 10, None, 0, None)
     with pytest.raises(_lib.SnntcError):
         _lib.check(rc)
+
+
+def test_loss_argument_errors(lib):
+    one = ctypes.c_void_p(256)                     # never dereferenced: the checks come first
+    assert lib.snntc_softmax_time_loss(one, one, one, one, -1, 4, None) == 3
+    assert lib.snntc_softmax_time_loss(None, one, one, one, 2, 4, None) == 3
+    assert lib.snntc_softmax_time_loss(one, one, None, None, 2, 4, None) == 3
+    assert lib.snntc_softmax_time_loss(one, one, one, one, 1 << 20, 1 << 20, None) == 2
+    assert lib.snntc_softmax_time_loss(one, one, one, one, 0, 4, None) == 0      # empty batch: nothing to do

@@ -178,3 +178,27 @@ def test_layer_autograd_matches_op_level_chain():
     assert torch.equal(conv.weight.grad, W2.grad)
     # dX of the layer is the padded gradient cropped back to the unpadded image
     assert torch.equal(X1.grad, X2.grad[:, 1:-1, 1:-1, :])
+
+
+@pytest.mark.parametrize("B,J", [(256, 10), (1, 1), (33, 1000), (7, 65)])
+def test_loss_kernel_against_closed_form(B, J):
+    """Fused loss kernel: per-sample loss and gradient within 1e-6 (relative to max(1, |value|)) of the
+    float64 closed form; unfired outputs (time = 1e5) take no probability and no gradient."""
+    import snntc_amd as snn
+    from oracle.closed_form import softmax_time_loss
+    rng = np.random.default_rng(B + J)
+    times = (1.0 + 4.0 * rng.random((B, J))).astype(np.float32)
+    if J > 2:
+        times[:, -1] = 1e5                                   # a neuron that never fired
+    label = np.eye(J, dtype=np.float32)[rng.integers(0, max(J - 1, 1), B)]
+    want_s, want_g = softmax_time_loss(times, label)
+    got_s, got_g = snn.softmax_time_loss(t(times), t(label))
+    assert np.all(np.abs(got_s.cpu().numpy() - want_s) <= 1e-6 * np.maximum(1.0, np.abs(want_s)))
+    assert np.all(np.abs(got_g.cpu().numpy() - want_g) <= 1e-6 / B + 1e-6 * np.abs(want_g))
+    if J > 2:
+        assert np.all(got_g.cpu().numpy()[:, -1] == 0.0)
+    # through loss_func and autograd: same mean and gradient, scaled by the upstream factor
+    T = t(times).requires_grad_(True)
+    (3.0 * snn.loss_func(T, t(label))).backward()
+    assert abs(float(snn.loss_func(T.detach(), t(label))) - want_s.mean()) <= 1e-6 * max(1.0, want_s.mean())
+    assert np.all(np.abs(T.grad.cpu().numpy() - 3.0 * want_g) <= 3e-6 / B + 3e-6 * np.abs(want_g))

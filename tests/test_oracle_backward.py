@@ -137,3 +137,24 @@ def test_golden_conv_gradients(name):
     xpad, w, p, g, out = (GOLDEN[f"{name}_{n}"] for n in ("xpad", "w", "params", "grad", "out"))
     dx, dw, _ = capi.cv_backward_dev(g, xpad, w, p, out, wide=True)
     assert np.array_equal(dx, GOLDEN[f"{name}_dx"]) and np.array_equal(dw, GOLDEN[f"{name}_dw"])
+
+
+def test_loss_closed_form_value_and_gradient():
+    """The float64 loss statement used to check the GPU loss kernel: a hand value, the uniform case,
+    and its gradient against central differences of its own value."""
+    from oracle.closed_form import softmax_time_loss
+    # two classes, times (1, 3), label on the early class: p = e^-1/(e^-1+e^-3) -> loss = log(1 + e^-2)
+    s, g = softmax_time_loss(np.array([[1.0, 3.0]]), np.array([[1.0, 0.0]]))
+    assert abs(s[0] - np.log1p(np.exp(-2.0))) < 1e-14
+    p = 1.0 / (1.0 + np.exp(-2.0))
+    assert np.allclose(g, [[1.0 - p, -(1.0 - p)]], atol=1e-14)        # earlier true class: push its time down
+    s, g = softmax_time_loss(np.full((3, 5), 2.5), np.eye(5)[[0, 2, 4]])
+    assert np.allclose(s, np.log(5.0)) and np.allclose(g.sum(axis=1), 0.0)
+    rng = np.random.default_rng(3)
+    t = 1.0 + 3.0 * rng.random((6, 9)); y = np.eye(9)[rng.integers(0, 9, 6)]
+    _, g = softmax_time_loss(t, y)
+    h = 1e-6
+    for (b, j) in [(0, 0), (2, 5), (5, 8), (3, 3)]:
+        tp, tm = t.copy(), t.copy(); tp[b, j] += h; tm[b, j] -= h
+        fd = (softmax_time_loss(tp, y)[0].mean() - softmax_time_loss(tm, y)[0].mean()) / (2 * h)
+        assert abs(fd - g[b, j]) < 1e-8
