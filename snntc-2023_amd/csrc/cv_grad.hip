@@ -21,6 +21,40 @@ namespace {
 // ---------------------------------------------------------------------------------------------
 constexpr int DX_TILE = 8;
 
+// Sixteen masked MACs  acc += upm_k * (x <= ym_k ? w_k : 0).  ym_k arrive as broadcast LDS reads; the
+// sixteen upm_k sit in ONE register (lane r of every row of 16 lanes holds upm of channel r) and
+// are fed to the FMA through its DPP row broadcast, which costs no instruction and no LDS
+// bandwidth -- with both operands read as broadcasts the kernel was bound by the LDS pipe.
+// Two temporaries alternate so that a DPP instruction never reads a register written by one of
+// the two instructions before it.
+#define SNNTC_DX_SEL(K, T)                                  \
+    "v_cmp_le_f32_e32 vcc, %[x], %[y" #K "]\n"              \
+    "v_cndmask_b32_e32 %[" #T "], 0, %[w" #K "], vcc\n"
+#define SNNTC_DX_FMA(K, T) \
+    "v_fmac_f32_dpp %[acc], %[u], %[" #T "] row_newbcast:" #K " row_mask:0xf bank_mask:0xf\n"
+
+__device__ __forceinline__ void dx_mac16(float& acc, float x, float u, const float (&y)[16], const float* w) {
+    float ta, tb;
+    asm volatile(
+        SNNTC_DX_SEL(0, ta) SNNTC_DX_SEL(1, tb) SNNTC_DX_FMA(0, ta)
+        SNNTC_DX_SEL(2, ta) SNNTC_DX_FMA(1, tb) SNNTC_DX_SEL(3, tb) SNNTC_DX_FMA(2, ta)
+        SNNTC_DX_SEL(4, ta) SNNTC_DX_FMA(3, tb) SNNTC_DX_SEL(5, tb) SNNTC_DX_FMA(4, ta)
+        SNNTC_DX_SEL(6, ta) SNNTC_DX_FMA(5, tb) SNNTC_DX_SEL(7, tb) SNNTC_DX_FMA(6, ta)
+        SNNTC_DX_SEL(8, ta) SNNTC_DX_FMA(7, tb) SNNTC_DX_SEL(9, tb) SNNTC_DX_FMA(8, ta)
+        SNNTC_DX_SEL(10, ta) SNNTC_DX_FMA(9, tb) SNNTC_DX_SEL(11, tb) SNNTC_DX_FMA(10, ta)
+        SNNTC_DX_SEL(12, ta) SNNTC_DX_FMA(11, tb) SNNTC_DX_SEL(13, tb) SNNTC_DX_FMA(12, ta)
+        SNNTC_DX_SEL(14, ta) SNNTC_DX_FMA(13, tb) SNNTC_DX_SEL(15, tb) SNNTC_DX_FMA(14, ta)
+        "s_nop 1\n" SNNTC_DX_FMA(15, tb)
+        : [acc] "+v"(acc), [ta] "=&v"(ta), [tb] "=&v"(tb)
+        : [x] "v"(x), [u] "v"(u), [y0] "v"(y[0]), [y1] "v"(y[1]), [y2] "v"(y[2]), [y3] "v"(y[3]), [y4] "v"(y[4]),
+          [y5] "v"(y[5]), [y6] "v"(y[6]), [y7] "v"(y[7]), [y8] "v"(y[8]), [y9] "v"(y[9]), [y10] "v"(y[10]),
+          [y11] "v"(y[11]), [y12] "v"(y[12]), [y13] "v"(y[13]), [y14] "v"(y[14]), [y15] "v"(y[15]),
+          [w0] "v"(w[0]), [w1] "v"(w[1]), [w2] "v"(w[2]), [w3] "v"(w[3]), [w4] "v"(w[4]), [w5] "v"(w[5]),
+          [w6] "v"(w[6]), [w7] "v"(w[7]), [w8] "v"(w[8]), [w9] "v"(w[9]), [w10] "v"(w[10]), [w11] "v"(w[11]),
+          [w12] "v"(w[12]), [w13] "v"(w[13]), [w14] "v"(w[14]), [w15] "v"(w[15])
+        : "vcc");
+}
+
 template <int KCB>
 __global__ void __launch_bounds__(256)
 cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restrict__ w,
@@ -91,14 +125,28 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
                         if (w0 + t >= W || ww < 0 || ww % Sw != 0 || ww / Sw >= Nw) continue;
                         const float* __restrict__ yrow = ys + (t - kw + Kw - 1) * KCB;
                         const float* __restrict__ urow = us + (t - kw + Kw - 1) * KCB;
+                        // groups of 16 output channels; the operands of the next group are read
+                        // while the current one computes
+                        float yq[2][16], u16[2];
 #pragma unroll
-                        for (int q = 0; q < KCB; q += 4) {
-                            const float4 y4 = *reinterpret_cast<const float4*>(yrow + q);
-                            const float4 u4 = *reinterpret_cast<const float4*>(urow + q);
-                            acc[t] = __fmaf_rn(u4.x, xv[t] <= y4.x ? wreg[q] : 0.0f, acc[t]);
-                            acc[t] = __fmaf_rn(u4.y, xv[t] <= y4.y ? wreg[q + 1] : 0.0f, acc[t]);
-                            acc[t] = __fmaf_rn(u4.z, xv[t] <= y4.z ? wreg[q + 2] : 0.0f, acc[t]);
-                            acc[t] = __fmaf_rn(u4.w, xv[t] <= y4.w ? wreg[q + 3] : 0.0f, acc[t]);
+                        for (int v = 0; v < 16; v += 4) {
+                            const float4 y4 = *reinterpret_cast<const float4*>(yrow + v);
+                            yq[0][v] = y4.x; yq[0][v + 1] = y4.y; yq[0][v + 2] = y4.z; yq[0][v + 3] = y4.w;
+                        }
+                        u16[0] = urow[lane & 15];             // lane r of every row of 16: upm of channel q+r
+#pragma unroll
+                        for (int g = 0; g < KCB / 16; ++g) {
+                            if (g + 1 < KCB / 16) {
+#pragma unroll
+                                for (int v = 0; v < 16; v += 4) {
+                                    const float4 y4 = *reinterpret_cast<const float4*>(yrow + (g + 1) * 16 + v);
+                                    yq[(g + 1) & 1][v] = y4.x; yq[(g + 1) & 1][v + 1] = y4.y;
+                                    yq[(g + 1) & 1][v + 2] = y4.z; yq[(g + 1) & 1][v + 3] = y4.w;
+                                }
+                                u16[(g + 1) & 1] = urow[(g + 1) * 16 + (lane & 15)];
+                            }
+                            __builtin_amdgcn_sched_barrier(0);
+                            dx_mac16(acc[t], xv[t], u16[g & 1], yq[g & 1], &wreg[g * 16]);
                         }
                     }
                 }
