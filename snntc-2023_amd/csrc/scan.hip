@@ -299,27 +299,12 @@ __device__ __forceinline__ void scan_chunk_vector(float& wsum, float& ysum, floa
                      : SNNTC_VSCAN_STATE : SNNTC_VSCAN_INPUTS : "vcc");
 }
 
-// LOW_LATENCY is the instantiation for launches with at most a couple of wavefronts per SIMD, where
-// nothing hides a stall: workgroups of at most four wavefronts (so that the work spreads over the
-// chip), seven chunks of (x, row) in flight instead of two, and the vector-only step block.
-constexpr int LOW_LATENCY_THREADS = 256;
-
-template <int COLS, bool WANT_K, bool LOW_LATENCY>
-__global__ void __launch_bounds__(LOW_LATENCY ? LOW_LATENCY_THREADS : LDS_SCAN_THREADS)
-scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
-                const int32_t* __restrict__ n_real, const float* __restrict__ w, float* __restrict__ y_out,
-                float* __restrict__ rcp_out, int32_t* __restrict__ k_out, int S, int I, int stride, int J,
-                int n_slices, int n_groups, NeuronParams np) {
-    extern __shared__ float wl[];                          // [I + bias][COLS]
-    constexpr int SEGS = kWave / COLS;                     // segments per wavefront
-    const int WAVES = blockDim.x / kWave;                  // 1..16, chosen by the launcher
-    const int slice = blockIdx.x % n_slices;
-    const int group = blockIdx.x / n_slices;
-    const int j0 = slice * COLS;
-    const int rows = I + np.bias;
-
-    // copy the column slice of W; loads are issued in batches so that a small workgroup does not
-    // pay one memory latency per element
+// Copies columns [j0, j0 + COLS) of all `rows` rows of W[rows, J] into LDS as wl[row][COLS] (zeros
+// past column J).  Loads are issued in batches so that a small workgroup does not pay one memory
+// latency per element.
+template <int COLS>
+__device__ __forceinline__ void fill_weight_slice(float* __restrict__ wl, const float* __restrict__ w, int rows,
+                                                  int J, int j0) {
     const int n_fill = rows * COLS;
     if ((J & 3) == 0) {
         constexpr int C4 = COLS / 4, FILL = 4;
@@ -355,6 +340,28 @@ scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ pe
             }
         }
     }
+}
+
+// LOW_LATENCY is the instantiation for launches with at most a couple of wavefronts per SIMD, where
+// nothing hides a stall: workgroups of at most four wavefronts (so that the work spreads over the
+// chip), seven chunks of (x, row) in flight instead of two, and the vector-only step block.
+constexpr int LOW_LATENCY_THREADS = 256;
+
+template <int COLS, bool WANT_K, bool LOW_LATENCY>
+__global__ void __launch_bounds__(LOW_LATENCY ? LOW_LATENCY_THREADS : LDS_SCAN_THREADS)
+scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
+                const int32_t* __restrict__ n_real, const float* __restrict__ w, float* __restrict__ y_out,
+                float* __restrict__ rcp_out, int32_t* __restrict__ k_out, int S, int I, int stride, int J,
+                int n_slices, int n_groups, NeuronParams np) {
+    extern __shared__ float wl[];                          // [I + bias][COLS]
+    constexpr int SEGS = kWave / COLS;                     // segments per wavefront
+    const int WAVES = blockDim.x / kWave;                  // 1..16, chosen by the launcher
+    const int slice = blockIdx.x % n_slices;
+    const int group = blockIdx.x / n_slices;
+    const int j0 = slice * COLS;
+    const int rows = I + np.bias;
+
+    fill_weight_slice<COLS>(wl, w, rows, J, j0);
     __syncthreads();
 
     const int lane = threadIdx.x % kWave;
@@ -458,6 +465,127 @@ scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ pe
     }
 }
 
+// Two neurons per lane.  Same workgroup layout as scan_lds_kernel, but a lane owns the adjacent
+// columns (2c, 2c+1) of its segment: one row address and one 8-byte LDS read serve two scans, a
+// wavefront covers 128/COLS segments, and the (x, row) chunks are fetched once for both.  Each of
+// the two scans keeps its own fired / closed masks and runs its own eight-step block under its own
+// EXEC.  This is the instantiation for launches with plenty of wavefronts per SIMD.
+template <int COLS, bool WANT_K>
+__global__ void __launch_bounds__(LDS_SCAN_THREADS)
+scan_lds_pair_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
+                     const int32_t* __restrict__ n_real, const float* __restrict__ w, float* __restrict__ y_out,
+                     float* __restrict__ rcp_out, int32_t* __restrict__ k_out, int S, int I, int stride, int J,
+                     int n_slices, int n_groups, NeuronParams np) {
+    extern __shared__ float wl[];                          // [I + bias][COLS]
+    constexpr int HALF = COLS / 2;                         // lanes per segment
+    constexpr int SEGS = kWave / HALF;                     // segments per wavefront
+    const int WAVES = blockDim.x / kWave;
+    const int slice = blockIdx.x % n_slices;
+    const int group = blockIdx.x / n_slices;
+    const int j0 = slice * COLS;
+    const int rows = I + np.bias;
+    fill_weight_slice<COLS>(wl, w, rows, J, j0);
+    __syncthreads();
+
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int sub = lane / HALF, cp = lane - sub * HALF;
+    const int j = j0 + 2 * cp;                             // first of the lane's two columns
+    const float2* __restrict__ wcol = reinterpret_cast<const float2*>(wl) + cp;
+    const int last_chunk = stride - CHUNK;
+
+    for (int item = group * WAVES + wave; item * SEGS < S; item += n_groups * WAVES) {
+        const int seg_raw = item * SEGS + sub;
+        const int seg = seg_raw < S ? seg_raw : S - 1;      // idle lanes shadow a valid segment
+        const bool live[2] = {seg_raw < S && j < J, seg_raw < S && j + 1 < J};
+        const float* __restrict__ xs = sorted + (size_t)seg * stride;
+        const int32_t* __restrict__ pr = perm + (size_t)seg * stride;
+        const int n_seg = n_real[seg];
+        const int n_full = n_seg & ~(CHUNK - 1);
+
+        float wsum[2], ysum[2], ya[2];
+        uint64_t fired[2], closed[2];
+        int kcnt[2] = {0, 0};
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            wsum[c] = -np.theta; ysum[c] = 0.0f; ya[c] = 0.0f;
+            bool fired0 = false;
+            if (np.bias) {
+                const float2 wb2 = wcol[I * HALF];
+                const float wb = c == 0 ? wb2.x : wb2.y;
+                wsum[c] += wb;
+                ysum[c] = np.biasvolt * wb;
+                ya[c] = wsum[c] < 0.0f ? -ysum[c] : ysum[c];
+                fired0 = ya[c] > fabsf(wsum[c]) * np.biasvolt;
+            }
+            fired[c] = __ballot(fired0);
+            closed[c] = ~__ballot(live[c]);                 // dead lanes never run
+        }
+
+        Chunk xp[3];
+        float wv[2][2][CHUNK];                              // [buffer][chain][step]
+        load_chunk_flat(xp[0], xs, pr, 0);
+        load_chunk_flat(xp[1], xs, pr, CHUNK <= last_chunk ? CHUNK : 0);
+#pragma unroll
+        for (int u = 0; u < CHUNK; ++u) {
+            const float2 w2 = wcol[xp[0].p[u] * HALF];
+            wv[0][0][u] = w2.x; wv[0][1][u] = w2.y;
+        }
+
+        for (int k0 = 0;; k0 += 6 * CHUNK) {
+            bool stop = false;
+#pragma unroll
+            for (int ph = 0; ph < 6; ++ph) {
+                const int k = k0 + ph * CHUNK;
+                const uint64_t in_range = __ballot(k < n_full);
+                const uint64_t run0 = in_range & ~closed[0], run1 = in_range & ~closed[1];
+                if ((run0 | run1) == 0) { stop = true; break; }
+                const int kn = k + 2 * CHUNK;
+                load_chunk_flat(xp[(ph + 2) % 3], xs, pr, kn <= last_chunk ? kn : 0);
+#pragma unroll
+                for (int u = 0; u < CHUNK; ++u) {
+                    const float2 w2 = wcol[xp[(ph + 1) % 3].p[u] * HALF];
+                    wv[(ph + 1) % 2][0][u] = w2.x; wv[(ph + 1) % 2][1][u] = w2.y;
+                }
+                if (run0 != 0)
+                    scan_chunk<WANT_K, false>(wsum[0], ysum[0], ya[0], kcnt[0], fired[0], closed[0], run0,
+                                              xp[ph % 3].x, wv[ph % 2][0]);
+                if (run1 != 0)
+                    scan_chunk<WANT_K, false>(wsum[1], ysum[1], ya[1], kcnt[1], fired[1], closed[1], run1,
+                                              xp[ph % 3].x, wv[ph % 2][1]);
+            }
+            if (stop) break;
+        }
+
+        // per-lane epilogue of each scan: up to CHUNK-1 trailing inputs, then the output
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            if (!live[c]) continue;
+            LaneState st;
+            st.wsum = wsum[c]; st.ysum = ysum[c]; st.wa = fabsf(wsum[c]); st.ya = ya[c];
+            const bool was_closed = (closed[c] >> lane) & 1;
+            st.fired = was_closed || ((fired[c] >> lane) & 1);
+            bool open = !was_closed;
+            int kc = kcnt[c];
+            for (int k = n_full; k < n_seg && open; ++k) {
+                const float2 w2 = wcol[pr[k] * HALF];
+                open = scan_step(st, xs[k], c == 0 ? w2.x : w2.y);
+                if (WANT_K && open) ++kc;
+            }
+            float y = np.max_time, r = 0.0f;
+            if (st.fired) {
+                r = 1.0f / st.wsum;
+                y = st.ysum * r;
+                if (y >= np.max_time) { y = np.max_time; r = 0.0f; }
+            }
+            const size_t o = (size_t)seg * J + j + c;
+            y_out[o] = y;
+            rcp_out[o] = r;
+            if (WANT_K) k_out[o] = (st.fired && r != 0.0f) ? kc : -1;
+        }
+    }
+}
+
 __global__ void __launch_bounds__(256)
 unpad_rows_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
                   float* __restrict__ sorted_out, int32_t* __restrict__ perm_out, int64_t n, int I, int stride) {
@@ -494,23 +622,32 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     int WAVES = (low_latency ? LOW_LATENCY_THREADS : LDS_SCAN_THREADS) / kWave;
     if (low_latency)
         while (WAVES > 1 && (int64_t)n_slices * ((items + WAVES - 1) / WAVES) < cus) WAVES >>= 1;
+    // With at least four wavefronts of two-neuron lanes for every SIMD, two neurons per lane (twice
+    // the segments per wavefront) is the cheaper instruction stream; in between, one neuron per
+    // lane in 16-wave workgroups balances better.
+    const int64_t pair_items = (S + 2 * SEGS - 1) / (2 * SEGS);
+    const bool pair = !low_latency && pair_items * n_slices >= (int64_t)cus * 4 * 4;
+    const int64_t work_items = pair ? pair_items : items;
     // resident workgroups per CU: split the segments so that slices x groups covers the chip
     const int wgs_per_cu = lds_bytes * 2 <= (size_t)LDS_SCAN_BYTES ? 2 : 1;
     int64_t n_groups = ((int64_t)cus * wgs_per_cu + n_slices - 1) / n_slices;
-    const int64_t max_groups = (items + WAVES - 1) / WAVES;
+    const int64_t max_groups = (work_items + WAVES - 1) / WAVES;
     if (n_groups > max_groups) n_groups = max_groups;
     if (n_groups < 1) n_groups = 1;
-    auto kern_k = low_latency ? scan_lds_kernel<COLS, true, true> : scan_lds_kernel<COLS, true, false>;
-    auto kern = low_latency ? scan_lds_kernel<COLS, false, true> : scan_lds_kernel<COLS, false, false>;
+    auto kern_k = low_latency ? scan_lds_kernel<COLS, true, true>
+                  : pair ? scan_lds_pair_kernel<COLS, true> : scan_lds_kernel<COLS, true, false>;
+    auto kern = low_latency ? scan_lds_kernel<COLS, false, true>
+                : pair ? scan_lds_pair_kernel<COLS, false> : scan_lds_kernel<COLS, false, false>;
     // raise the dynamic-LDS limit of both instantiations once (not per launch: the call is not
     // allowed while a stream is being captured into a graph)
-    static bool lds_limit_raised[2] = {false, false};
-    if (!lds_limit_raised[low_latency]) {
+    static bool lds_limit_raised[3] = {false, false, false};
+    const int variant = low_latency ? 1 : (pair ? 2 : 0);
+    if (!lds_limit_raised[variant]) {
         SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern_k),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, LDS_SCAN_BYTES));
         SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, LDS_SCAN_BYTES));
-        lds_limit_raised[low_latency] = true;
+        lds_limit_raised[variant] = true;
     }
     dim3 grid((unsigned)(n_slices * n_groups)), block((unsigned)(WAVES * kWave));
     {
