@@ -465,20 +465,33 @@ scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ pe
     }
 }
 
-// Two neurons per lane.  Same workgroup layout as scan_lds_kernel, but a lane owns the adjacent
-// columns (2c, 2c+1) of its segment: one row address and one 8-byte LDS read serve two scans, a
-// wavefront covers 128/COLS segments, and the (x, row) chunks are fetched once for both.  Each of
-// the two scans keeps its own fired / closed masks and runs its own eight-step block under its own
-// EXEC.  This is the instantiation for launches with plenty of wavefronts per SIMD.
-template <int COLS, bool WANT_K>
-__global__ void __launch_bounds__(LDS_SCAN_THREADS)
-scan_lds_pair_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
-                     const int32_t* __restrict__ n_real, const float* __restrict__ w, float* __restrict__ y_out,
-                     float* __restrict__ rcp_out, int32_t* __restrict__ k_out, int S, int I, int stride, int J,
-                     int n_slices, int n_groups, NeuronParams np) {
+// CH (2 or 4) neurons per lane.  Same workgroup layout as scan_lds_kernel, but a lane owns CH
+// adjacent columns of its segment: one row address and one 8- or 16-byte LDS read serve CH scans,
+// a wavefront covers 64*CH/COLS segments, and the (x, row) chunks are fetched once for all of
+// them.  Each scan keeps its own fired / closed masks and runs its own eight-step block under its
+// own EXEC.  This is the instantiation for launches with plenty of wavefronts per SIMD.
+template <int CH>
+__device__ __forceinline__ void read_columns(const float* p, float (&out)[CH]) {
+    if (CH == 2) {
+        const float2 v = *reinterpret_cast<const float2*>(p);
+        out[0] = v.x; out[1] = v.y;
+    } else {
+        const float4 v = *reinterpret_cast<const float4*>(p);
+        out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+    }
+}
+
+constexpr int MULTI_SCAN_THREADS = 512;
+
+template <int COLS, int CH, bool WANT_K>
+__global__ void __launch_bounds__(CH == 2 ? LDS_SCAN_THREADS : MULTI_SCAN_THREADS)
+scan_lds_multi_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
+                      const int32_t* __restrict__ n_real, const float* __restrict__ w, float* __restrict__ y_out,
+                      float* __restrict__ rcp_out, int32_t* __restrict__ k_out, int S, int I, int stride, int J,
+                      int n_slices, int n_groups, NeuronParams np) {
     extern __shared__ float wl[];                          // [I + bias][COLS]
-    constexpr int HALF = COLS / 2;                         // lanes per segment
-    constexpr int SEGS = kWave / HALF;                     // segments per wavefront
+    constexpr int LANES = COLS / CH;                       // lanes per segment
+    constexpr int SEGS = kWave / LANES;                    // segments per wavefront
     const int WAVES = blockDim.x / kWave;
     const int slice = blockIdx.x % n_slices;
     const int group = blockIdx.x / n_slices;
@@ -489,32 +502,33 @@ scan_lds_pair_kernel(const float* __restrict__ sorted, const int32_t* __restrict
 
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    const int sub = lane / HALF, cp = lane - sub * HALF;
-    const int j = j0 + 2 * cp;                             // first of the lane's two columns
-    const float2* __restrict__ wcol = reinterpret_cast<const float2*>(wl) + cp;
+    const int sub = lane / LANES, cg = lane - sub * LANES;
+    const int j = j0 + CH * cg;                            // first of the lane's columns
+    const float* __restrict__ wcol = wl + CH * cg;
     const int last_chunk = stride - CHUNK;
 
     for (int item = group * WAVES + wave; item * SEGS < S; item += n_groups * WAVES) {
         const int seg_raw = item * SEGS + sub;
         const int seg = seg_raw < S ? seg_raw : S - 1;      // idle lanes shadow a valid segment
-        const bool live[2] = {seg_raw < S && j < J, seg_raw < S && j + 1 < J};
         const float* __restrict__ xs = sorted + (size_t)seg * stride;
         const int32_t* __restrict__ pr = perm + (size_t)seg * stride;
         const int n_seg = n_real[seg];
         const int n_full = n_seg & ~(CHUNK - 1);
 
-        float wsum[2], ysum[2], ya[2];
-        uint64_t fired[2], closed[2];
-        int kcnt[2] = {0, 0};
+        float wsum[CH], ysum[CH], ya[CH];
+        uint64_t fired[CH], closed[CH];
+        int kcnt[CH];
+        bool live[CH];
+        float wb[CH];
+        if (np.bias) read_columns<CH>(wcol + I * COLS, wb);
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            wsum[c] = -np.theta; ysum[c] = 0.0f; ya[c] = 0.0f;
+        for (int c = 0; c < CH; ++c) {
+            live[c] = seg_raw < S && j + c < J;
+            wsum[c] = -np.theta; ysum[c] = 0.0f; ya[c] = 0.0f; kcnt[c] = 0;
             bool fired0 = false;
             if (np.bias) {
-                const float2 wb2 = wcol[I * HALF];
-                const float wb = c == 0 ? wb2.x : wb2.y;
-                wsum[c] += wb;
-                ysum[c] = np.biasvolt * wb;
+                wsum[c] += wb[c];
+                ysum[c] = np.biasvolt * wb[c];
                 ya[c] = wsum[c] < 0.0f ? -ysum[c] : ysum[c];
                 fired0 = ya[c] > fabsf(wsum[c]) * np.biasvolt;
             }
@@ -523,13 +537,15 @@ scan_lds_pair_kernel(const float* __restrict__ sorted, const int32_t* __restrict
         }
 
         Chunk xp[3];
-        float wv[2][2][CHUNK];                              // [buffer][chain][step]
+        float wv[2][CH][CHUNK];                             // [buffer][scan][step]
         load_chunk_flat(xp[0], xs, pr, 0);
         load_chunk_flat(xp[1], xs, pr, CHUNK <= last_chunk ? CHUNK : 0);
 #pragma unroll
         for (int u = 0; u < CHUNK; ++u) {
-            const float2 w2 = wcol[xp[0].p[u] * HALF];
-            wv[0][0][u] = w2.x; wv[0][1][u] = w2.y;
+            float wr[CH];
+            read_columns<CH>(wcol + xp[0].p[u] * COLS, wr);
+#pragma unroll
+            for (int c = 0; c < CH; ++c) wv[0][c][u] = wr[c];
         }
 
         for (int k0 = 0;; k0 += 6 * CHUNK) {
@@ -538,28 +554,31 @@ scan_lds_pair_kernel(const float* __restrict__ sorted, const int32_t* __restrict
             for (int ph = 0; ph < 6; ++ph) {
                 const int k = k0 + ph * CHUNK;
                 const uint64_t in_range = __ballot(k < n_full);
-                const uint64_t run0 = in_range & ~closed[0], run1 = in_range & ~closed[1];
-                if ((run0 | run1) == 0) { stop = true; break; }
+                uint64_t run[CH], any = 0;
+#pragma unroll
+                for (int c = 0; c < CH; ++c) { run[c] = in_range & ~closed[c]; any |= run[c]; }
+                if (any == 0) { stop = true; break; }
                 const int kn = k + 2 * CHUNK;
                 load_chunk_flat(xp[(ph + 2) % 3], xs, pr, kn <= last_chunk ? kn : 0);
 #pragma unroll
                 for (int u = 0; u < CHUNK; ++u) {
-                    const float2 w2 = wcol[xp[(ph + 1) % 3].p[u] * HALF];
-                    wv[(ph + 1) % 2][0][u] = w2.x; wv[(ph + 1) % 2][1][u] = w2.y;
+                    float wr[CH];
+                    read_columns<CH>(wcol + xp[(ph + 1) % 3].p[u] * COLS, wr);
+#pragma unroll
+                    for (int c = 0; c < CH; ++c) wv[(ph + 1) % 2][c][u] = wr[c];
                 }
-                if (run0 != 0)
-                    scan_chunk<WANT_K, false>(wsum[0], ysum[0], ya[0], kcnt[0], fired[0], closed[0], run0,
-                                              xp[ph % 3].x, wv[ph % 2][0]);
-                if (run1 != 0)
-                    scan_chunk<WANT_K, false>(wsum[1], ysum[1], ya[1], kcnt[1], fired[1], closed[1], run1,
-                                              xp[ph % 3].x, wv[ph % 2][1]);
+#pragma unroll
+                for (int c = 0; c < CH; ++c)
+                    if (run[c] != 0)
+                        scan_chunk<WANT_K, false>(wsum[c], ysum[c], ya[c], kcnt[c], fired[c], closed[c], run[c],
+                                                  xp[ph % 3].x, wv[ph % 2][c]);
             }
             if (stop) break;
         }
 
         // per-lane epilogue of each scan: up to CHUNK-1 trailing inputs, then the output
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
+        for (int c = 0; c < CH; ++c) {
             if (!live[c]) continue;
             LaneState st;
             st.wsum = wsum[c]; st.ysum = ysum[c]; st.wa = fabsf(wsum[c]); st.ya = ya[c];
@@ -568,8 +587,7 @@ scan_lds_pair_kernel(const float* __restrict__ sorted, const int32_t* __restrict
             bool open = !was_closed;
             int kc = kcnt[c];
             for (int k = n_full; k < n_seg && open; ++k) {
-                const float2 w2 = wcol[pr[k] * HALF];
-                open = scan_step(st, xs[k], c == 0 ? w2.x : w2.y);
+                open = scan_step(st, xs[k], wcol[pr[k] * COLS + c]);
                 if (WANT_K && open) ++kc;
             }
             float y = np.max_time, r = 0.0f;
@@ -622,12 +640,14 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     int WAVES = (low_latency ? LOW_LATENCY_THREADS : LDS_SCAN_THREADS) / kWave;
     if (low_latency)
         while (WAVES > 1 && (int64_t)n_slices * ((items + WAVES - 1) / WAVES) < cus) WAVES >>= 1;
-    // With at least four wavefronts of two-neuron lanes for every SIMD, two neurons per lane (twice
+    // With at least four wavefronts of multi-neuron lanes for every SIMD, CH neurons per lane (CH times
     // the segments per wavefront) is the cheaper instruction stream; in between, one neuron per
     // lane in 16-wave workgroups balances better.
-    const int64_t pair_items = (S + 2 * SEGS - 1) / (2 * SEGS);
-    const bool pair = !low_latency && pair_items * n_slices >= (int64_t)cus * 4 * 4;
-    const int64_t work_items = pair ? pair_items : items;
+    constexpr int CH = 2;          // four per lane need 151 registers: too few wavefronts per SIMD, measured slower
+    const int64_t multi_items = (S + CH * SEGS - 1) / (CH * SEGS);
+    const bool pair = !low_latency && multi_items * n_slices >= (int64_t)cus * 4 * 4;
+    const int64_t work_items = pair ? multi_items : items;
+    if (pair && CH == 4) WAVES = MULTI_SCAN_THREADS / kWave;
     // resident workgroups per CU: split the segments so that slices x groups covers the chip
     const int wgs_per_cu = lds_bytes * 2 <= (size_t)LDS_SCAN_BYTES ? 2 : 1;
     int64_t n_groups = ((int64_t)cus * wgs_per_cu + n_slices - 1) / n_slices;
@@ -635,9 +655,9 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     if (n_groups > max_groups) n_groups = max_groups;
     if (n_groups < 1) n_groups = 1;
     auto kern_k = low_latency ? scan_lds_kernel<COLS, true, true>
-                  : pair ? scan_lds_pair_kernel<COLS, true> : scan_lds_kernel<COLS, true, false>;
+                  : pair ? scan_lds_multi_kernel<COLS, CH, true> : scan_lds_kernel<COLS, true, false>;
     auto kern = low_latency ? scan_lds_kernel<COLS, false, true>
-                : pair ? scan_lds_pair_kernel<COLS, false> : scan_lds_kernel<COLS, false, false>;
+                : pair ? scan_lds_multi_kernel<COLS, CH, false> : scan_lds_kernel<COLS, false, false>;
     // raise the dynamic-LDS limit of both instantiations once (not per launch: the call is not
     // allowed while a stream is being captured into a graph)
     static bool lds_limit_raised[3] = {false, false, false};
