@@ -133,7 +133,7 @@ scan_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
 // ---------------------------------------------------------------------------------------------
 constexpr int LDS_SCAN_THREADS = 1024;
 constexpr int LDS_SCAN_BYTES = 160 * 1024;
-constexpr int LDS_SCAN_TARGET = 80 * 1024;   // two workgroups per CU when a slice this small exists
+constexpr int LDS_SCAN_TARGET = 160 * 1024;  // widest slice that fits: the register budget allows one 16-wave workgroup per CU anyway, and fewer slices re-read the sorted rows less often
 
 struct Chunk {
     float x[CHUNK];
