@@ -55,36 +55,47 @@ __device__ __forceinline__ void dx_mac16(float& acc, float x, float u, const flo
         : "vcc");
 }
 
-template <int KCB>
-__global__ void __launch_bounds__(256)
+// HALVES = 2 is for layers with at most 32 input channels: the two halves of a wavefront take the
+// same channels of two neighbouring 8-pixel tiles, so no lane idles.  Which patch lies under a tap
+// then differs between the halves; a half whose patch does not exist reads a spare slot that holds
+// (ym, upm) = (-inf, 0) and so adds nothing.
+template <int KCB, int HALVES>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KCB == 64 && HALVES == 2 ? 3 : 4)))
 cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restrict__ w,
                           const float* __restrict__ upm, const float* __restrict__ ym,
                           float* __restrict__ dxpad, int H, int W, int C, int Kc, int Kh, int Kw, int Sh, int Sw,
                           int Nh, int Nw, int tiles_w, int c_blocks, int64_t n_items, float max_cmp) {
-    extern __shared__ float staged[];                    // per wavefront: [2][TILE + Kw - 1][KCB]
+    extern __shared__ float staged[];                    // per wavefront: [2][n_slots + 1][KCB]
+    constexpr int SPAN = DX_TILE * HALVES;               // pixels of one wavefront
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int64_t item = (int64_t)blockIdx.x * (blockDim.x / kWave) + wave;
     if (item >= n_items) return;
     const int lane = threadIdx.x % kWave;
+    const int half = HALVES == 2 ? lane / 32 : 0;
     const int cb = (int)(item % c_blocks);
     int64_t rest = item / c_blocks;
     const int tw = (int)(rest % tiles_w); rest /= tiles_w;
     const int h = (int)(rest % H);
     const int a = (int)(rest / H);
-    const int w0 = tw * DX_TILE;
-    const int c = cb * kWave + lane;
+    const int w0 = tw * SPAN;                            // first pixel of the wavefront
+    const int p0 = w0 + half * DX_TILE;                  // first pixel of this lane
+    const int c = HALVES == 2 ? (lane & 31) : cb * kWave + lane;
     const bool lane_ok = c < C;
     const unsigned cc = (unsigned)(lane_ok ? c : C - 1);
-    const int n_slots = DX_TILE + Kw - 1;                // slot d holds the patch whose left column is w0-Kw+1+d
-    float* __restrict__ ys = staged + (size_t)wave * 2 * n_slots * KCB;
-    float* __restrict__ us = ys + n_slots * KCB;
+    const int n_slots = SPAN + Kw - 1;                   // slot d: the patch whose left column is w0-Kw+1+d
+    float* __restrict__ ys = staged + (size_t)wave * 2 * (n_slots + 1) * KCB;
+    float* __restrict__ us = ys + (n_slots + 1) * KCB;
+    if (lane < KCB) {                                    // the spare slot
+        ys[n_slots * KCB + lane] = -INFINITY;
+        us[n_slots * KCB + lane] = 0.0f;
+    }
 
     float xv[DX_TILE], acc[DX_TILE];
     bool any_real = false;
     const float* __restrict__ xrow = xpad + ((size_t)(a * H + h) * W) * C + cc;
 #pragma unroll
     for (int t = 0; t < DX_TILE; ++t) {
-        const int wx = min(w0 + t, W - 1);
+        const int wx = min(p0 + t, W - 1);
         xv[t] = xrow[(size_t)wx * C];
         acc[t] = 0.0f;
         any_real |= xv[t] <= max_cmp;
@@ -121,10 +132,13 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
                     }
 #pragma unroll
                     for (int t = 0; t < DX_TILE; ++t) {
-                        const int ww = w0 + t - kw;
-                        if (w0 + t >= W || ww < 0 || ww % Sw != 0 || ww / Sw >= Nw) continue;
-                        const float* __restrict__ yrow = ys + (t - kw + Kw - 1) * KCB;
-                        const float* __restrict__ urow = us + (t - kw + Kw - 1) * KCB;
+                        const int ww = p0 + t - kw;
+                        const bool has_patch = p0 + t < W && ww >= 0 && ww % Sw == 0 && ww / Sw < Nw;
+                        if (!__any(has_patch)) continue;
+                        int slot = has_patch ? p0 + t - w0 - kw + Kw - 1 : n_slots;
+                        if (HALVES == 1) slot = __builtin_amdgcn_readfirstlane(slot);   // same for every lane
+                        const float* __restrict__ yrow = ys + slot * KCB;
+                        const float* __restrict__ urow = us + slot * KCB;
                         // groups of 16 output channels; the operands of the next group are read
                         // while the current one computes
                         float yq[2][16], u16[2];
@@ -157,7 +171,7 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
         float* __restrict__ orow = dxpad + ((size_t)(a * H + h) * W) * C + c;
 #pragma unroll
         for (int t = 0; t < DX_TILE; ++t)
-            if (w0 + t < W) orow[(size_t)(w0 + t) * C] = acc[t];
+            if (p0 + t < W) orow[(size_t)(p0 + t) * C] = acc[t];
     }
 }
 
@@ -234,34 +248,35 @@ cv_grad_weight_wide_kernel(const float* __restrict__ xpad, const float* __restri
 }  // namespace
 
 bool cv_grad_input_chan_supported(const ConvGeom& g) {
-    // the staging buffer (four wavefronts, TILE + Kw - 1 patches) has to fit the default 64 KB of LDS
-    return g.C >= 32 && g.Kc % 16 == 0 && (DX_TILE + g.Kw - 1) * 64 * 8 * 4 <= 64 * 1024;
+    // the staging buffer (four wavefronts, up to 2 * TILE + Kw patches) has to fit the default 64 KB of LDS
+    return g.C >= 32 && g.Kc % 16 == 0 && (2 * DX_TILE + g.Kw) * 64 * 8 * 4 <= 64 * 1024;
 }
 
 int launch_cv_grad_input_chan(const float* xpad, const float* w, const float* upm, const float* ym,
                               float* dxpad, const ConvGeom& g, const NeuronParams& np, hipStream_t stream) {
-    const int tiles_w = (int)((g.W + DX_TILE - 1) / DX_TILE);
-    const int c_blocks = (int)((g.C + kWave - 1) / kWave);
+    const int halves = g.C <= 32 ? 2 : 1;
+    const int span = DX_TILE * halves;
+    const int tiles_w = (int)((g.W + span - 1) / span);
+    const int c_blocks = halves == 2 ? 1 : (int)((g.C + kWave - 1) / kWave);
     const int64_t n_items = g.B * g.H * tiles_w * c_blocks;
     const int64_t blocks = (n_items + 3) / 4;
     if (blocks > 0x7fffffffLL) return fail(SNNTC_ERR_TOO_LARGE, "conv backward: grid too large");
     dim3 grid((unsigned)blocks), block(256);
     const int kcb = g.Kc % 64 == 0 ? 64 : (g.Kc % 32 == 0 ? 32 : 16);
-    const size_t lds = (size_t)4 * 2 * (DX_TILE + g.Kw - 1) * kcb * sizeof(float);
+    const size_t lds = (size_t)4 * 2 * (span + g.Kw) * kcb * sizeof(float);
+    void (*kern)(const float*, const float*, const float*, const float*, float*, int, int, int, int, int, int, int,
+                 int, int, int, int, int, int64_t, float);
+    if (halves == 2)
+        kern = kcb == 64 ? cv_grad_input_chan_kernel<64, 2> : kcb == 32 ? cv_grad_input_chan_kernel<32, 2>
+                                                                         : cv_grad_input_chan_kernel<16, 2>;
+    else
+        kern = kcb == 64 ? cv_grad_input_chan_kernel<64, 1> : kcb == 32 ? cv_grad_input_chan_kernel<32, 1>
+                                                                         : cv_grad_input_chan_kernel<16, 1>;
     {
         KernelTimerScope timer_("cv_grad_input", stream);
-        if (g.Kc % 64 == 0)
-            hipLaunchKernelGGL(cv_grad_input_chan_kernel<64>, grid, block, lds, stream, xpad, w, upm, ym, dxpad,
-                               (int)g.H, (int)g.W, (int)g.C, (int)g.Kc, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw,
-                               (int)g.Nh, (int)g.Nw, tiles_w, c_blocks, n_items, np.max_cmp);
-        else if (g.Kc % 32 == 0)
-            hipLaunchKernelGGL(cv_grad_input_chan_kernel<32>, grid, block, lds, stream, xpad, w, upm, ym, dxpad,
-                               (int)g.H, (int)g.W, (int)g.C, (int)g.Kc, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw,
-                               (int)g.Nh, (int)g.Nw, tiles_w, c_blocks, n_items, np.max_cmp);
-        else
-            hipLaunchKernelGGL(cv_grad_input_chan_kernel<16>, grid, block, lds, stream, xpad, w, upm, ym, dxpad,
-                               (int)g.H, (int)g.W, (int)g.C, (int)g.Kc, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw,
-                               (int)g.Nh, (int)g.Nw, tiles_w, c_blocks, n_items, np.max_cmp);
+        hipLaunchKernelGGL(kern, grid, block, lds, stream, xpad, w, upm, ym, dxpad, (int)g.H, (int)g.W, (int)g.C,
+                           (int)g.Kc, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.Nh, (int)g.Nw, tiles_w,
+                           c_blocks, n_items, np.max_cmp);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
