@@ -245,6 +245,103 @@ cv_grad_weight_wide_kernel(const float* __restrict__ xpad, const float* __restri
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// dW for layers with at most 32 output channels.  Lane = (half, kc): the two halves of a wavefront
+// take alternate patches, so no lane idles.  The 32 inputs of a patch that a block's rows need sit
+// in two registers (lane r of every row of 16 lanes holds inputs r and 16 + r of the half's own
+// patch) and reach the subtraction through its DPP row broadcast: still three instructions per
+// MAC, with a different patch in each half.  Partial sums of the halves and of the four
+// wavefronts are added in a fixed order through LDS.
+// ---------------------------------------------------------------------------------------------
+#define SNNTC_DW_ROW(R, A)                                                                       \
+    "v_sub_f32_dpp %[d], %[x], %[y] row_newbcast:" #R " row_mask:0xf bank_mask:0xf\n"             \
+    "v_min_f32_e32 %[d], 0, %[d]\n"                                                              \
+    "v_fmac_f32_e32 %[" #A "], %[d], %[u]\n"
+
+__device__ __forceinline__ void dw_rows16(float (&acc)[DWW_RI], int base, float x, float y, float u) {
+    float d;
+    float* a = acc + base;
+    asm volatile(
+        SNNTC_DW_ROW(0, a0) SNNTC_DW_ROW(1, a1) SNNTC_DW_ROW(2, a2) SNNTC_DW_ROW(3, a3)
+        SNNTC_DW_ROW(4, a4) SNNTC_DW_ROW(5, a5) SNNTC_DW_ROW(6, a6) SNNTC_DW_ROW(7, a7)
+        SNNTC_DW_ROW(8, a8) SNNTC_DW_ROW(9, a9) SNNTC_DW_ROW(10, a10) SNNTC_DW_ROW(11, a11)
+        SNNTC_DW_ROW(12, a12) SNNTC_DW_ROW(13, a13) SNNTC_DW_ROW(14, a14) SNNTC_DW_ROW(15, a15)
+        : [d] "=&v"(d), [a0] "+v"(a[0]), [a1] "+v"(a[1]), [a2] "+v"(a[2]), [a3] "+v"(a[3]), [a4] "+v"(a[4]),
+          [a5] "+v"(a[5]), [a6] "+v"(a[6]), [a7] "+v"(a[7]), [a8] "+v"(a[8]), [a9] "+v"(a[9]), [a10] "+v"(a[10]),
+          [a11] "+v"(a[11]), [a12] "+v"(a[12]), [a13] "+v"(a[13]), [a14] "+v"(a[14]), [a15] "+v"(a[15])
+        : [x] "v"(x), [y] "v"(y), [u] "v"(u));
+}
+
+__global__ void __launch_bounds__(256)
+cv_grad_weight_narrow_kernel(const float* __restrict__ xpad, const float* __restrict__ upm,
+                             const float* __restrict__ ym, float* __restrict__ dst, int S, int Kc, int rows,
+                             int seg_per_slice, int H, int W, int C, int Kw, int Sh, int Sw, int Nh, int Nw,
+                             int bias_row, float biasvolt) {
+    __shared__ float red[4][DWW_RI + 1][kWave];
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int half = lane >> 5, kc = lane & 31;
+    const unsigned jc = (unsigned)min(kc, Kc - 1);
+    const int i0 = blockIdx.y * DWW_RI;
+    const int tap = i0 / C, c0 = i0 - tap * C;
+    const int kh = tap / Kw, kw = tap - kh * Kw;
+
+    const int s_begin = blockIdx.z * seg_per_slice;
+    const int s_end = min(S, s_begin + seg_per_slice);
+    const int per_wave = (s_end - s_begin + 3) / 4;
+    const int s_lo = s_begin + wave * per_wave;
+    const int s_hi = min(s_end, s_lo + per_wave);
+
+    float acc[DWW_RI];
+#pragma unroll
+    for (int r = 0; r < DWW_RI; ++r) acc[r] = 0.0f;
+    const bool with_bias = bias_row >= 0 && blockIdx.y == 0;
+    float acc_bias = 0.0f;
+
+    if (s_lo < s_hi) {
+        const int per_img = Nh * Nw;
+        // this lane's patch: s_lo + half, then every second one; (a, nh, nw) follow it incrementally
+        int s = s_lo + half;
+        int sc = min(s, s_hi - 1);
+        int a = sc / per_img;
+        int r2 = sc - a * per_img;
+        int nh = r2 / Nw, nw = r2 - nh * Nw;
+        const int n_iter = (s_hi - s_lo + 1) / 2;
+        for (int it = 0; it < n_iter; ++it) {
+            const bool have = s < s_hi;
+            const float* __restrict__ xb =
+                xpad + ((size_t)(a * H + nh * Sh + kh) * W + (size_t)(nw * Sw + kw)) * C + c0 + (lane & 15);
+            const float x0 = xb[0], x1 = xb[16];
+            const float yv = ym[(size_t)sc * Kc + jc];
+            const float uv = have ? upm[(size_t)sc * Kc + jc] : 0.0f;
+            dw_rows16(acc, 0, x0, yv, uv);
+            dw_rows16(acc, 16, x1, yv, uv);
+            if (with_bias) acc_bias = __fmaf_rn(fminf(biasvolt - yv, 0.0f), uv, acc_bias);
+            s += 2;
+            if (s < s_hi) {                               // a lane past its last patch keeps pointing at it
+                sc = s;
+                nw += 2;
+                while (nw >= Nw) { nw -= Nw; if (++nh == Nh) { nh = 0; ++a; } }
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < DWW_RI; ++r) red[wave][r][lane] = acc[r];
+    red[wave][DWW_RI][lane] = acc_bias;
+    __syncthreads();
+    if (wave == 0 && half == 0 && kc < Kc) {
+        float* out = dst + (size_t)blockIdx.z * rows * Kc;
+#pragma unroll 4
+        for (int r = 0; r <= DWW_RI; ++r) {
+            if (r == DWW_RI && !with_bias) break;
+            float sum = 0.0f;
+#pragma unroll
+            for (int wv = 0; wv < 4; ++wv) sum = (sum + red[wv][r][kc]) + red[wv][r][kc + 32];
+            out[(size_t)(r == DWW_RI ? bias_row : i0 + r) * Kc + kc] = sum;
+        }
+    }
+}
+
 }  // namespace
 
 bool cv_grad_input_chan_supported(const ConvGeom& g) {
@@ -296,9 +393,10 @@ int launch_cv_grad_weight_wide(const float* xpad, const float* upm, const float*
     if (grid.y > 65535u) return fail(SNNTC_ERR_TOO_LARGE, "weight gradient: too many weight rows");
     {
         KernelTimerScope timer_("grad_weight", stream);
-        hipLaunchKernelGGL(cv_grad_weight_wide_kernel, grid, dim3(256), 0, stream, xpad, upm, ym, dst, (int)g.S,
-                           (int)g.Kc, (int)rows, seg_per_slice, (int)g.H, (int)g.W, (int)g.C, (int)g.Kw, (int)g.Sh,
-                           (int)g.Sw, (int)g.Nh, (int)g.Nw, np.bias ? (int)g.P : -1, np.biasvolt);
+        hipLaunchKernelGGL(g.Kc <= 32 ? cv_grad_weight_narrow_kernel : cv_grad_weight_wide_kernel, grid, dim3(256), 0,
+                           stream, xpad, upm, ym, dst, (int)g.S, (int)g.Kc, (int)rows, seg_per_slice, (int)g.H,
+                           (int)g.W, (int)g.C, (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.Nh, (int)g.Nw,
+                           np.bias ? (int)g.P : -1, np.biasvolt);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
