@@ -202,3 +202,82 @@ def test_loss_kernel_against_closed_form(B, J):
     (3.0 * snn.loss_func(T, t(label))).backward()
     assert abs(float(snn.loss_func(T.detach(), t(label))) - want_s.mean()) <= 1e-6 * max(1.0, want_s.mean())
     assert np.all(np.abs(T.grad.cpu().numpy() - 3.0 * want_g) <= 3e-6 / B + 3e-6 * np.abs(want_g))
+
+
+PARAM_SWEEP = [
+    # biasvolt, theta, max_time
+    (0.7, 1.0, 1e5),
+    (2.5, 0.5, 1e5),
+    (1.0, 2.0, 50.0),        # small MAX: inputs above MAX-0.1 are treated as never-fired
+    (0.0, 1.5, 20.0),
+]
+
+
+def _compare_forward_backward(fwd_ref, bwd_ref, fwd_gpu, bwd_gpu, g, B):
+    ref_out, ref_k, ref_sorted, ref_perm = fwd_ref()
+    out, sz, perm, ck = (v.cpu().numpy() for v in fwd_gpu())
+    assert np.array_equal(sz, ref_sorted) and np.array_equal(perm, ref_perm)
+    assert np.array_equal(ck, ref_k), f"causal-set sizes differ at {np.argwhere(ck != ref_k)[:5]}"
+    assert np.array_equal(out.view(np.uint32), ref_out.view(np.uint32)), "y / 1/S not bit-exact"
+    dx, dw, _ = (v.cpu().numpy() for v in bwd_gpu(ref_out))
+    rdx, rdw, adx, adw = bwd_ref(ref_out)
+    check_grad(dx, rdx, adx, "dX")
+    check_grad(dw, rdw, adw, "dW")
+
+
+@pytest.mark.parametrize("biasvolt,theta,max_time", PARAM_SWEEP)
+def test_dense_non_default_parameters_and_sentinel_inputs(biasvolt, theta, max_time):
+    """biasvolt, threshold and MAX other than the defaults; some inputs are the MAX sentinel (an upstream
+    neuron that never fired), one row consists of sentinels only, one weight column is all negative."""
+    import snntc_amd as snn
+    rng = np.random.default_rng(int(10 * biasvolt + 100 * theta))
+    B, I, J = 37, 150, 45
+    rows = I + (1 if biasvolt > 1e-8 else 0)
+    x = np.exp(1.0 - rng.random((B, I))).astype(np.float32)
+    x[rng.random((B, I)) < 0.15] = np.float32(max_time)
+    x[5, :] = np.float32(max_time)
+    x[6, : I // 2] = np.float32(max_time - 0.05)            # above MAX - 0.1: still "never fired"
+    w = (4.0 / I + np.sqrt(1.0 / I) * rng.standard_normal((rows, J))).astype(np.float32) * np.float32(theta)
+    w[:, 3] = -np.abs(w[:, 3])
+    p = capi.fc_params(biasvolt, max_time=max_time, theta=theta)
+    g = np.zeros((2 * B, J), np.float32); g[:B] = rng.standard_normal((B, J))
+
+    def bwd_ref(out):
+        rdx, rdw, _ = capi.fc_backward_dev(g, x, w, p, out, wide=True)
+        ao = out.copy(); ao[B:] = np.abs(ao[B:])
+        adx, adw, _ = capi.fc_backward_dev(np.abs(g), x, np.abs(w), p, ao, wide=True)
+        return rdx, rdw, adx, adw
+
+    _compare_forward_backward(lambda: capi.fc_forward_dev(x, w, p, want_aux=True), bwd_ref,
+                              lambda: snn.snnfc(t(x), t(w), p, return_aux=True),
+                              lambda out: snn.snnfc_grad(t(g), t(x), t(w), p, t(out)), g, B)
+
+
+@pytest.mark.parametrize("biasvolt,theta,max_time", PARAM_SWEEP)
+@pytest.mark.parametrize("C,Kc", [(32, 32), (64, 16), (5, 9)])
+def test_conv_non_default_parameters_and_sentinel_inputs(biasvolt, theta, max_time, C, Kc):
+    import snntc_amd as snn
+    from oracle.closed_form import same_pad
+    rng = np.random.default_rng(int(10 * biasvolt + 100 * theta) + C)
+    B, H, W, K = 2, 11, 10, 3
+    P = K * K * C
+    rows = P + (1 if biasvolt > 1e-8 else 0)
+    x = np.exp(rng.random((B, H, W, C))).astype(np.float32)
+    x[rng.random((B, H, W, C)) < 0.1] = np.float32(max_time)          # unfired upstream neurons
+    x[0, 4:7, 3:6, :] = np.float32(max_time)                          # a whole patch of them
+    (tp, bt), (lf, rt) = same_pad(H, K, 1), same_pad(W, K, 1)
+    xpad = np.pad(x, ((0, 0), (tp, bt), (lf, rt), (0, 0)), constant_values=np.float32(max_time))
+    w = (4.0 / P + np.sqrt(1.0 / P) * rng.standard_normal((rows, Kc))).astype(np.float32) * np.float32(theta)
+    p = capi.cv_params(K, K, 1, 1, same=True, biasvolt=biasvolt, max_time=max_time, theta=theta)
+    Nh, Nw, _ = capi.cv_dims(xpad.shape, p)
+    g = np.zeros((2 * B, Nh, Nw, Kc), np.float32); g[:B] = rng.standard_normal((B, Nh, Nw, Kc))
+
+    def bwd_ref(out):
+        rdx, rdw, _ = capi.cv_backward_dev(g, xpad, w, p, out, wide=True)
+        ao = out.copy(); ao[B:] = np.abs(ao[B:])
+        adx, adw, _ = capi.cv_backward_dev(np.abs(g), xpad, np.abs(w), p, ao, wide=True)
+        return rdx, rdw, adx, adw
+
+    _compare_forward_backward(lambda: capi.cv_forward_dev(xpad, w, p, want_aux=True), bwd_ref,
+                              lambda: snn.snncv(t(xpad), t(w), p, return_aux=True),
+                              lambda out: snn.snncv_grad(t(g), t(xpad), t(w), p, t(out)), g, B)

@@ -256,3 +256,26 @@ def test_same_padding_rule():
                 if total >= 0:
                     assert before == total // 2 and after == total - total // 2
                     assert (n + total - k) // s + 1 == -(-n // s)          # output size ceil(n/s)
+
+
+@pytest.mark.parametrize("biasvolt,theta,max_time", [(0.7, 1.0, 1e5), (2.5, 0.5, 1e5), (1.0, 2.0, 50.0), (0.0, 1.5, 20.0)])
+def test_fc_forward_dev_non_default_parameters_match_closed_form(biasvolt, theta, max_time):
+    """biasvolt, threshold and MAX away from their defaults, with MAX sentinels among the inputs: the
+    oracle against the float64 closed form (first valid prefix of the sorted inputs)."""
+    rng = np.random.default_rng(int(10 * biasvolt + 100 * theta))
+    B, I, J = 9, 80, 17
+    rows = I + (1 if biasvolt > 1e-8 else 0)
+    x = np.exp(1.0 - rng.random((B, I))).astype(np.float32)
+    x[rng.random((B, I)) < 0.15] = np.float32(max_time)
+    x[2, :] = np.float32(max_time)
+    w = ((4.0 / I + np.sqrt(1.0 / I) * rng.standard_normal((rows, J))) * theta).astype(np.float32)
+    p = capi.fc_params(biasvolt, max_time=max_time, theta=theta)
+    out, k, _, _ = capi.fc_forward_dev(x, w, p, want_aux=True)
+    y, kc, S = cf.fc_forward_closed_form(x, w, p)
+    assert np.array_equal(k, kc)
+    fired = kc >= 0
+    assert fired.any() and (~fired).any()
+    cond = np.maximum(1.0, 1.0 / np.abs(S[fired]))
+    assert np.all(np.abs(out[:B][fired] - y[fired]) <= 2e-5 * np.abs(y[fired]) * cond)
+    assert np.all(out[:B][~fired] == np.float32(max_time)) and np.all(out[B:][~fired] == 0)
+    assert np.all(out[:B][2] == np.float32(max_time)) or biasvolt > 1e-8     # a row of sentinels: only the bias can fire
