@@ -281,3 +281,26 @@ def test_conv_non_default_parameters_and_sentinel_inputs(biasvolt, theta, max_ti
     _compare_forward_backward(lambda: capi.cv_forward_dev(xpad, w, p, want_aux=True), bwd_ref,
                               lambda: snn.snncv(t(xpad), t(w), p, return_aux=True),
                               lambda out: snn.snncv_grad(t(g), t(xpad), t(w), p, t(out)), g, B)
+
+
+def test_empty_batch_and_single_elements():
+    """B = 0 yields empty outputs and an all-zero weight gradient; 1x1x1 shapes work."""
+    import snntc_amd as snn
+    p = capi.fc_params(1.0)
+    w = np.ones((6, 4), np.float32)
+    y = snn.snnfc(torch.empty((0, 5), device=DEV), t(w), p)
+    assert tuple(y.shape) == (0, 4)
+    dx, dw, dp = snn.snnfc_grad(torch.empty((0, 4), device=DEV), torch.empty((0, 5), device=DEV), t(w), p, y)
+    assert tuple(dx.shape) == (0, 5) and torch.all(dw == 0) and torch.all(dp == 0)
+    pc = capi.cv_params(3, 3, 1, 1, same=True, biasvolt=1.0)
+    wc = np.ones((9 * 2 + 1, 3), np.float32)
+    yc = snn.snncv(torch.empty((0, 6, 6, 2), device=DEV), t(wc), pc)
+    assert tuple(yc.shape) == (0, 4, 4, 3)
+    dxc, dwc, _ = snn.snncv_grad(torch.empty((0, 4, 4, 3), device=DEV), torch.empty((0, 6, 6, 2), device=DEV), t(wc), pc, yc)
+    assert tuple(dxc.shape) == (0, 6, 6, 2) and torch.all(dwc == 0)
+    # one sample, one input, one output, no bias: y = w z / (w - 1) for w > 1
+    x1 = np.array([[2.0]], np.float32); w1 = np.array([[3.0]], np.float32)
+    y1 = snn.snnfc(t(x1), t(w1), capi.fc_params(0.0)).cpu().numpy()
+    assert y1[0, 0] == np.float32(3.0) and y1[1, 0] == np.float32(0.5)
+    ref = capi.fc_forward_dev(x1, w1, capi.fc_params(0.0))
+    assert np.array_equal(y1, ref[0] if isinstance(ref, tuple) else ref)
