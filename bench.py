@@ -31,10 +31,13 @@ for _p in (ROOT, os.path.join(ROOT, "snntc-2023_amd")):
         sys.path.insert(0, _p)
 
 # HBM bytes per launch of the scan kernel, measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (two runs,
-# KiB per dispatch, FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0 as a plain 256 MiB device copy reads
-# on those counters); summary in profiles/scan_hbm_traffic_pmc.txt.  Counters cannot be read from inside
-# this script, so the figures are carried here per workload.
-MEASURED_SCAN_TRAFFIC_BYTES = {"mlp": 24.0e6, "conv": 653.1e6}
+# KiB per dispatch, FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0 as the plain 256 MiB device copies of
+# --calibration-copies read on those counters); summary in profiles/scan_hbm_traffic_pmc.txt.  Counters cannot
+# be read from inside this script, so the figures are carried here per workload (mlp: mean of its three launches).
+MEASURED_SCAN_TRAFFIC_BYTES = {"mlp": 24.1e6, "conv": 341.1e6}
+# Share of the scan kernel's clocks in which the vector ALUs issue (SQ_ACTIVE_INST_VALU * 4 / SIMDs / clocks,
+# profiles/valu_utilisation_pmc.txt); the counter ratio saturates slightly above 1.
+MEASURED_SCAN_VALU_BUSY = {"mlp": 0.62, "conv": 1.0}
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 VALU_PEAK_TFLOPS = 157.3     # MI355X fp32 vector peak (256 CU x 256 flop/clk x 2.4 GHz)
@@ -456,6 +459,7 @@ def main():
     roof = roofline_for(dominant, flops, nbytes, k["avg_us"] * 1e-3, k["launches_per_step"])
     if dominant == "scan":
         roof["traffic"] = MEASURED_SCAN_TRAFFIC_BYTES.get(args.workload)
+        roof["valu_busy"] = MEASURED_SCAN_VALU_BUSY.get(args.workload)
     roof.update({"kernel": dominant, "avg_launch_us": k["avg_us"], "launches_per_step": k["launches_per_step"],
                  "algorithmic_flops_per_step": flops, "algorithmic_bytes_per_step": nbytes})
     for name, kk in kernels.items():
