@@ -634,12 +634,11 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     const int n_slices = (int)((J + COLS - 1) / COLS);
     const int64_t items = (S + SEGS - 1) / SEGS;
     // A launch that cannot put more than two wavefronts on every SIMD runs the low-latency
-    // instantiation, in workgroups small enough (4, 2 or 1 wavefronts) to reach every CU: the same
-    // work packed into a few full workgroups would leave most of the chip idle.
+    // instantiation, in workgroups of four wavefronts (one per SIMD of a CU, and four times the
+    // threads of a single wavefront for copying the weight slice): the same work packed into a
+    // few full workgroups would leave most of the chip idle.
     const bool low_latency = items * n_slices <= (int64_t)cus * 4 * 2;
     int WAVES = (low_latency ? LOW_LATENCY_THREADS : LDS_SCAN_THREADS) / kWave;
-    if (low_latency)
-        while (WAVES > 1 && (int64_t)n_slices * ((items + WAVES - 1) / WAVES) < cus) WAVES >>= 1;
     // With at least four wavefronts of multi-neuron lanes for every SIMD, CH neurons per lane (CH times
     // the segments per wavefront) is the cheaper instruction stream; in between, one neuron per
     // lane in 16-wave workgroups balances better.
