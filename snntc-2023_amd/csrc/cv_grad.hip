@@ -176,26 +176,31 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
 }
 
 // ---------------------------------------------------------------------------------------------
-// dW.  Lane = output channel kc; a block owns DWW_RI consecutive weight rows that share one tap
-// (kh, kw), i.e. DWW_RI consecutive input channels, so the x values of a patch are one contiguous
-// scalar fetch.  The patch range is cut into gridDim.z slices (partial sums are added in slice
-// order afterwards) and each slice over the four wavefronts of the block.
+// dW.  Lane = output channel kc.  The weight rows of one kernel row kh, (kw, c) flattened, are
+// Kw*C consecutive floats of the padded image for every patch; a block owns up to DWW_RI
+// consecutive ones, so the x values of a patch are one contiguous scalar fetch.  The patch range is cut into gridDim.z slices (partial sums are added in
+// slice order afterwards) and each slice over the four wavefronts of the block.
 // ---------------------------------------------------------------------------------------------
 constexpr int DWW_RI = 32;
 
+// FULL: every block has all DWW_RI rows (Kw*C is a multiple of it); the partial-block code is left out.
+template <bool FULL>
 __global__ void __launch_bounds__(256)
 cv_grad_weight_wide_kernel(const float* __restrict__ xpad, const float* __restrict__ upm,
                            const float* __restrict__ ym, float* __restrict__ dst, int S, int Kc, int rows,
                            int seg_per_slice, int H, int W, int C, int Kw, int Sh, int Sw, int Nh, int Nw,
-                           int bias_row, float biasvolt) {
+                           int bias_row, float biasvolt, int s_safe) {
     __shared__ float red[3][DWW_RI + 1][kWave];
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int j = blockIdx.x * kWave + lane;
     const unsigned jc = (unsigned)min(j, Kc - 1);
-    const int i0 = blockIdx.y * DWW_RI;                 // first weight row of the block
-    const int tap = i0 / C, c0 = i0 - tap * C;          // tap = kh*Kw + kw
-    const int kh = tap / Kw, kw = tap - kh * Kw;
+    const int KwC = Kw * C;
+    const int chunks = (KwC + DWW_RI - 1) / DWW_RI;     // blocks per kernel row
+    const int kh = blockIdx.y / chunks;
+    const int q0 = (blockIdx.y - kh * chunks) * DWW_RI; // first (kw, c) of the block
+    const int n_rows = min(DWW_RI, KwC - q0);
+    const int i0 = kh * KwC + q0;                       // first weight row of the block
 
     const int s_begin = blockIdx.z * seg_per_slice;
     const int s_end = min(S, s_begin + seg_per_slice);
@@ -217,15 +222,44 @@ cv_grad_weight_wide_kernel(const float* __restrict__ xpad, const float* __restri
         int nh = r2 / Nw, nw = r2 - nh * Nw;
         const float* __restrict__ ycol = ym + jc;
         const float* __restrict__ ucol = upm + jc;
-        for (int s = s_lo; s < s_hi; ++s) {
-            const float* __restrict__ xb =
-                xpad + ((size_t)(a * H + nh * Sh + kh) * W + (size_t)(nw * Sw + kw)) * C + c0;
-            const float yv = ycol[(size_t)s * Kc];
-            const float uv = ucol[(size_t)s * Kc];
+        if (FULL || n_rows == DWW_RI) {
+            for (int s = s_lo; s < s_hi; ++s) {
+                const float* __restrict__ xb =
+                    xpad + ((size_t)(a * H + nh * Sh + kh) * W + (size_t)(nw * Sw)) * C + q0;
+                const float yv = ycol[(size_t)s * Kc];
+                const float uv = ucol[(size_t)s * Kc];
 #pragma unroll
-            for (int r = 0; r < DWW_RI; ++r) acc[r] = __fmaf_rn(fminf(xb[r] - yv, 0.0f), uv, acc[r]);
-            if (with_bias) acc_bias = __fmaf_rn(fminf(biasvolt - yv, 0.0f), uv, acc_bias);
-            if (++nw == Nw) { nw = 0; if (++nh == Nh) { nh = 0; ++a; } }
+                for (int r = 0; r < DWW_RI; ++r) acc[r] = __fmaf_rn(fminf(xb[r] - yv, 0.0f), uv, acc[r]);
+                if (with_bias) acc_bias = __fmaf_rn(fminf(biasvolt - yv, 0.0f), uv, acc_bias);
+                if (++nw == Nw) { nw = 0; if (++nh == Nh) { nh = 0; ++a; } }
+            }
+        } else {
+            // a block at the end of a kernel row fetches past its rows (the values are discarded) ...
+            int s = s_lo;
+            const int s_fast = min(s_hi, s_safe);
+            for (; s < s_fast; ++s) {
+                const float* __restrict__ xb =
+                    xpad + ((size_t)(a * H + nh * Sh + kh) * W + (size_t)(nw * Sw)) * C + q0;
+                const float yv = ycol[(size_t)s * Kc];
+                const float uv = ucol[(size_t)s * Kc];
+#pragma unroll
+                for (int r = 0; r < DWW_RI; ++r) acc[r] = __fmaf_rn(fminf(xb[r] - yv, 0.0f), uv, acc[r]);
+                if (with_bias) acc_bias = __fmaf_rn(fminf(biasvolt - yv, 0.0f), uv, acc_bias);
+                if (++nw == Nw) { nw = 0; if (++nh == Nh) { nh = 0; ++a; } }
+            }
+            // ... except for the last few patches of the tensor, where that fetch could leave it: there
+            // the unused rows re-read the block's last row
+            for (; s < s_hi; ++s) {
+                const float* __restrict__ xb =
+                    xpad + ((size_t)(a * H + nh * Sh + kh) * W + (size_t)(nw * Sw)) * C + q0;
+                const float yv = ycol[(size_t)s * Kc];
+                const float uv = ucol[(size_t)s * Kc];
+#pragma unroll
+                for (int r = 0; r < DWW_RI; ++r)
+                    acc[r] = __fmaf_rn(fminf(xb[min(r, n_rows - 1)] - yv, 0.0f), uv, acc[r]);
+                if (with_bias) acc_bias = __fmaf_rn(fminf(biasvolt - yv, 0.0f), uv, acc_bias);
+                if (++nw == Nw) { nw = 0; if (++nh == Nh) { nh = 0; ++a; } }
+            }
         }
     }
     if (wave > 0) {
@@ -238,7 +272,8 @@ cv_grad_weight_wide_kernel(const float* __restrict__ xpad, const float* __restri
         float* out = dst + (size_t)blockIdx.z * rows * Kc;
 #pragma unroll
         for (int r = 0; r < DWW_RI; ++r)
-            out[(size_t)(i0 + r) * Kc + j] = ((acc[r] + red[0][r][lane]) + red[1][r][lane]) + red[2][r][lane];
+            if (r < n_rows)
+                out[(size_t)(i0 + r) * Kc + j] = ((acc[r] + red[0][r][lane]) + red[1][r][lane]) + red[2][r][lane];
         if (with_bias)
             out[(size_t)bias_row * Kc + j] =
                 ((acc_bias + red[0][DWW_RI][lane]) + red[1][DWW_RI][lane]) + red[2][DWW_RI][lane];
@@ -276,15 +311,18 @@ __global__ void __launch_bounds__(256)
 cv_grad_weight_narrow_kernel(const float* __restrict__ xpad, const float* __restrict__ upm,
                              const float* __restrict__ ym, float* __restrict__ dst, int S, int Kc, int rows,
                              int seg_per_slice, int H, int W, int C, int Kw, int Sh, int Sw, int Nh, int Nw,
-                             int bias_row, float biasvolt) {
+                             int bias_row, float biasvolt, int /*s_safe*/) {
     __shared__ float red[4][DWW_RI + 1][kWave];
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int half = lane >> 5, kc = lane & 31;
     const unsigned jc = (unsigned)min(kc, Kc - 1);
-    const int i0 = blockIdx.y * DWW_RI;
-    const int tap = i0 / C, c0 = i0 - tap * C;
-    const int kh = tap / Kw, kw = tap - kh * Kw;
+    const int KwC = Kw * C;
+    const int chunks = (KwC + DWW_RI - 1) / DWW_RI;
+    const int kh = blockIdx.y / chunks;
+    const int q0 = (blockIdx.y - kh * chunks) * DWW_RI;
+    const int n_rows = min(DWW_RI, KwC - q0);
+    const int i0 = kh * KwC + q0;
 
     const int s_begin = blockIdx.z * seg_per_slice;
     const int s_end = min(S, s_begin + seg_per_slice);
@@ -309,9 +347,9 @@ cv_grad_weight_narrow_kernel(const float* __restrict__ xpad, const float* __rest
         const int n_iter = (s_hi - s_lo + 1) / 2;
         for (int it = 0; it < n_iter; ++it) {
             const bool have = s < s_hi;
-            const float* __restrict__ xb =
-                xpad + ((size_t)(a * H + nh * Sh + kh) * W + (size_t)(nw * Sw + kw)) * C + c0 + (lane & 15);
-            const float x0 = xb[0], x1 = xb[16];
+            const size_t xo = ((size_t)(a * H + nh * Sh + kh) * W + (size_t)(nw * Sw)) * C + q0;
+            const int l16 = lane & 15;                   // rows past the block's last one re-read it
+            const float x0 = xpad[xo + min(l16, n_rows - 1)], x1 = xpad[xo + min(l16 + 16, n_rows - 1)];
             const float yv = ym[(size_t)sc * Kc + jc];
             const float uv = have ? upm[(size_t)sc * Kc + jc] : 0.0f;
             dw_rows16(acc, 0, x0, yv, uv);
@@ -333,7 +371,7 @@ cv_grad_weight_narrow_kernel(const float* __restrict__ xpad, const float* __rest
         float* out = dst + (size_t)blockIdx.z * rows * Kc;
 #pragma unroll 4
         for (int r = 0; r <= DWW_RI; ++r) {
-            if (r == DWW_RI && !with_bias) break;
+            if (r == DWW_RI ? !with_bias : r >= n_rows) continue;
             float sum = 0.0f;
 #pragma unroll
             for (int wv = 0; wv < 4; ++wv) sum = (sum + red[wv][r][kc]) + red[wv][r][kc + 32];
@@ -379,24 +417,42 @@ int launch_cv_grad_input_chan(const float* xpad, const float* w, const float* up
     return SNNTC_OK;
 }
 
-bool cv_grad_weight_wide_supported(const ConvGeom& g) { return g.C % DWW_RI == 0; }
+// Any channel count; with very short kernel rows (Kw*C < 9) a block would mostly carry unused rows.
+bool cv_grad_weight_wide_supported(const ConvGeom& g) { return g.Kw * g.C >= 9; }
+
+static int64_t cv_grad_weight_row_blocks(const ConvGeom& g) {
+    return g.Kh * ((g.Kw * g.C + DWW_RI - 1) / DWW_RI);
+}
 
 int cv_grad_weight_wide_blocks(const ConvGeom& g) {
-    return (int)(((g.Kc + kWave - 1) / kWave) * (g.P / DWW_RI));
+    return (int)(((g.Kc + kWave - 1) / kWave) * cv_grad_weight_row_blocks(g));
 }
 
 // All rows of dW, bias row included (or of every partial-sum slice when nsplit > 1).
 int launch_cv_grad_weight_wide(const float* xpad, const float* upm, const float* ym, float* dst, int nsplit,
                                const ConvGeom& g, int64_t rows, const NeuronParams& np, hipStream_t stream) {
     const int seg_per_slice = (int)((g.S + nsplit - 1) / nsplit);
-    dim3 grid((unsigned)((g.Kc + kWave - 1) / kWave), (unsigned)(g.P / DWW_RI), (unsigned)nsplit);
+    dim3 grid((unsigned)((g.Kc + kWave - 1) / kWave), (unsigned)cv_grad_weight_row_blocks(g), (unsigned)nsplit);
     if (grid.y > 65535u) return fail(SNNTC_ERR_TOO_LARGE, "weight gradient: too many weight rows");
+    // patches before s_safe can fetch DWW_RI floats from any of their kernel-row starts without leaving
+    // the image tensor (only the last few patches of the last image cannot)
+    const int64_t n_x = g.B * g.H * g.W * g.C;
+    int64_t s_safe = g.S;
+    while (s_safe > 0) {
+        const int64_t sp = s_safe - 1, per_img = g.Nh * g.Nw;
+        const int64_t a = sp / per_img, nh = (sp % per_img) / g.Nw, nw = sp % g.Nw;
+        const int64_t last_start = ((a * g.H + nh * g.Sh + g.Kh - 1) * g.W + nw * g.Sw) * g.C + g.Kw * g.C - 1;
+        if (last_start + DWW_RI <= n_x) break;
+        --s_safe;
+    }
     {
         KernelTimerScope timer_("grad_weight", stream);
-        hipLaunchKernelGGL(g.Kc <= 32 ? cv_grad_weight_narrow_kernel : cv_grad_weight_wide_kernel, grid, dim3(256), 0,
+        const bool full = (g.Kw * g.C) % DWW_RI == 0;
+        hipLaunchKernelGGL(g.Kc <= 32 ? cv_grad_weight_narrow_kernel
+                           : full ? cv_grad_weight_wide_kernel<true> : cv_grad_weight_wide_kernel<false>, grid, dim3(256), 0,
                            stream, xpad, upm, ym, dst, (int)g.S, (int)g.Kc, (int)rows, seg_per_slice, (int)g.H,
                            (int)g.W, (int)g.C, (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.Nh, (int)g.Nw,
-                           np.bias ? (int)g.P : -1, np.biasvolt);
+                           np.bias ? (int)g.P : -1, np.biasvolt, (int)s_safe);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
