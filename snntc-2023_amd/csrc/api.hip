@@ -157,13 +157,15 @@ int forward_chain(const SegmentSource& src, const FcFwdWs& ws, const float* w, f
 
 // Backward scratch.  `rows` is the weight row count including a possible bias row; the partial-sum
 // area is sized for the worst case of 256 slices only when slicing can happen at all.
-struct BwdWs { float* upm; float* ym; float* wt; float* partial; int max_split; size_t bytes; };
-BwdWs bwd_ws(void* ws, int64_t S, int64_t rows, int64_t J, int64_t min_base_blocks) {
+struct BwdWs { float* upm; float* ym; float* wt; float* dxp; float* partial; int max_split; size_t bytes; };
+// patch_scratch: elements of the per-patch gradient of conv layers whose dX goes through patch space
+BwdWs bwd_ws(void* ws, int64_t S, int64_t rows, int64_t J, int64_t min_base_blocks, int64_t patch_scratch = 0) {
     Carver c(ws);
     BwdWs r;
     r.upm = c.take<float>(S * J);
     r.ym = c.take<float>(S * J);
     r.wt = c.take<float>(rows * J);
+    r.dxp = c.take<float>(patch_scratch);
     r.max_split = weight_grad_splits(S, min_base_blocks);
     r.partial = c.take<float>(r.max_split > 1 ? (int64_t)r.max_split * rows * J : 0);
     r.bytes = c.used;
@@ -423,7 +425,8 @@ int snntc_cv_backward_workspace_bytes(int64_t B, int64_t H, int64_t W, int64_t C
     int rc = cv_geom(B, H, W, C, Kc, 0, params_host, false, "snntc_cv_backward_workspace_bytes", &g);
     if (rc) return rc;
     if (!bytes) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_cv_backward_workspace_bytes: bytes is NULL");
-    *bytes = bwd_ws(nullptr, g.S, g.P + 1, Kc, cv_weight_base_blocks(g)).bytes;
+    *bytes = bwd_ws(nullptr, g.S, g.P + 1, Kc, cv_weight_base_blocks(g),
+                    cv_grad_input_chan_supported(g) ? 0 : g.S * g.P).bytes;
     return SNNTC_OK;
 }
 
@@ -460,7 +463,8 @@ int snntc_cv_backward(const float* grad, const float* xpad, const float* w, cons
         return dw ? launch_fill_zero(dw, w_rows * Kc, st) : SNNTC_OK;
     }
     if (!grad || !xpad || !w || !oldout) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_cv_backward: NULL tensor pointer");
-    BwdWs ws = bwd_ws(workspace, g.S, g.P + 1, Kc, cv_weight_base_blocks(g));
+    BwdWs ws = bwd_ws(workspace, g.S, g.P + 1, Kc, cv_weight_base_blocks(g),
+                      cv_grad_input_chan_supported(g) ? 0 : g.S * g.P);
     rc = check_workspace(workspace, workspace_bytes, ws.bytes);
     if (rc) return rc;
     const NeuronParams np = neuron_params(params_host[0], params_host[4], params_host[11]);
@@ -472,7 +476,7 @@ int snntc_cv_backward(const float* grad, const float* xpad, const float* w, cons
         } else {
             rc = launch_transpose(w, ws.wt, g.P, Kc, st);   // wt[Kc, P]
             if (rc) return rc;
-            rc = launch_cv_grad_input(xpad, ws.wt, ws.upm, ws.ym, dxpad, g, g.P, st);
+            rc = launch_cv_grad_input(conv_source(xpad, g), ws.wt, ws.upm, ws.ym, ws.dxp, dxpad, g, g.P, st);
         }
         if (rc) return rc;
     }

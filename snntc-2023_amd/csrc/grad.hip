@@ -52,6 +52,23 @@ __global__ void __launch_bounds__(256) fill_zero_kernel(float* __restrict__ p, i
     if (t < n) p[t] = 0.0f;
 }
 
+// Source offset of weight row e relative to the segment base (dense: the column; conv: kh/kw/c).
+__device__ __forceinline__ int row_offset(const SegmentSource& src, int e) {
+    if (!src.conv) return e;
+    const int span = src.Kw * src.C;
+    const int kh = e / span;
+    return kh * src.W * src.C + (e - kh * span);
+}
+
+// Base of segment s inside the source tensor.
+__device__ __forceinline__ const float* segment_base(const SegmentSource& src, int s) {
+    if (!src.conv) return src.base + (size_t)s * src.I;
+    const int per_img = src.Nh * src.Nw;
+    const int a = s / per_img, r2 = s - a * per_img;
+    const int nh = r2 / src.Nw, nw = r2 - nh * src.Nw;
+    return src.base + ((size_t)(a * src.H + nh * src.Sh) * src.W + (size_t)nw * src.Sw) * src.C;
+}
+
 // ---------------------------------------------------------------------------------------------
 // Dense dX.  Lanes run across inputs i (wt[j, i] is read coalesced), each thread carries RB
 // samples whose y/up values are wave-uniform; the four wavefronts of a block split the j range
@@ -60,10 +77,14 @@ __global__ void __launch_bounds__(256) fill_zero_kernel(float* __restrict__ p, i
 constexpr int DX_RB = 4;
 constexpr int DX_UNROLL = 8;
 
+// PATCHES: the "samples" are the implicit patches of a conv layer (src.conv) and the result is the
+// gradient per patch element, dx[S, P], which cv_col2im_kernel then folds back onto the image.
+template <bool PATCHES>
 __global__ void __launch_bounds__(256)
-fc_grad_input_kernel(const float* __restrict__ x, const float* __restrict__ wt,
+fc_grad_input_kernel(const SegmentSource src, const float* __restrict__ wt,
                      const float* __restrict__ upm, const float* __restrict__ ym, float* __restrict__ dx,
                      int B, int I, int J, int wt_stride) {
+    const float* __restrict__ x = src.base;
     __shared__ float red[3][DX_RB][kWave];
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -77,7 +98,7 @@ fc_grad_input_kernel(const float* __restrict__ x, const float* __restrict__ wt,
 #pragma unroll
     for (int r = 0; r < DX_RB; ++r) {
         const int brow = min(b0 + r, B - 1);
-        xr[r] = x[(size_t)brow * I + ic];
+        xr[r] = PATCHES ? segment_base(src, brow)[row_offset(src, (int)ic)] : x[(size_t)brow * I + ic];
         yrow[r] = ym + (size_t)brow * J;
         urow[r] = upm + (size_t)brow * J;
         acc[r] = 0.0f;
@@ -132,23 +153,6 @@ fc_grad_input_kernel(const float* __restrict__ x, const float* __restrict__ wt,
 // ---------------------------------------------------------------------------------------------
 constexpr int DW_RI = 8;
 constexpr int DW_UNROLL = 4;
-
-// Source offset of weight row e relative to the segment base (dense: the column; conv: kh/kw/c).
-__device__ __forceinline__ int row_offset(const SegmentSource& src, int e) {
-    if (!src.conv) return e;
-    const int span = src.Kw * src.C;
-    const int kh = e / span;
-    return kh * src.W * src.C + (e - kh * span);
-}
-
-// Base of segment s inside the source tensor.
-__device__ __forceinline__ const float* segment_base(const SegmentSource& src, int s) {
-    if (!src.conv) return src.base + (size_t)s * src.I;
-    const int per_img = src.Nh * src.Nw;
-    const int a = s / per_img, r2 = s - a * per_img;
-    const int nh = r2 / src.Nw, nw = r2 - nh * src.Nw;
-    return src.base + ((size_t)(a * src.H + nh * src.Sh) * src.W + (size_t)nw * src.Sw) * src.C;
-}
 
 __global__ void __launch_bounds__(256)
 grad_weight_kernel(SegmentSource src, const float* __restrict__ upm, const float* __restrict__ ym,
@@ -254,14 +258,14 @@ reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ ou
 }
 
 // ---------------------------------------------------------------------------------------------
-// Conv dX, gather form.  One thread per element of the padded image (channel fastest, so lanes
-// read wt[kc, (kh,kw,c)] coalesced); it visits every output pixel whose window covers its pixel.
+// Conv dX for layers the channel-lane kernel does not take (fewer than 32 input channels): the
+// gradient per patch element, dxp[S, P], comes from the dense kernel above run over the implicit
+// patches; here every element of the padded image adds up the patch elements that alias it, in
+// (kh, kw) order.  Gather form: no atomics, fixed summation order.
 // ---------------------------------------------------------------------------------------------
 __global__ void __launch_bounds__(256)
-cv_grad_input_kernel(const float* __restrict__ xpad, const float* __restrict__ wt,
-                     const float* __restrict__ upm, const float* __restrict__ ym, float* __restrict__ dxpad,
-                     int64_t n, int H, int W, int C, int Kc, int Kh, int Kw, int Sh, int Sw, int Nh, int Nw,
-                     int wt_stride) {
+cv_col2im_kernel(const float* __restrict__ dxp, float* __restrict__ dxpad, int64_t n, int H, int W, int C, int Kh,
+                 int Kw, int Sh, int Sw, int Nh, int Nw) {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= n) return;
     const int c = (int)(t % C);
@@ -270,27 +274,16 @@ cv_grad_input_kernel(const float* __restrict__ xpad, const float* __restrict__ w
     const int64_t rowi = pix / W;
     const int h = (int)(rowi % H);
     const int a = (int)(rowi / H);
-    const float xv = xpad[t];
-
-    // output rows nh with nh*Sh <= h <= nh*Sh + Kh - 1
-    const int nh_lo = max(0, (h - Kh + Sh) / Sh);      // ceil((h-Kh+1)/Sh) for the non-negative case
-    const int nh_hi = min(Nh - 1, h / Sh);
-    const int nw_lo = max(0, (wx - Kw + Sw) / Sw);
-    const int nw_hi = min(Nw - 1, wx / Sw);
-
+    const int P = Kh * Kw * C;
     float acc = 0.0f;
-    for (int nh = nh_lo; nh <= nh_hi; ++nh) {
-        const int kh = h - nh * Sh;
-        for (int nw = nw_lo; nw <= nw_hi; ++nw) {
-            const int kw = wx - nw * Sw;
-            const int i = (kh * Kw + kw) * C + c;
-            const size_t so = ((size_t)(a * Nh + nh) * Nw + nw) * Kc;
-            const float* __restrict__ wrow = wt + i;
-            for (int kc = 0; kc < Kc; ++kc) {
-                const float yv = ym[so + kc];
-                const float uv = upm[so + kc];
-                acc = __fmaf_rn(xv <= yv ? uv : 0.0f, wrow[(size_t)kc * wt_stride], acc);
-            }
+    for (int kh = 0; kh < Kh; ++kh) {
+        const int hh = h - kh;
+        if (hh < 0 || hh % Sh != 0 || hh / Sh >= Nh) continue;
+        for (int kw = 0; kw < Kw; ++kw) {
+            const int ww = wx - kw;
+            if (ww < 0 || ww % Sw != 0 || ww / Sw >= Nw) continue;
+            const size_t s = (size_t)(a * Nh + hh / Sh) * Nw + ww / Sw;
+            acc += dxp[s * P + (kh * Kw + kw) * C + c];
         }
     }
     dxpad[t] = acc;
@@ -337,7 +330,9 @@ int launch_fc_grad_input(const float* x, const float* wt, const float* upm, cons
     dim3 grid((unsigned)((B + DX_RB - 1) / DX_RB), (unsigned)((I + kWave - 1) / kWave));
     if (grid.y > 65535u) return fail(SNNTC_ERR_TOO_LARGE, "dense backward: input size %lld too large", (long long)I);
     { KernelTimerScope timer_("fc_grad_input", stream);
-    hipLaunchKernelGGL(fc_grad_input_kernel, grid, dim3(256), 0, stream, x, wt, upm, ym, dx, (int)B, (int)I,
+    SegmentSource src{};
+    src.base = x; src.conv = 0; src.I = (int)I;
+    hipLaunchKernelGGL(fc_grad_input_kernel<false>, grid, dim3(256), 0, stream, src, wt, upm, ym, dx, (int)B, (int)I,
                        (int)J, (int)wt_stride);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
@@ -392,15 +387,22 @@ int launch_reduce_partials(const float* partial, float* dw, int64_t n, int nspli
     return SNNTC_OK;
 }
 
-int launch_cv_grad_input(const float* xpad, const float* wt, const float* upm, const float* ym,
+// dxp: scratch of S * P floats (gradient per patch element)
+int launch_cv_grad_input(const SegmentSource& src, const float* wt, const float* upm, const float* ym, float* dxp,
                          float* dxpad, const ConvGeom& g, int64_t wt_stride, hipStream_t stream) {
     const int64_t n = g.B * g.H * g.W * g.C;
     if (n <= 0) return SNNTC_OK;
     if (g.Kc <= 0 || g.S <= 0) return launch_fill_zero(dxpad, n, stream);
+    dim3 grid((unsigned)((g.S + DX_RB - 1) / DX_RB), (unsigned)((g.P + kWave - 1) / kWave));
+    if (grid.y > 65535u) return fail(SNNTC_ERR_TOO_LARGE, "conv backward: patch length %lld too large", (long long)g.P);
     { KernelTimerScope timer_("cv_grad_input", stream);
-    hipLaunchKernelGGL(cv_grad_input_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream, xpad, wt, upm, ym,
-                       dxpad, n, (int)g.H, (int)g.W, (int)g.C, (int)g.Kc, (int)g.Kh, (int)g.Kw, (int)g.Sh,
-                       (int)g.Sw, (int)g.Nh, (int)g.Nw, (int)wt_stride);
+    hipLaunchKernelGGL(fc_grad_input_kernel<true>, grid, dim3(256), 0, stream, src, wt, upm, ym, dxp, (int)g.S,
+                       (int)g.P, (int)g.Kc, (int)wt_stride);
+    }
+    SNNTC_HIP_CHECK(hipGetLastError());
+    { KernelTimerScope timer_("cv_col2im", stream);
+    hipLaunchKernelGGL(cv_col2im_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream, dxp, dxpad, n, (int)g.H,
+                       (int)g.W, (int)g.C, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.Nh, (int)g.Nw);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;

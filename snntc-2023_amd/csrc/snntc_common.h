@@ -112,7 +112,8 @@ int cv_grad_weight_wide_blocks(const ConvGeom& g);
 int launch_cv_grad_weight_wide(const float* xpad, const float* upm, const float* ym, float* dst, int nsplit,
                                const ConvGeom& g, int64_t rows, const NeuronParams& np, hipStream_t stream);
 
-int launch_cv_grad_input(const float* xpad, const float* wt, const float* upm, const float* ym,
+// Conv dX for layers launch_cv_grad_input_chan does not take; dxp is scratch of S * P floats.
+int launch_cv_grad_input(const SegmentSource& src, const float* wt, const float* upm, const float* ym, float* dxp,
                          float* dxpad, const ConvGeom& g, int64_t wt_stride, hipStream_t stream);
 
 int launch_fill_zero(float* p, int64_t n, hipStream_t stream);
