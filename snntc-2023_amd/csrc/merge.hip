@@ -135,20 +135,31 @@ merge_patches_kernel(const float* __restrict__ pix_z, const int32_t* __restrict_
 
     // ---- stage the sorted pixels under the tile ------------------------------------------------
     const int n_px = Kh * tile_cols * C;
-    for (int idx = threadIdx.x; idx < n_px; idx += MERGE_THREADS) {
-        const int c = idx % C;
-        const int pc = idx / C;
-        const int col = pc % tile_cols, kh = pc / tile_cols;
-        const int wp = w_first + col;
-        float z = INFINITY;
-        int ch = c;
-        if (wp < W) {
-            const size_t g = ((size_t)(a * H + nh * Sh + kh) * W + wp) * Cs + c;
-            z = pix_z[g];
-            ch = pix_c[g];
+    // loads are issued in batches: one at a time would cost a memory latency per element
+    constexpr int STAGE = 8;
+    for (int base = threadIdx.x; base < n_px; base += STAGE * MERGE_THREADS) {
+        float zv[STAGE];
+        int cv[STAGE];
+#pragma unroll
+        for (int u = 0; u < STAGE; ++u) {
+            const int idx = base + u * MERGE_THREADS;
+            const int c = idx % C;
+            const int pc = idx / C;
+            const int col = pc % tile_cols, kh = pc / tile_cols;
+            const int wp = w_first + col;
+            zv[u] = INFINITY;
+            cv[u] = c;
+            if (idx < n_px && wp < W) {
+                const size_t g = ((size_t)(a * H + nh * Sh + kh) * W + wp) * Cs + c;
+                zv[u] = pix_z[g];
+                cv[u] = pix_c[g];
+            }
         }
-        px_z[idx] = z;
-        px_c[idx] = (uint16_t)ch;
+#pragma unroll
+        for (int u = 0; u < STAGE; ++u) {
+            const int idx = base + u * MERGE_THREADS;
+            if (idx < n_px) { px_z[idx] = zv[u]; px_c[idx] = (uint16_t)cv[u]; }
+        }
     }
     __syncthreads();
 
