@@ -240,21 +240,35 @@ grad_weight_kernel(SegmentSource src, const float* __restrict__ upm, const float
     }
 }
 
-__global__ void __launch_bounds__(256)
+// A block adds up 32 elements: its eight groups of 32 threads each take a contiguous eighth of the
+// slices (two chains per thread keep loads in flight) and the eight sums are added in group order.
+// The order of additions depends only on nsplit, never on timing.
+constexpr int RED_ELEMS = 32, RED_GROUPS = 8;
+
+__global__ void __launch_bounds__(RED_ELEMS * RED_GROUPS)
 reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ out, int64_t n, int nsplit) {
-    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= n) return;
-    // slices are added in ascending order, four independent chains to keep the loads in flight
-    float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
-    int z = 0;
-    for (; z + 4 <= nsplit; z += 4) {
-        a0 += partial[(size_t)z * n + t];
-        a1 += partial[(size_t)(z + 1) * n + t];
-        a2 += partial[(size_t)(z + 2) * n + t];
-        a3 += partial[(size_t)(z + 3) * n + t];
+    __shared__ float part[RED_GROUPS][RED_ELEMS];
+    const int e = threadIdx.x % RED_ELEMS, g = threadIdx.x / RED_ELEMS;
+    const int64_t t = (int64_t)blockIdx.x * RED_ELEMS + e;
+    const int per = (nsplit + RED_GROUPS - 1) / RED_GROUPS;
+    const int z_lo = g * per, z_hi = min(nsplit, z_lo + per);
+    float a0 = 0.0f, a1 = 0.0f;
+    if (t < n) {
+        int z = z_lo;
+        for (; z + 2 <= z_hi; z += 2) {
+            a0 += partial[(size_t)z * n + t];
+            a1 += partial[(size_t)(z + 1) * n + t];
+        }
+        if (z < z_hi) a0 += partial[(size_t)z * n + t];
     }
-    for (; z < nsplit; ++z) a0 += partial[(size_t)z * n + t];
-    out[t] = (a0 + a1) + (a2 + a3);
+    part[g][e] = a0 + a1;
+    __syncthreads();
+    if (g == 0 && t < n) {
+        float sum = part[0][e];
+#pragma unroll
+        for (int k = 1; k < RED_GROUPS; ++k) sum += part[k][e];
+        out[t] = sum;
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -380,8 +394,8 @@ int launch_reduce_partials(const float* partial, float* dw, int64_t n, int nspli
     if (n <= 0 || nsplit <= 1) return SNNTC_OK;
     {
         KernelTimerScope timer_("reduce_partials", stream);
-        hipLaunchKernelGGL(reduce_partials_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream, partial, dw,
-                           n, nsplit);
+        hipLaunchKernelGGL(reduce_partials_kernel, dim3(blocks_for(n, RED_ELEMS)), dim3(RED_ELEMS * RED_GROUPS), 0,
+                           stream, partial, dw, n, nsplit);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
