@@ -296,7 +296,10 @@ cv_grad_weight_wide_kernel(const float* __restrict__ xpad, const float* __restri
 __device__ __forceinline__ void dw_rows16(float (&acc)[DWW_RI], int base, float x, float y, float u) {
     float d;
     float* a = acc + base;
+    // the leading s_nop covers the two wait states a DPP read needs after a vector write of the same
+    // register, should the compiler have placed a copy into x right before the block
     asm volatile(
+        "s_nop 1\n"
         SNNTC_DW_ROW(0, a0) SNNTC_DW_ROW(1, a1) SNNTC_DW_ROW(2, a2) SNNTC_DW_ROW(3, a3)
         SNNTC_DW_ROW(4, a4) SNNTC_DW_ROW(5, a5) SNNTC_DW_ROW(6, a6) SNNTC_DW_ROW(7, a7)
         SNNTC_DW_ROW(8, a8) SNNTC_DW_ROW(9, a9) SNNTC_DW_ROW(10, a10) SNNTC_DW_ROW(11, a11)
