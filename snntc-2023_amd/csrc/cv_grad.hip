@@ -111,13 +111,28 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
             for (int kc0 = 0; kc0 < Kc; kc0 += KCB) {
                 // stage the patch row: slots whose patch does not exist are never read
                 __builtin_amdgcn_wave_barrier();
-                for (int d = 0; d < n_slots; ++d) {
-                    const int ww = w0 - Kw + 1 + d;
-                    if (ww < 0 || ww % Sw != 0 || ww / Sw >= Nw) continue;
-                    if (lane < KCB) {
-                        const size_t so = (row0 + ww / Sw) * Kc + kc0 + lane;
-                        ys[d * KCB + lane] = ym[so];
-                        us[d * KCB + lane] = upm[so];
+                // loads of STAGE slots are issued together: one slot at a time would cost a memory
+                // latency per slot, and nothing of this wavefront overlaps with it
+                constexpr int STAGE = 6;
+                for (int d0 = 0; d0 < n_slots; d0 += STAGE) {
+                    float yv[STAGE], uv[STAGE];
+                    bool have[STAGE];
+#pragma unroll
+                    for (int k = 0; k < STAGE; ++k) {
+                        const int ww = w0 - Kw + 1 + d0 + k;
+                        have[k] = d0 + k < n_slots && ww >= 0 && ww % Sw == 0 && ww / Sw < Nw && lane < KCB;
+                        if (have[k]) {
+                            const size_t so = (row0 + ww / Sw) * Kc + kc0 + lane;
+                            yv[k] = ym[so];
+                            uv[k] = upm[so];
+                        }
+                    }
+#pragma unroll
+                    for (int k = 0; k < STAGE; ++k) {
+                        if (have[k]) {
+                            ys[(d0 + k) * KCB + lane] = yv[k];
+                            us[(d0 + k) * KCB + lane] = uv[k];
+                        }
                     }
                 }
                 __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
