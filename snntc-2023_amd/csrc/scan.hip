@@ -133,7 +133,9 @@ scan_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
 // ---------------------------------------------------------------------------------------------
 constexpr int LDS_SCAN_THREADS = 1024;
 constexpr int LDS_SCAN_BYTES = 160 * 1024;
-constexpr int LDS_SCAN_TARGET = 160 * 1024;  // widest slice that fits: the register budget allows one 16-wave workgroup per CU anyway, and fewer slices re-read the sorted rows less often
+// The widest slice that fits is taken: the register budget allows one 16-wave workgroup per CU anyway,
+// and fewer slices re-read the sorted rows less often.
+constexpr int LDS_SCAN_TARGET = 160 * 1024;
 
 struct Chunk {
     float x[CHUNK];
@@ -644,9 +646,9 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     // lane in 16-wave workgroups balances better.
     constexpr int CH = 2;          // four per lane need 151 registers: too few wavefronts per SIMD, measured slower
     const int64_t multi_items = (S + CH * SEGS - 1) / (CH * SEGS);
-    const bool pair = !low_latency && multi_items * n_slices >= (int64_t)cus * 4 * 4;
-    const int64_t work_items = pair ? multi_items : items;
-    if (pair && CH == 4) WAVES = MULTI_SCAN_THREADS / kWave;
+    const bool multi = !low_latency && multi_items * n_slices >= (int64_t)cus * 4 * 4;
+    const int64_t work_items = multi ? multi_items : items;
+    if (multi && CH == 4) WAVES = MULTI_SCAN_THREADS / kWave;
     // resident workgroups per CU: split the segments so that slices x groups covers the chip
     const int wgs_per_cu = lds_bytes * 2 <= (size_t)LDS_SCAN_BYTES ? 2 : 1;
     int64_t n_groups = ((int64_t)cus * wgs_per_cu + n_slices - 1) / n_slices;
@@ -654,13 +656,13 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     if (n_groups > max_groups) n_groups = max_groups;
     if (n_groups < 1) n_groups = 1;
     auto kern_k = low_latency ? scan_lds_kernel<COLS, true, true>
-                  : pair ? scan_lds_multi_kernel<COLS, CH, true> : scan_lds_kernel<COLS, true, false>;
+                  : multi ? scan_lds_multi_kernel<COLS, CH, true> : scan_lds_kernel<COLS, true, false>;
     auto kern = low_latency ? scan_lds_kernel<COLS, false, true>
-                : pair ? scan_lds_multi_kernel<COLS, CH, false> : scan_lds_kernel<COLS, false, false>;
+                : multi ? scan_lds_multi_kernel<COLS, CH, false> : scan_lds_kernel<COLS, false, false>;
     // raise the dynamic-LDS limit of both instantiations once (not per launch: the call is not
     // allowed while a stream is being captured into a graph)
     static bool lds_limit_raised[3] = {false, false, false};
-    const int variant = low_latency ? 1 : (pair ? 2 : 0);
+    const int variant = low_latency ? 1 : (multi ? 2 : 0);
     if (!lds_limit_raised[variant]) {
         SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern_k),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, LDS_SCAN_BYTES));
