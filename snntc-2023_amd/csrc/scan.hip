@@ -358,8 +358,10 @@ scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ pe
     extern __shared__ float wl[];                          // [I + bias][COLS]
     constexpr int SEGS = kWave / COLS;                     // segments per wavefront
     const int WAVES = blockDim.x / kWave;                  // 1..16, chosen by the launcher
-    const int slice = blockIdx.x % n_slices;
-    const int group = blockIdx.x / n_slices;
+    // slice-major over XCD-contiguous ids: the workgroups of one XCD share a few weight slices
+    const int block = xcd_contiguous(blockIdx.x, gridDim.x);
+    const int slice = block / n_groups;
+    const int group = block - slice * n_groups;
     const int j0 = slice * COLS;
     const int rows = I + np.bias;
 
@@ -495,8 +497,10 @@ scan_lds_multi_kernel(const float* __restrict__ sorted, const int32_t* __restric
     constexpr int LANES = COLS / CH;                       // lanes per segment
     constexpr int SEGS = kWave / LANES;                    // segments per wavefront
     const int WAVES = blockDim.x / kWave;
-    const int slice = blockIdx.x % n_slices;
-    const int group = blockIdx.x / n_slices;
+    // slice-major over XCD-contiguous ids: the workgroups of one XCD share a few weight slices
+    const int block = xcd_contiguous(blockIdx.x, gridDim.x);
+    const int slice = block / n_groups;
+    const int group = block - slice * n_groups;
     const int j0 = slice * COLS;
     const int rows = I + np.bias;
     fill_weight_slice<COLS>(wl, w, rows, J, j0);

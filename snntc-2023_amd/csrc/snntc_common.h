@@ -26,6 +26,17 @@ int fail(int code, const char* fmt, ...);
 
 inline size_t align_up(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
 
+// Workgroups are handed to the eight XCDs (each with an L2 of its own) round-robin by workgroup
+// id.  xcd_contiguous() renumbers a 1-D grid so that every XCD works on one contiguous range of
+// the returned ids: neighbours in that numbering, which share operands, then share an L2 too.
+// A bijection on [0, total) for any total.
+constexpr int kXcds = 8;
+__device__ __forceinline__ int xcd_contiguous(int block, int total) {
+    const int xcd = block % kXcds, local = block / kXcds;
+    const int per = total / kXcds, extra = total % kXcds;
+    return xcd * per + (xcd < extra ? xcd : extra) + local;
+}
+
 // Opt-in per-kernel timing (snntc_profile_*): while enabled, every launcher brackets its kernel
 // with a pair of HIP events on the launch stream.  Disabled (the default) it costs one branch.
 struct KernelTimerScope {
