@@ -90,11 +90,12 @@ class MlpTrainStep(Workload):
 
     def step(self):
         torch = self.torch
-        loss = self.snn.loss_func(self.forward(), self.onehot)
-        grads = torch.autograd.grad(loss, self.params)
-        with torch.no_grad():
-            torch._foreach_add_(self.params, list(grads), alpha=-self.lr)     # SGD, one multi-tensor kernel
-        return loss
+        times = self.forward()
+        # the loss kernel hands back the gradient of the batch mean: backpropagation starts from it
+        sample_loss, dtimes = self.snn.softmax_time_loss(times.detach(), self.onehot)
+        grads = torch.autograd.grad(times, self.params, grad_outputs=dtimes)
+        self.snn.sgd_update(self.params, grads, self.lr)                      # SGD, all layers in one launch
+        return sample_loss.mean()
 
     def layers(self):
         with self.torch.no_grad():
@@ -184,11 +185,12 @@ class CifarTrainStep(Workload):
 
     def step(self):
         torch = self.torch
-        loss = self.snn.loss_func(self.forward(), self.onehot)
-        grads = torch.autograd.grad(loss, self.params)
-        with torch.no_grad():
-            torch._foreach_add_(self.params, list(grads), alpha=-self.lr)     # SGD, one multi-tensor kernel
-        return loss
+        times = self.forward()
+        # the loss kernel hands back the gradient of the batch mean: backpropagation starts from it
+        sample_loss, dtimes = self.snn.softmax_time_loss(times.detach(), self.onehot)
+        grads = torch.autograd.grad(times, self.params, grad_outputs=dtimes)
+        self.snn.sgd_update(self.params, grads, self.lr)                      # SGD, all layers in one launch
+        return sample_loss.mean()
 
     def layers(self):
         with self.torch.no_grad():

@@ -161,6 +161,17 @@ SNNTC_API int snntc_softmax_time_loss(const float* times, const float* label, fl
                             int64_t B, int64_t J, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * SGD update of a training step: w[t][e] -= lr * dw[t][e] for e in [0, n[t]), t in [0, count).
+ * The reference leaves the update to the framework's optimizer (snntc/snntc-mnist.py:70,92-93);
+ * here all weight tensors of a network are updated by one launch (per 32 tensors).
+ * w, dw and n are HOST arrays of `count` entries holding device pointers / element counts; they
+ * are read before the call returns.  Tensors with n[t] == 0 are skipped.
+ * Errors: count < 0, n[t] < 0, a NULL array or a NULL tensor with n[t] > 0 -> BAD_ARGUMENT.
+ * ------------------------------------------------------------------------------------------- */
+SNNTC_API int snntc_sgd_update(float* const* w, const float* const* dw, const int64_t* n, int64_t count, float lr,
+                     void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * Per-kernel timing (no counterpart in the reference, which only times whole scripts with
  * time.time()).  While enabled, every kernel the library launches is bracketed by a pair of HIP
  * events on its launch stream; this is the only process-wide state the library keeps and it is

@@ -306,6 +306,19 @@ int snntc_softmax_time_loss(const float* times, const float* label, float* sampl
     return launch_softmax_time_loss(times, label, sample_loss, dtimes, B, J, static_cast<hipStream_t>(stream));
 }
 
+int snntc_sgd_update(float* const* w, const float* const* dw, const int64_t* n, int64_t count, float lr,
+                     void* stream) {
+    if (count < 0 || count > INT32_MAX) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_sgd_update: bad tensor count");
+    if (count == 0) return SNNTC_OK;
+    if (!w || !dw || !n) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_sgd_update: null array");
+    for (int64_t t = 0; t < count; ++t) {
+        if (n[t] < 0) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_sgd_update: tensor %lld has a negative size", (long long)t);
+        if (n[t] > 0 && (!w[t] || !dw[t]))
+            return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_sgd_update: tensor %lld is a null pointer", (long long)t);
+    }
+    return launch_sgd_update(w, dw, n, (int)count, lr, static_cast<hipStream_t>(stream));
+}
+
 int snntc_profile_enable(int on) {
     std::lock_guard<std::mutex> lock(g_prof_mutex);
     prof_drain();

@@ -240,14 +240,14 @@ __device__ __forceinline__ void scan_chunk(float& wsum, float& ysum, float& ya, 
 #pragma unroll
         for (int u = 0; u < CHUNK; ++u) xs[u] = __builtin_amdgcn_readfirstlane(__float_as_int(x[u]));
         if (WANT_K)
-            asm volatile(SNNTC_SCAN_BODY_K : SNNTC_SCAN_STATE : SNNTC_SCAN_INPUTS("s", xs) : "vcc");
+            asm volatile(SNNTC_SCAN_BODY_K : SNNTC_SCAN_STATE : SNNTC_SCAN_INPUTS("s", xs) : "vcc", "scc");
         else
-            asm volatile(SNNTC_SCAN_BODY : SNNTC_SCAN_STATE : SNNTC_SCAN_INPUTS("s", xs) : "vcc");
+            asm volatile(SNNTC_SCAN_BODY : SNNTC_SCAN_STATE : SNNTC_SCAN_INPUTS("s", xs) : "vcc", "scc");
     } else {
         if (WANT_K)
-            asm volatile(SNNTC_SCAN_BODY_K : SNNTC_SCAN_STATE : SNNTC_SCAN_INPUTS("v", x) : "vcc");
+            asm volatile(SNNTC_SCAN_BODY_K : SNNTC_SCAN_STATE : SNNTC_SCAN_INPUTS("v", x) : "vcc", "scc");
         else
-            asm volatile(SNNTC_SCAN_BODY : SNNTC_SCAN_STATE : SNNTC_SCAN_INPUTS("v", x) : "vcc");
+            asm volatile(SNNTC_SCAN_BODY : SNNTC_SCAN_STATE : SNNTC_SCAN_INPUTS("v", x) : "vcc", "scc");
     }
 }
 
@@ -293,12 +293,12 @@ __device__ __forceinline__ void scan_chunk_vector(float& wsum, float& ysum, floa
                      SNNTC_VSCAN_STEP(2) SNNTC_SCAN_COUNT SNNTC_VSCAN_STEP(3) SNNTC_SCAN_COUNT SNNTC_VSCAN_STEP(4)
                      SNNTC_SCAN_COUNT SNNTC_VSCAN_STEP(5) SNNTC_SCAN_COUNT SNNTC_VSCAN_STEP(6) SNNTC_SCAN_COUNT
                      SNNTC_VSCAN_STEP(7) SNNTC_SCAN_COUNT SNNTC_VSCAN_EPILOGUE
-                     : SNNTC_VSCAN_STATE : SNNTC_VSCAN_INPUTS : "vcc");
+                     : SNNTC_VSCAN_STATE : SNNTC_VSCAN_INPUTS : "vcc", "scc");
     else
         asm volatile(SNNTC_VSCAN_PROLOGUE SNNTC_VSCAN_STEP(0) SNNTC_VSCAN_STEP(1) SNNTC_VSCAN_STEP(2)
                      SNNTC_VSCAN_STEP(3) SNNTC_VSCAN_STEP(4) SNNTC_VSCAN_STEP(5) SNNTC_VSCAN_STEP(6)
                      SNNTC_VSCAN_STEP(7) SNNTC_VSCAN_EPILOGUE
-                     : SNNTC_VSCAN_STATE : SNNTC_VSCAN_INPUTS : "vcc");
+                     : SNNTC_VSCAN_STATE : SNNTC_VSCAN_INPUTS : "vcc", "scc");
 }
 
 // Copies columns [j0, j0 + COLS) of all `rows` rows of W[rows, J] into LDS as wl[row][COLS] (zeros

@@ -128,6 +128,10 @@ int launch_cv_grad_input(const SegmentSource& src, const float* wt, const float*
                          float* dxpad, const ConvGeom& g, int64_t wt_stride, hipStream_t stream);
 
 int launch_fill_zero(float* p, int64_t n, hipStream_t stream);
+
+// w[t] -= lr * dw[t] for `count` tensors of n[t] elements (host arrays of device pointers).
+int launch_sgd_update(float* const* w, const float* const* dw, const int64_t* n, int count, float lr,
+                      hipStream_t stream);
 int launch_softmax_time_loss(const float* times, const float* label, float* sample_loss, float* dtimes,
                              int64_t B, int64_t J, hipStream_t stream);
 

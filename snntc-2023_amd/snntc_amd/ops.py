@@ -272,6 +272,33 @@ def softmax_time_loss(times, label, want_loss=True, want_grad=True):
     return loss, grad
 
 
+def sgd_update(params, grads, lr):
+    """In place ``w -= lr * dw`` for every (w, dw) pair, all tensors in one launch: the SGD update of
+    a training step (the reference hands it to the framework's optimizer, snntc/snntc-mnist.py:70)."""
+    lib = _lib.load()
+    params, grads = list(params), list(grads)
+    if len(params) != len(grads):
+        raise ValueError(f"sgd_update: {len(params)} weight tensors but {len(grads)} gradients")
+    if not params:
+        return
+    ws, gs = [], []
+    for i, (w, g) in enumerate(zip(params, grads)):
+        w = w.data if isinstance(w, torch.nn.Parameter) else w
+        if not (isinstance(w, torch.Tensor) and w.is_cuda and w.dtype == torch.float32 and w.is_contiguous()):
+            raise _lib.SnntcLibraryError(f"sgd_update: weight {i} must be a contiguous float32 tensor on a ROCm GPU")
+        if tuple(g.shape) != tuple(w.shape) or g.dtype != torch.float32 or g.device != w.device:
+            raise ValueError(f"sgd_update: gradient {i} does not match its weight tensor")
+        ws.append(w)
+        gs.append(g.detach().contiguous())
+    k = len(ws)
+    vp = ctypes.c_void_p
+    w_arr = (vp * k)(*[w.data_ptr() for w in ws])
+    g_arr = (vp * k)(*[g.data_ptr() for g in gs])
+    n_arr = (ctypes.c_int64 * k)(*[w.numel() for w in ws])
+    with torch.cuda.device(ws[0].device):
+        _lib.check(lib.snntc_sgd_update(w_arr, g_arr, n_arr, k, float(lr), _stream(ws[0].device)))
+
+
 class SoftmaxTimeLoss(torch.autograd.Function):
     """mean_b CE(label_b, softmax(-times_b)); the gradient is produced by the forward kernel."""
 

@@ -137,3 +137,18 @@ def test_loss_argument_errors(lib):
     assert lib.snntc_softmax_time_loss(one, one, None, None, 2, 4, None) == 3
     assert lib.snntc_softmax_time_loss(one, one, one, one, 1 << 20, 1 << 20, None) == 2
     assert lib.snntc_softmax_time_loss(one, one, one, one, 0, 4, None) == 0      # empty batch: nothing to do
+
+
+def test_sgd_update_argument_errors(lib):
+    vp, i64 = ctypes.c_void_p, ctypes.c_int64
+    one = (vp * 2)(256, 256)                       # never dereferenced: the checks come first
+    null_in = (vp * 2)(256, None)
+    n = (i64 * 2)(4, 4)
+    assert lib.snntc_sgd_update(one, one, n, -1, 0.1, None) == 3
+    assert lib.snntc_sgd_update(None, one, n, 2, 0.1, None) == 3
+    assert lib.snntc_sgd_update(one, one, None, 2, 0.1, None) == 3
+    assert lib.snntc_sgd_update(one, one, (i64 * 2)(4, -4), 2, 0.1, None) == 3
+    assert lib.snntc_sgd_update(null_in, one, n, 2, 0.1, None) == 3
+    assert lib.snntc_sgd_update(one, null_in, n, 2, 0.1, None) == 3
+    assert lib.snntc_sgd_update(None, None, None, 0, 0.1, None) == 0            # no tensors: nothing to do
+    assert lib.snntc_sgd_update(null_in, null_in, (i64 * 2)(0, 0), 2, 0.1, None) == 0   # empty tensors are skipped

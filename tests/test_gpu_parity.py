@@ -204,6 +204,32 @@ def test_loss_kernel_against_closed_form(B, J):
     assert np.all(np.abs(T.grad.cpu().numpy() - 3.0 * want_g) <= 3e-6 / B + 3e-6 * np.abs(want_g))
 
 
+def test_sgd_update_matches_numpy():
+    """w -= lr*dw over tensors of awkward sizes (empty, shorter than a vector, unaligned views, more
+    than one table of 32): within one rounding of the float32 formula, and nothing else is touched."""
+    import snntc_amd as snn
+    rng = np.random.default_rng(5)
+    sizes = [(785, 800), (801, 10), (0, 7), (1,), (3,), (5, 1023)] + [(int(n),) for n in rng.integers(1, 5000, 34)]
+    ws = [rng.standard_normal(sz).astype(np.float32) for sz in sizes]
+    gs = [rng.standard_normal(sz).astype(np.float32) for sz in sizes]
+    lr = 0.0123
+    dev_w = [t(w) for w in ws]
+    # one weight is a view that starts 4 bytes into its buffer: the vector path must not be taken for it
+    backing = torch.zeros(ws[5].size + 1, device=DEV)
+    backing[1:] = t(ws[5]).reshape(-1)
+    dev_w[5] = backing[1:].view(sizes[5])
+    snn.sgd_update(dev_w, [t(g) for g in gs], lr)
+    for w, g, got in zip(ws, gs, dev_w):
+        want = w.astype(np.float64) - lr * g.astype(np.float64)
+        err = np.abs(got.cpu().numpy() - want)
+        assert np.all(err <= 1.2e-7 * np.maximum(np.abs(want), np.abs(w)) + 1e-30)
+    assert float(backing[0]) == 0.0
+    with pytest.raises(ValueError):
+        snn.sgd_update(dev_w[:2], [t(gs[0])], lr)
+    with pytest.raises(ValueError):
+        snn.sgd_update(dev_w[:1], [t(gs[1])], lr)
+
+
 PARAM_SWEEP = [
     # biasvolt, theta, max_time
     (0.7, 1.0, 1e5),
