@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the SNN-TC hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mlp|dense|conv|cifar]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mlp|dense|conv|cifar|imagenet]
 
 Prints ONE JSON line.  A "step" is one pass of the workload over one synthetic batch that is
 already resident in HBM:
@@ -176,7 +176,8 @@ class CifarTrainStep(Workload):
         self.acts = []
         for l in self.net:
             if isinstance(l, str):
-                h = h.reshape(h.shape[0], -1)
+                # "flatten", or the global min-time pool (earliest spike of every channel)
+                h = h.amin(dim=(1, 2)) if l == "global_min" else h.reshape(h.shape[0], -1)
                 continue
             if record and hasattr(l, "weight"):
                 self.acts.append((l, h))
@@ -204,7 +205,39 @@ class CifarTrainStep(Workload):
         return out
 
 
-WORKLOADS = {"mlp": MlpTrainStep, "dense": DenseLayerStep, "conv": ConvLayerStep, "cifar": CifarTrainStep}
+class ImagenetFwdBwd(CifarTrainStep):
+    """BASELINE config 5: forward + loss + backward (no weight update)."""
+    name = "imagenet-shaped conv net B=32 fwd+bwd"
+
+    def __init__(self, torch, snn, dev, seed=0, batch=32):
+        rng = np.random.default_rng(seed)
+        self.torch, self.batch, self.snn = torch, batch, snn
+        x = rng.random((batch, 224, 224, 3)).astype(np.float32)
+        self.z = torch.from_numpy(np.exp(1.0 - x)).to(dev)
+        labels = rng.integers(0, 1000, batch)
+        self.onehot = torch.from_numpy(np.eye(1000, dtype=np.float32)[labels]).to(dev)
+
+        def conv(ci, co, k=3, s=1):
+            return snn.SNN_conv(ci, co, k, s, 'SAME', weight=_w_init(rng, k * k * ci, co)).to(dev)
+
+        pool = lambda: snn.SNN_maxpool2d(2, 2, 'SAME')
+        self.net = [conv(3, 64, 7, 2), pool(),
+                    conv(64, 64), conv(64, 64), pool(),
+                    conv(64, 128), conv(128, 128), pool(),
+                    conv(128, 256), conv(256, 256), pool(),
+                    conv(256, 512), conv(512, 512),
+                    "global_min", snn.SNN_dense(512, 1000, weight=_w_init(rng, 512, 1000)).to(dev)]
+        self.params = [l.weight for l in self.net if hasattr(l, "weight")]
+
+    def step(self):
+        times = self.forward()
+        sample_loss, dtimes = self.snn.softmax_time_loss(times.detach(), self.onehot)
+        self.grads = self.torch.autograd.grad(times, self.params, grad_outputs=dtimes)
+        return sample_loss.mean()
+
+
+WORKLOADS = {"mlp": MlpTrainStep, "dense": DenseLayerStep, "conv": ConvLayerStep, "cifar": CifarTrainStep,
+             "imagenet": ImagenetFwdBwd}
 
 
 # ------------------------------------------------------------------------------------------------
@@ -315,9 +348,10 @@ def roofline_for(name, flops, nbytes, avg_ms, launches_per_step):
     t_valu = flops / (VALU_PEAK_TFLOPS * 1e12)
     if t_valu >= t_hbm:
         ach = flops / t / 1e12
-        return {"bound": "valu", "achieved": ach, "peak": VALU_PEAK_TFLOPS, "unit": "TFLOP/s",
+        return {"bound": "mfma", "achieved": ach, "peak": VALU_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": ach / VALU_PEAK_TFLOPS, "traffic": None,
-                "note": "compute side of the roofline priced at the fp32 vector peak; no MFMA instructions are issued"}
+                "note": "compute-bound: priced at the fp32 peak (157.3 TFLOP/s, equally the fp32 vector-ALU peak); "
+                        "the path runs on the vector ALUs, no MFMA instruction is issued"}
     ach = nbytes / t / 1e9
     return {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS,
             "traffic": None}
@@ -357,16 +391,24 @@ def cpu_baseline(workload_key, seed=0):
                 g = np.zeros((2 * B, a.shape[1]), np.float32); g[:B] = dx
         what = f"the same dense layer stack, {reps} steps"
     else:
+        # conv layers (hw, C, Kc, kernel, stride); pooling and loss are left out of the CPU sample
         if workload_key == "conv":
-            specs, dense, B = [(32, 64, 64)], (), 32
-        else:  # cifar: conv layers (hw, C, Kc); pooling and loss are left out of the CPU sample
-            specs = [(32, 3, 32), (32, 32, 32), (16, 32, 64), (16, 64, 64), (8, 64, 128)]
+            specs, dense, B = [(32, 64, 64, 3, 1)], (), 32
+        elif workload_key == "cifar":
+            specs = [(32, 3, 32, 3, 1), (32, 32, 32, 3, 1), (16, 32, 64, 3, 1), (16, 64, 64, 3, 1), (8, 64, 128, 3, 1)]
             dense, B = ((2048, 512), (512, 10)), 32
-        for hw, C, Kc in specs:
+        else:  # imagenet
+            specs = [(224, 3, 64, 7, 2), (56, 64, 64, 3, 1), (56, 64, 64, 3, 1), (28, 64, 128, 3, 1),
+                     (28, 128, 128, 3, 1), (14, 128, 256, 3, 1), (14, 256, 256, 3, 1), (7, 256, 512, 3, 1),
+                     (7, 512, 512, 3, 1)]
+            dense, B = ((512, 1000),), 1
+        for hw, C, Kc, k, st in specs:
             x = np.exp(rng.random((B, hw, hw, C))).astype(np.float32)
-            xpad = np.pad(x, ((0, 0), (1, 1), (1, 1), (0, 0)), constant_values=np.float32(1e5))
-            w = _w_init(rng, 9 * C, Kc)
-            p = capi.cv_params(3, 3, 1, 1, same=True, biasvolt=1.0)
+            pad = max((-(-hw // st) - 1) * st + k - hw, 0)         # SAME: the smaller half goes in front
+            xpad = np.pad(x, ((0, 0), (pad // 2, pad - pad // 2), (pad // 2, pad - pad // 2), (0, 0)),
+                          constant_values=np.float32(1e5))
+            w = _w_init(rng, k * k * C, Kc)
+            p = capi.cv_params(k, k, st, st, same=True, biasvolt=1.0)
             y = capi.cv_forward_host(xpad, w, p)
             out = np.concatenate((y, np.zeros_like(y)), axis=0)
             g = np.zeros_like(out); g[:B] = rng.standard_normal(y.shape)
