@@ -13,6 +13,8 @@
 // so one unsigned compare against a threshold decides precedence including ties.
 // The result is identical to the bitonic path (and to a stable argsort); it replaces the same
 // reference code (snntc/snncv_kernels.cu.cc:112-166).
+#include <atomic>
+
 #include "snntc_common.h"
 
 namespace snntc {
@@ -302,11 +304,14 @@ int launch_merge_patches(const float* pix_z, const int32_t* pix_c, int64_t Cs, f
     const int eb = per_lane >= 4 ? 4 : (int)per_lane;
     auto kern = eb == 1 ? merge_patches_kernel<1> : eb == 2 ? merge_patches_kernel<2>
               : eb == 3 ? merge_patches_kernel<3> : merge_patches_kernel<4>;
-    static bool lds_limit_raised[5] = {false, false, false, false, false};
-    if (!lds_limit_raised[eb]) {
+    static std::atomic<bool> lds_limit_raised[kMaxDevices][5];     // once per device and instantiation
+    int dev = 0;
+    SNNTC_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(SNNTC_ERR_UNSUPPORTED, "patch merge: device index %d not supported", dev);
+    if (!lds_limit_raised[dev][eb].load(std::memory_order_acquire)) {
         SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
-        lds_limit_raised[eb] = true;
+        lds_limit_raised[dev][eb].store(true, std::memory_order_release);
     }
     {
         KernelTimerScope timer_("merge_patches", stream);

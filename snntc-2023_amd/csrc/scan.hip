@@ -14,6 +14,8 @@
 // steps are requested while the current eight are consumed.  A lane that has closed its causal set
 // drops out of the loop (it is masked off and issues no further reads); the wavefront leaves when
 // its last lane has.
+#include <atomic>
+
 #include "snntc_common.h"
 
 namespace snntc {
@@ -628,13 +630,17 @@ template <int COLS>
 int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_real, const float* w, float* y,
                     float* rcp, int32_t* causal_k, int64_t S, int64_t I, int64_t stride, int64_t J,
                     const NeuronParams& np, size_t lds_bytes, hipStream_t stream) {
-    static int cus = 0;
+    // per device: CU count, and whether the dynamic-LDS limit of the instantiations was raised
+    static std::atomic<int> cu_count[kMaxDevices];
+    int dev = 0;
+    SNNTC_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(SNNTC_ERR_UNSUPPORTED, "scan: device index %d not supported", dev);
+    int cus = cu_count[dev].load(std::memory_order_relaxed);
     if (cus == 0) {
-        int dev = 0;
         hipDeviceProp_t prop;
-        SNNTC_HIP_CHECK(hipGetDevice(&dev));
         SNNTC_HIP_CHECK(hipGetDeviceProperties(&prop, dev));
         cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+        cu_count[dev].store(cus, std::memory_order_relaxed);
     }
     constexpr int SEGS = kWave / COLS;
     const int n_slices = (int)((J + COLS - 1) / COLS);
@@ -665,14 +671,14 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
                 : multi ? scan_lds_multi_kernel<COLS, CH, false> : scan_lds_kernel<COLS, false, false>;
     // raise the dynamic-LDS limit of both instantiations once (not per launch: the call is not
     // allowed while a stream is being captured into a graph)
-    static bool lds_limit_raised[3] = {false, false, false};
+    static std::atomic<bool> lds_limit_raised[kMaxDevices][3];
     const int variant = low_latency ? 1 : (multi ? 2 : 0);
-    if (!lds_limit_raised[variant]) {
+    if (!lds_limit_raised[dev][variant].load(std::memory_order_acquire)) {
         SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern_k),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, LDS_SCAN_BYTES));
         SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, LDS_SCAN_BYTES));
-        lds_limit_raised[variant] = true;
+        lds_limit_raised[dev][variant].store(true, std::memory_order_release);
     }
     dim3 grid((unsigned)(n_slices * n_groups)), block((unsigned)(WAVES * kWave));
     {

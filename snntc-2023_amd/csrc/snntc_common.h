@@ -13,6 +13,7 @@ namespace snntc {
 constexpr int kWave = 64;              // CDNA wavefront width
 constexpr int kMaxSegment = 8192;      // longest sortable segment (power-of-two padded)
 constexpr size_t kAlign = 256;         // workspace sub-buffer alignment
+constexpr int kMaxDevices = 64;        // device indices the per-device one-time state covers
 
 // Records a formatted message for snntc_last_error() and returns `code`.
 int fail(int code, const char* fmt, ...);
