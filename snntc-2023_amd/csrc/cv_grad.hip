@@ -65,7 +65,7 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
                           const float* __restrict__ upm, const float* __restrict__ ym,
                           float* __restrict__ dxpad, int H, int W, int C, int Kc, int Kh, int Kw, int Sh, int Sw,
                           int Nh, int Nw, int tiles_w, int c_blocks, int64_t n_items, float max_cmp) {
-    extern __shared__ float staged[];                    // per wavefront: [2][n_slots + 1][KCB]
+    extern __shared__ __align__(16) float staged[];                    // per wavefront: [2][n_slots + 1][KCB]
     constexpr int SPAN = DX_TILE * HALVES;               // pixels of one wavefront
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int64_t item = (int64_t)blockIdx.x * (blockDim.x / kWave) + wave;

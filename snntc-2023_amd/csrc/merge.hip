@@ -117,7 +117,7 @@ merge_patches_kernel(const float* __restrict__ pix_z, const int32_t* __restrict_
                      float* __restrict__ sorted, int32_t* __restrict__ perm, int32_t* __restrict__ n_real,
                      int H, int W, int C, int Kh, int Kw, int Sh, int Sw, int Nh, int Nw, int TW, int tiles_w,
                      int stride, float max_cmp) {
-    extern __shared__ unsigned char lds_raw[];
+    extern __shared__ __align__(16) unsigned char lds_raw[];
     const int tile_cols = (TW - 1) * Sw + Kw;
     const int KhC = Kh * C;
     const int P = KhC * Kw;

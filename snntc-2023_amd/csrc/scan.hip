@@ -303,6 +303,23 @@ __device__ __forceinline__ void scan_chunk_vector(float& wsum, float& ysum, floa
                      : SNNTC_VSCAN_STATE : SNNTC_VSCAN_INPUTS : "vcc", "scc");
 }
 
+// Eight inputs added to the running sums of the lanes in `run`, no tests: what a wavefront does for
+// the chunks whose tests another wavefront of its workgroup evaluates (scan_lds_split_kernel).
+#define SNNTC_ACC_STEP(U)                                  \
+    "v_add_f32_e32 %[wsum], %[wsum], %[w" #U "]\n"         \
+    "v_fmac_f32_e32 %[ysum], %[x" #U "], %[w" #U "]\n"
+__device__ __forceinline__ void accumulate_chunk(float& wsum, float& ysum, int& kcnt, uint64_t run,
+                                                 const float (&x)[CHUNK], const float (&w)[CHUNK]) {
+    uint64_t saved_exec;
+    asm volatile("s_mov_b64 %[save], exec\n"
+                 "s_mov_b64 exec, %[run]\n" SNNTC_ACC_STEP(0) SNNTC_ACC_STEP(1) SNNTC_ACC_STEP(2) SNNTC_ACC_STEP(3)
+                     SNNTC_ACC_STEP(4) SNNTC_ACC_STEP(5) SNNTC_ACC_STEP(6) SNNTC_ACC_STEP(7)
+                 "v_add_u32_e32 %[kcnt], 8, %[kcnt]\n"
+                 "s_mov_b64 exec, %[save]\n"
+                 : [wsum] "+v"(wsum), [ysum] "+v"(ysum), [kcnt] "+v"(kcnt), [save] "=&s"(saved_exec)
+                 : SNNTC_SCAN_INPUTS("v", x));
+}
+
 // Copies columns [j0, j0 + COLS) of all `rows` rows of W[rows, J] into LDS as wl[row][COLS] (zeros
 // past column J).  Loads are issued in batches so that a small workgroup does not pay one memory
 // latency per element.
@@ -326,6 +343,40 @@ __device__ __forceinline__ void fill_weight_slice(float* __restrict__ wl, const 
                 const int idx = base + u * blockDim.x;
                 if (idx < rows * C4) reinterpret_cast<float4*>(wl)[idx] = v[u];
             }
+        }
+    } else if (j0 == 0 && J > 1 && J < COLS && (reinterpret_cast<uintptr_t>(w) & 15) == 0 && rows * J < (1 << 24)) {
+        // One slice holds every column (a 10-wide head): the source is a single run of rows*J floats.
+        // It is read as aligned float4 regardless of J, eight per thread in flight, and each value
+        // is dropped at [row][col]; the padding columns are zeroed first.
+        for (int idx = threadIdx.x; idx < n_fill / 4; idx += blockDim.x)
+            reinterpret_cast<float4*>(wl)[idx] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        __syncthreads();
+        constexpr int FILL = 8;
+        const int n = rows * J, n4 = n / 4;
+        const unsigned magic = 0xffffffffu / (unsigned)J + 1;      // e / J == umulhi(e, magic) for e < 2^24
+        for (int base = threadIdx.x; base < n4; base += FILL * blockDim.x) {
+            float4 v[FILL];
+#pragma unroll
+            for (int u = 0; u < FILL; ++u) {
+                const int idx = base + u * blockDim.x;
+                if (idx < n4) v[u] = reinterpret_cast<const float4*>(w)[idx];
+            }
+#pragma unroll
+            for (int u = 0; u < FILL; ++u) {
+                const int idx = base + u * blockDim.x;
+                if (idx < n4) {
+                    const float q[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const unsigned e = 4u * idx + t, r = __umulhi(e, magic);
+                        wl[r * COLS + (e - r * J)] = q[t];
+                    }
+                }
+            }
+        }
+        if ((int)threadIdx.x < n - 4 * n4) {
+            const unsigned e = 4u * n4 + threadIdx.x, r = __umulhi(e, magic);
+            wl[r * COLS + (e - r * J)] = w[e];
         }
     } else {
         constexpr int FILL = 16;
@@ -357,7 +408,7 @@ scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ pe
                 const int32_t* __restrict__ n_real, const float* __restrict__ w, float* __restrict__ y_out,
                 float* __restrict__ rcp_out, int32_t* __restrict__ k_out, int S, int I, int stride, int J,
                 int n_slices, int n_groups, NeuronParams np) {
-    extern __shared__ float wl[];                          // [I + bias][COLS]
+    extern __shared__ __align__(16) float wl[];                          // [I + bias][COLS]
     constexpr int SEGS = kWave / COLS;                     // segments per wavefront
     const int WAVES = blockDim.x / kWave;                  // 1..16, chosen by the launcher
     // slice-major over XCD-contiguous ids: the workgroups of one XCD share a few weight slices
@@ -471,6 +522,233 @@ scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ pe
     }
 }
 
+// Launches of a few dozen work items (the 10-wide head of a classifier): one item per workgroup,
+// its four wavefronts sharing the item instead of taking one each.  The running sums of a scan are
+// inherently sequential, its tests are not.  Wavefront 0 (the producer) only accumulates: two
+// instructions per input, and after every chunk of eight it leaves the sums in LDS and advances a
+// progress counter.  Wavefronts 1..3 (the testers) take every third chunk: they wait for the sums
+// before their chunk, recompute the fired state from them and the last input before the chunk, and
+// run the ordinary eight-step block with all its tests.  Each tester records the first close it
+// sees; the earliest of all is the scan's (a close found in a chunk is exact as long as no earlier
+// step closed, and an earlier close wins the minimum anyway).  The producer walks the trailing
+// inputs (fewer than eight) and supplies the result of a scan that never closes.
+// The item's sorted rows and row indices are copied into LDS first: at this pace chunks fetched
+// from memory a few ahead would not cover the memory latency.
+constexpr int SPLIT_WAVES = 4, SPLIT_TESTERS = SPLIT_WAVES - 1;
+constexpr int SPLIT_STATIC_LDS = 3 * SPLIT_WAVES * kWave * 4 + 16;
+constexpr int SPLIT_SPIN_LIMIT = 1 << 20;                  // polls of the progress counter before a tester gives up
+
+// dynamic LDS of the split kernel: weight slice, rows, sums after every chunk
+__host__ __device__ inline size_t split_lds_bytes(size_t slice_bytes, int segs, int stride) {
+    return slice_bytes + (size_t)segs * stride * 8 + (size_t)(stride / CHUNK) * 2 * kWave * 4;
+}
+
+template <int COLS, bool WANT_K>
+__global__ void __launch_bounds__(LOW_LATENCY_THREADS)
+scan_lds_split_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
+                      const int32_t* __restrict__ n_real, const float* __restrict__ w, float* __restrict__ y_out,
+                      float* __restrict__ rcp_out, int32_t* __restrict__ k_out, int S, int I, int stride, int J,
+                      int n_slices, int n_groups, NeuronParams np) {
+    extern __shared__ __align__(16) float wl[];                          // [I + bias][COLS], rows, sums
+    __shared__ int k_found[SPLIT_WAVES][kWave];
+    __shared__ float w_found[SPLIT_WAVES][kWave], y_found[SPLIT_WAVES][kWave];
+    __shared__ int progress;                               // chunks whose sums are in LDS
+    constexpr int SEGS = kWave / COLS;
+    constexpr int NONE = 0x7fffffff;
+    const int block = xcd_contiguous(blockIdx.x, gridDim.x);
+    const int slice = block / n_groups;
+    const int group = block - slice * n_groups;
+    const int j0 = slice * COLS;
+    const int rows = I + np.bias;
+    float* __restrict__ xrows = wl + rows * COLS;          // [SEGS][stride]
+    int32_t* __restrict__ prows = reinterpret_cast<int32_t*>(xrows + SEGS * stride);
+    float* __restrict__ sums = reinterpret_cast<float*>(prows + SEGS * stride);   // [chunk][wsum|ysum][lane]
+
+    fill_weight_slice<COLS>(wl, w, rows, J, j0);
+
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int sub = lane / COLS, col = lane - sub * COLS;
+    const int j = j0 + col;
+    const float* __restrict__ wcol = wl + col;
+    const int last_chunk = stride - CHUNK;
+
+    for (int item = group; item * SEGS < S; item += n_groups) {
+        const int seg0 = item * SEGS;
+        const int n_segs = S - seg0 < SEGS ? S - seg0 : SEGS;
+        {
+            const float4* __restrict__ gx = reinterpret_cast<const float4*>(sorted + (size_t)seg0 * stride);
+            const int4* __restrict__ gp = reinterpret_cast<const int4*>(perm + (size_t)seg0 * stride);
+            const int n4 = n_segs * stride / 4;            // stride is a multiple of 16 entries
+            for (int e = threadIdx.x; e < n4; e += blockDim.x) {
+                reinterpret_cast<float4*>(xrows)[e] = gx[e];
+                reinterpret_cast<int4*>(prows)[e] = gp[e];
+            }
+            if (threadIdx.x == 0) progress = 0;
+        }
+        __syncthreads();                                    // rows (and, the first time, the weights) are in place
+
+        const int seg_raw = seg0 + sub;
+        const bool live = seg_raw < S && j < J;
+        const int seg = seg_raw < S ? seg_raw : S - 1;
+        const int row = seg - seg0;                         // idle lanes shadow the item's last segment
+        const float* __restrict__ xs = xrows + row * stride;
+        const int32_t* __restrict__ pr = prows + row * stride;
+        const int n = live ? n_real[seg] : 0;
+        const int n_full = n & ~(CHUNK - 1);
+
+        float wsum = -np.theta, ysum = 0.0f, ya = 0.0f;
+        bool fired0 = false;
+        if (np.bias) {
+            const float wb = wcol[I * COLS];
+            wsum += wb;
+            ysum = np.biasvolt * wb;
+            ya = wsum < 0.0f ? -ysum : ysum;
+            fired0 = ya > fabsf(wsum) * np.biasvolt;
+        }
+        int k_close = NONE, consumed = 0;
+        bool fired_end = false, failed = false;
+
+        if (wave == 0) {
+            // ---- producer -----------------------------------------------------------------------
+            int kcnt = 0;
+            // chunk c is consumed from xp[c % NBUF] / wv[c % 2]; after it, chunk c+NBUF is read into its
+            // place and the weights of chunk c+2 are fetched
+            constexpr int NBUF = 4;
+            Chunk xp[NBUF];
+            float wv[2][CHUNK];
+#pragma unroll
+            for (int b = 0; b < NBUF; ++b) load_chunk_flat(xp[b], xs, pr, b * CHUNK <= last_chunk ? b * CHUNK : 0);
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int u = 0; u < CHUNK; ++u) wv[b][u] = wcol[xp[b].p[u] * COLS];
+            // chunks of this item (the longest row decides): the counter's final value
+            int n_full_max = n_full;
+#pragma unroll
+            for (int d = kWave / 2; d > 0; d >>= 1) n_full_max = max(n_full_max, __shfl_xor(n_full_max, d, kWave));
+            // Order inside a phase: accumulate, store the sums, then issue the LDS reads for later
+            // chunks.  The counter is moved two phases late and without waiting: LDS serves a
+            // wavefront's requests in order, and the weights the accumulation of chunk c consumes were
+            // requested right after the sums of chunk c-2 were stored -- once they have arrived,
+            // those sums are in place.
+            for (int k0 = 0;; k0 += NBUF * CHUNK) {
+                bool stop = false;
+#pragma unroll
+                for (int ph = 0; ph < NBUF; ++ph) {
+                    const int k = k0 + ph * CHUNK;
+                    const uint64_t run = __ballot(k < n_full);
+                    if (run == 0) { stop = true; break; }
+                    accumulate_chunk(wsum, ysum, kcnt, run, xp[ph % NBUF].x, wv[ph % 2]);
+                    asm volatile("" ::: "memory");
+                    if (k >= 2 * CHUNK) __hip_atomic_store(&progress, k / CHUNK - 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    float* __restrict__ out = sums + (size_t)(k / CHUNK) * 2 * kWave;
+                    out[lane] = wsum;
+                    out[kWave + lane] = ysum;
+                    asm volatile("" ::: "memory");
+                    const int kn = k + NBUF * CHUNK;
+                    load_chunk_flat(xp[ph % NBUF], xs, pr, kn <= last_chunk ? kn : 0);
+#pragma unroll
+                    for (int u = 0; u < CHUNK; ++u) wv[ph % 2][u] = wcol[xp[(ph + 2) % NBUF].p[u] * COLS];
+                }
+                if (stop) break;
+            }
+            // the last chunk's sums: wait for them, then let the counter reach its final value
+            __hip_atomic_store(&progress, (n_full_max + CHUNK - 1) / CHUNK, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+            // the trailing inputs, for a scan that no tester closes
+            if (live) {
+                LaneState st;
+                st.wsum = wsum; st.ysum = ysum; st.wa = fabsf(wsum);
+                st.ya = wsum < 0.0f ? -ysum : ysum;
+                st.fired = n_full > 0 ? st.ya > xs[n_full - 1] * st.wa : fired0;
+                bool open = true;
+                for (int k = n_full; k < n && open; ++k) {
+                    open = scan_step(st, xs[k], wcol[pr[k] * COLS]);
+                    if (open) ++kcnt;
+                }
+                if (!open) k_close = kcnt;
+                fired_end = st.fired;
+                wsum = st.wsum; ysum = st.ysum;
+            }
+            k_found[0][lane] = k_close;
+            w_found[0][lane] = wsum;
+            y_found[0][lane] = ysum;
+            consumed = kcnt;                                // all n inputs when nothing closed
+        } else {
+            // ---- tester: chunks wave-1, wave-1+3, ... ---------------------------------------------
+            uint64_t closed = 0;
+            float w_close = 0.0f, y_close = 0.0f;
+            float yg = fired0 ? ya : INFINITY;
+            Chunk cur, nxt;
+            float wcur[CHUNK];
+            int c = wave - 1;
+            load_chunk_flat(cur, xs, pr, c * CHUNK <= last_chunk ? c * CHUNK : 0);
+#pragma unroll
+            for (int u = 0; u < CHUNK; ++u) wcur[u] = wcol[cur.p[u] * COLS];
+            for (;; c += SPLIT_TESTERS) {
+                const int k = c * CHUNK;
+                const uint64_t run = __ballot(k < n_full) & ~closed;
+                if (run == 0) break;                        // every lane closed here or past its inputs
+                const int kn = k + SPLIT_TESTERS * CHUNK;
+                load_chunk_flat(nxt, xs, pr, kn <= last_chunk ? kn : 0);
+                if (c > 0) {
+                    // bounded wait: if the sums never arrive the tester goes on with what is there and
+                    // the result is marked invalid (no early exit: every wavefront reaches the barriers)
+                    int spins = 0;
+                    while (__builtin_amdgcn_readfirstlane(__hip_atomic_load(&progress, __ATOMIC_ACQUIRE,
+                                                                            __HIP_MEMORY_SCOPE_WORKGROUP)) < c &&
+                           spins < SPLIT_SPIN_LIMIT) {
+                        __builtin_amdgcn_s_sleep(1);
+                        ++spins;
+                    }
+                    failed |= spins >= SPLIT_SPIN_LIMIT;
+                    const float* __restrict__ in = sums + (size_t)(c - 1) * 2 * kWave;
+                    wsum = in[lane];
+                    ysum = in[kWave + lane];
+                    ya = wsum < 0.0f ? -ysum : ysum;        // fired state after input k-1, from the sums
+                    yg = ya > xs[k - 1] * fabsf(wsum) ? ya : INFINITY;
+                }
+                const uint64_t before = closed;
+                int kc = k;
+                scan_chunk_vector<true>(wsum, ysum, ya, yg, kc, closed, run, cur.x, wcur);
+                if (((closed & ~before) >> lane) & 1) { k_close = kc; w_close = wsum; y_close = ysum; }
+#pragma unroll
+                for (int u = 0; u < CHUNK; ++u) wcur[u] = wcol[nxt.p[u] * COLS];
+                cur = nxt;
+            }
+            k_found[wave][lane] = failed ? -1 : k_close;    // -1 poisons the result below
+            w_found[wave][lane] = w_close;
+            y_found[wave][lane] = y_close;
+        }
+        __syncthreads();
+        if (wave == 0 && live) {
+            int best = 0, kb = k_found[0][lane];
+            bool bad = false;
+#pragma unroll
+            for (int v = 1; v < SPLIT_WAVES; ++v) {
+                const int kv = k_found[v][lane];
+                bad |= kv < 0;
+                if (kv < kb) { kb = kv; best = v; }
+            }
+            // no close anywhere: the producer went through all n inputs, fired_end is the scan's
+            const bool fired = kb != NONE || fired_end;
+            const float ws = w_found[best][lane], ys = y_found[best][lane];
+            float y = np.max_time, r = 0.0f;
+            if (fired) {
+                r = 1.0f / ws;
+                y = ys * r;
+                if (y >= np.max_time) { y = np.max_time; r = 0.0f; }
+            }
+            if (bad) y = r = __builtin_nanf("");            // a tester gave up waiting: make it visible
+            const size_t o = (size_t)seg * J + j;
+            y_out[o] = y;
+            rcp_out[o] = r;
+            if (WANT_K) k_out[o] = (fired && r != 0.0f) ? (kb != NONE ? kb : consumed) : -1;
+        }
+        __syncthreads();                                    // LDS is reused by the next item
+    }
+}
+
 // CH (2 or 4) neurons per lane.  Same workgroup layout as scan_lds_kernel, but a lane owns CH
 // adjacent columns of its segment: one row address and one 8- or 16-byte LDS read serve CH scans,
 // a wavefront covers 64*CH/COLS segments, and the (x, row) chunks are fetched once for all of
@@ -495,7 +773,7 @@ scan_lds_multi_kernel(const float* __restrict__ sorted, const int32_t* __restric
                       const int32_t* __restrict__ n_real, const float* __restrict__ w, float* __restrict__ y_out,
                       float* __restrict__ rcp_out, int32_t* __restrict__ k_out, int S, int I, int stride, int J,
                       int n_slices, int n_groups, NeuronParams np) {
-    extern __shared__ float wl[];                          // [I + bias][COLS]
+    extern __shared__ __align__(16) float wl[];                          // [I + bias][COLS]
     constexpr int LANES = COLS / CH;                       // lanes per segment
     constexpr int SEGS = kWave / LANES;                    // segments per wavefront
     const int WAVES = blockDim.x / kWave;
@@ -659,35 +937,44 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     const bool multi = !low_latency && multi_items * n_slices >= (int64_t)cus * 4 * 4;
     const int64_t work_items = multi ? multi_items : items;
     if (multi && CH == 4) WAVES = MULTI_SCAN_THREADS / kWave;
+    // Fewer items than CUs: a whole workgroup per item, its wavefronts sharing the item's tests.
+    const size_t split_lds = split_lds_bytes(lds_bytes, SEGS, (int)stride);
+    const bool split = low_latency && items * n_slices <= (int64_t)cus && I >= 2 * CHUNK * SPLIT_WAVES &&
+                       split_lds + SPLIT_STATIC_LDS <= (size_t)LDS_SCAN_BYTES;
+    if (split) WAVES = 1;                                   // items per workgroup pass
     // resident workgroups per CU: split the segments so that slices x groups covers the chip
     const int wgs_per_cu = lds_bytes * 2 <= (size_t)LDS_SCAN_BYTES ? 2 : 1;
     int64_t n_groups = ((int64_t)cus * wgs_per_cu + n_slices - 1) / n_slices;
     const int64_t max_groups = (work_items + WAVES - 1) / WAVES;
     if (n_groups > max_groups) n_groups = max_groups;
     if (n_groups < 1) n_groups = 1;
-    auto kern_k = low_latency ? scan_lds_kernel<COLS, true, true>
+    auto kern_k = split ? scan_lds_split_kernel<COLS, true>
+                  : low_latency ? scan_lds_kernel<COLS, true, true>
                   : multi ? scan_lds_multi_kernel<COLS, CH, true> : scan_lds_kernel<COLS, true, false>;
-    auto kern = low_latency ? scan_lds_kernel<COLS, false, true>
+    auto kern = split ? scan_lds_split_kernel<COLS, false>
+                : low_latency ? scan_lds_kernel<COLS, false, true>
                 : multi ? scan_lds_multi_kernel<COLS, CH, false> : scan_lds_kernel<COLS, false, false>;
     // raise the dynamic-LDS limit of both instantiations once (not per launch: the call is not
     // allowed while a stream is being captured into a graph)
-    static std::atomic<bool> lds_limit_raised[kMaxDevices][3];
-    const int variant = low_latency ? 1 : (multi ? 2 : 0);
+    static std::atomic<bool> lds_limit_raised[kMaxDevices][4];
+    const int variant = split ? 3 : low_latency ? 1 : (multi ? 2 : 0);
+    const int lds_limit = split ? LDS_SCAN_BYTES - SPLIT_STATIC_LDS : LDS_SCAN_BYTES;
     if (!lds_limit_raised[dev][variant].load(std::memory_order_acquire)) {
         SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern_k),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS_SCAN_BYTES));
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_limit));
         SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS_SCAN_BYTES));
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_limit));
         lds_limit_raised[dev][variant].store(true, std::memory_order_release);
     }
-    dim3 grid((unsigned)(n_slices * n_groups)), block((unsigned)(WAVES * kWave));
+    dim3 grid((unsigned)(n_slices * n_groups)), block((unsigned)(split ? LOW_LATENCY_THREADS : WAVES * kWave));
     {
         KernelTimerScope timer_("scan", stream);
+        const size_t dyn_lds = split ? split_lds : lds_bytes;
         if (causal_k)
-            hipLaunchKernelGGL(kern_k, grid, block, lds_bytes, stream, sorted, perm, n_real, w, y, rcp, causal_k,
+            hipLaunchKernelGGL(kern_k, grid, block, dyn_lds, stream, sorted, perm, n_real, w, y, rcp, causal_k,
                                (int)S, (int)I, (int)stride, (int)J, n_slices, (int)n_groups, np);
         else
-            hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, sorted, perm, n_real, w, y, rcp, causal_k,
+            hipLaunchKernelGGL(kern, grid, block, dyn_lds, stream, sorted, perm, n_real, w, y, rcp, causal_k,
                                (int)S, (int)I, (int)stride, (int)J, n_slices, (int)n_groups, np);
     }
     SNNTC_HIP_CHECK(hipGetLastError());

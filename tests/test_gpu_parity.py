@@ -204,6 +204,43 @@ def test_loss_kernel_against_closed_form(B, J):
     assert np.all(np.abs(T.grad.cpu().numpy() - 3.0 * want_g) <= 3e-6 / B + 3e-6 * np.abs(want_g))
 
 
+HEAD_CASES = [
+    # seed, B, I, J, bias: classifier heads, i.e. fewer (sample group, column slice) work items than CUs
+    (20, 70, 800, 10, True),       # batch not a multiple of the segments a wavefront holds
+    (21, 9, 512, 10, False),
+    (22, 33, 2048, 5, True),
+    (23, 130, 264, 16, True),      # J equal to the slice width (vector weight copy)
+    (24, 6, 72, 3, True),
+]
+
+
+@pytest.mark.parametrize("seed,B,I,J,bias", HEAD_CASES)
+def test_dense_head_forward_bit_exact(seed, B, I, J, bias):
+    """Layers with a handful of outputs, where the wavefronts of a workgroup share one scan.  Rows
+    differ in their number of real inputs (some inputs lie above MAX-0.1, a few rows have none at
+    all), weights of both signs make neurons fire and stop firing again, and some neurons never fire:
+    y, 1/S and the causal-set sizes must equal the oracle bit for bit, with and without the extra outputs."""
+    import snntc_amd as snn
+    rng = np.random.default_rng(seed)
+    x = np.exp(2.0 * rng.random((B, I))).astype(np.float32)
+    late = rng.random((B, I)) < rng.random((B, 1)) * 0.5          # per-row share of never-arriving inputs
+    x[late] = np.float32(1e5)
+    x[0] = np.float32(1e5)                                         # a row without any real input
+    rows = I + (1 if bias else 0)
+    w = ((3.0 / I) + rng.standard_normal((rows, J)) * np.sqrt(2.0 / I)).astype(np.float32)
+    w[:, 0] = -np.abs(w[:, 0])                                     # a neuron that can never fire
+    p = capi.fc_params(1.0 if bias else 0.0)
+    ref_out, ref_k, _, _ = capi.fc_forward_dev(x, w, p, want_aux=True)
+    out, _, _, ck = snn.snnfc(t(x), t(w), p, return_aux=True)
+    out2 = snn.snnfc(t(x), t(w), p)
+    torch.cuda.synchronize()
+    out, ck, out2 = out.cpu().numpy(), ck.cpu().numpy(), out2.cpu().numpy()
+    assert np.array_equal(ck, ref_k), f"causal-set sizes differ at {np.argwhere(ck != ref_k)[:5]}"
+    assert np.array_equal(out.view(np.uint32), ref_out.view(np.uint32)), "y / 1/S not bit-exact"
+    assert np.array_equal(out2.view(np.uint32), ref_out.view(np.uint32)), "plain entry point not bit-exact"
+    assert np.all(ref_k[:, 0] == -1) and (ref_k >= 0).any(), "the case should hold firing and silent neurons"
+
+
 def test_sgd_update_matches_numpy():
     """w -= lr*dw over tensors of awkward sizes (empty, shorter than a vector, unaligned views, more
     than one table of 32): within one rounding of the float32 formula, and nothing else is touched."""
