@@ -34,10 +34,11 @@ for _p in (ROOT, os.path.join(ROOT, "snntc-2023_amd")):
 # KiB per dispatch, FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0 as the plain 256 MiB device copies of
 # --calibration-copies read on those counters); summary in profiles/scan_hbm_traffic_pmc.txt.  Counters cannot
 # be read from inside this script, so the figures are carried here per workload (mlp: mean of its three launches).
-MEASURED_SCAN_TRAFFIC_BYTES = {"mlp": 24.1e6, "conv": 341.1e6}
+MEASURED_SCAN_TRAFFIC_BYTES = {"mlp": 12.7e6, "conv": 341.3e6}
 # Share of the scan kernel's clocks in which the vector ALUs issue (SQ_ACTIVE_INST_VALU * 4 / SIMDs / clocks,
-# profiles/valu_utilisation_pmc.txt); the counter ratio saturates slightly above 1.
-MEASURED_SCAN_VALU_BUSY = {"mlp": 0.62, "conv": 1.0}
+# profiles/valu_utilisation_pmc.txt; mlp: mean of its three launches, 0.63 for the two 800-wide layers and 0.06 for
+# the 10-wide head); the counter ratio saturates slightly above 1.
+MEASURED_SCAN_VALU_BUSY = {"mlp": 0.44, "conv": 1.0}
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 VALU_PEAK_TFLOPS = 157.3     # MI355X fp32 vector peak (256 CU x 256 flop/clk x 2.4 GHz)
