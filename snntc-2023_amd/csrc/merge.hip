@@ -274,10 +274,17 @@ size_t merge_lds_bytes(int C, int Kh, int Kw, int Sw, int TW) {
 }
 
 // Patches per tile: as many as fit in 52 KB of LDS (so three workgroups share a CU), at
-// most 16, never more than the row holds.
+// most 16, never more than the row holds.  Layers with so many channels that not even two
+// patches fit in 52 KB take what fits in MERGE_LDS_CAP (one workgroup per CU).
+constexpr size_t MERGE_LDS_CAP = 128 * 1024;
 int merge_tile_width(const ConvGeom& g) {
-    int tw = g.Nw < 16 ? (int)g.Nw : 16;
+    const int tw_max = g.Nw < 16 ? (int)g.Nw : 16;
+    int tw = tw_max;
     while (tw > 1 && merge_lds_bytes((int)g.C, (int)g.Kh, (int)g.Kw, (int)g.Sw, tw) > 52 * 1024) --tw;
+    if (tw < 2) {
+        tw = tw_max;
+        while (tw > 1 && merge_lds_bytes((int)g.C, (int)g.Kh, (int)g.Kw, (int)g.Sw, tw) > MERGE_LDS_CAP) --tw;
+    }
     return tw;
 }
 
@@ -288,7 +295,7 @@ int merge_tile_width(const ConvGeom& g) {
 bool merge_sort_supported(const ConvGeom& g) {
     if (g.C < 32 || g.C % NB != 0 || g.C > 4096 || g.Kh * g.Kw < 2 || g.Kh > 255) return false;
     const int tw = merge_tile_width(g);
-    return merge_lds_bytes((int)g.C, (int)g.Kh, (int)g.Kw, (int)g.Sw, tw) <= 96 * 1024 && tw >= 2;
+    return merge_lds_bytes((int)g.C, (int)g.Kh, (int)g.Kw, (int)g.Sw, tw) <= MERGE_LDS_CAP && tw >= 2;
 }
 
 int launch_merge_patches(const float* pix_z, const int32_t* pix_c, int64_t Cs, float* sorted, int32_t* perm,
@@ -310,7 +317,7 @@ int launch_merge_patches(const float* pix_z, const int32_t* pix_c, int64_t Cs, f
     if (dev < 0 || dev >= kMaxDevices) return fail(SNNTC_ERR_UNSUPPORTED, "patch merge: device index %d not supported", dev);
     if (!lds_limit_raised[dev][eb].load(std::memory_order_acquire)) {
         SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)MERGE_LDS_CAP));
         lds_limit_raised[dev][eb].store(true, std::memory_order_release);
     }
     {
