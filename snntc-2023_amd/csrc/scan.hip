@@ -923,12 +923,20 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     constexpr int SEGS = kWave / COLS;
     const int n_slices = (int)((J + COLS - 1) / COLS);
     const int64_t items = (S + SEGS - 1) / SEGS;
-    // A launch that cannot put more than two wavefronts on every SIMD runs the low-latency
-    // instantiation, in workgroups of four wavefronts (one per SIMD of a CU, and four times the
-    // threads of a single wavefront for copying the weight slice): the same work packed into a
-    // few full workgroups would leave most of the chip idle.
-    const bool low_latency = items * n_slices <= (int64_t)cus * 4 * 2;
-    int WAVES = (low_latency ? LOW_LATENCY_THREADS : LDS_SCAN_THREADS) / kWave;
+    // workgroups the chip holds at once (two per CU when two weight slices fit in its LDS)
+    const int wgs_per_cu = lds_bytes * 2 <= (size_t)LDS_SCAN_BYTES ? 2 : 1;
+    const int64_t capacity = (int64_t)cus * wgs_per_cu;
+    // A launch whose work items all find a wavefront of their own in workgroups of four (one
+    // wavefront per SIMD of a CU, and four times the threads of a single wavefront for copying the
+    // weight slice) runs the low-latency instantiation: the same work packed into a few full
+    // workgroups would leave most of the chip idle.  Larger launches get the workgroup size, 4 to
+    // 16 wavefronts, that spreads them over all CUs in one go.
+    const bool low_latency = (items + 3) / 4 * n_slices <= capacity;
+    int WAVES = LOW_LATENCY_THREADS / kWave;
+    if (!low_latency) {
+        const int64_t per_wg = (items * n_slices + capacity - 1) / capacity;
+        WAVES = (int)(per_wg >= 16 ? 16 : (per_wg + 3) / 4 * 4);
+    }
     // With at least four wavefronts of multi-neuron lanes for every SIMD, CH neurons per lane (CH times
     // the segments per wavefront) is the cheaper instruction stream; in between, one neuron per
     // lane in 16-wave workgroups balances better.
@@ -936,15 +944,14 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     const int64_t multi_items = (S + CH * SEGS - 1) / (CH * SEGS);
     const bool multi = !low_latency && multi_items * n_slices >= (int64_t)cus * 4 * 4;
     const int64_t work_items = multi ? multi_items : items;
-    if (multi && CH == 4) WAVES = MULTI_SCAN_THREADS / kWave;
+    if (multi) WAVES = (CH == 4 ? MULTI_SCAN_THREADS : LDS_SCAN_THREADS) / kWave;
     // Fewer items than CUs: a whole workgroup per item, its wavefronts sharing the item's tests.
     const size_t split_lds = split_lds_bytes(lds_bytes, SEGS, (int)stride);
     const bool split = low_latency && items * n_slices <= (int64_t)cus && I >= 2 * CHUNK * SPLIT_WAVES &&
                        split_lds + SPLIT_STATIC_LDS <= (size_t)LDS_SCAN_BYTES;
     if (split) WAVES = 1;                                   // items per workgroup pass
-    // resident workgroups per CU: split the segments so that slices x groups covers the chip
-    const int wgs_per_cu = lds_bytes * 2 <= (size_t)LDS_SCAN_BYTES ? 2 : 1;
-    int64_t n_groups = ((int64_t)cus * wgs_per_cu + n_slices - 1) / n_slices;
+    // split the segments so that slices x groups covers the chip without a second round of workgroups
+    int64_t n_groups = capacity / n_slices;
     const int64_t max_groups = (work_items + WAVES - 1) / WAVES;
     if (n_groups > max_groups) n_groups = max_groups;
     if (n_groups < 1) n_groups = 1;
