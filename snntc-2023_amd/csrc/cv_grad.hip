@@ -64,11 +64,16 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KCB ==
 cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restrict__ w,
                           const float* __restrict__ upm, const float* __restrict__ ym,
                           float* __restrict__ dxpad, int H, int W, int C, int Kc, int Kh, int Kw, int Sh, int Sw,
-                          int Nh, int Nw, int tiles_w, int c_blocks, int64_t n_items, float max_cmp) {
+                          int Nh, int Nw, int tiles_w, int c_blocks, int64_t n_items, float max_cmp, int ksplit) {
     extern __shared__ __align__(16) float staged[];                    // per wavefront: [2][n_slots + 1][KCB]
+    __shared__ float partial[3][DX_TILE][kWave];         // ksplit = 4: sums of wavefronts 1..3
     constexpr int SPAN = DX_TILE * HALVES;               // pixels of one wavefront
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    const int64_t item = (int64_t)blockIdx.x * (blockDim.x / kWave) + wave;
+    // ksplit = 1: a tile per wavefront.  ksplit = 4 (layers with few tiles and many output channels):
+    // a tile per workgroup, its wavefronts take a quarter of the output channels each and their
+    // sums are added in wavefront order.
+    const int64_t item = ksplit == 1 ? (int64_t)blockIdx.x * (blockDim.x / kWave) + wave : (int64_t)blockIdx.x;
+    const int ks = ksplit == 1 ? 0 : wave;
     if (item >= n_items) return;
     const int lane = threadIdx.x % kWave;
     const int half = HALVES == 2 ? lane / 32 : 0;
@@ -108,7 +113,8 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
             const int nh = hh / Sh;
             if (nh >= Nh) continue;
             const size_t row0 = (size_t)(a * Nh + nh) * Nw;
-            for (int kc0 = 0; kc0 < Kc; kc0 += KCB) {
+            const int kc_share = Kc / ksplit;
+            for (int kc0 = ks * kc_share; kc0 < (ks + 1) * kc_share; kc0 += KCB) {
                 // stage the patch row: slots whose patch does not exist are never read
                 __builtin_amdgcn_wave_barrier();
                 // loads of STAGE slots are issued together: one slot at a time would cost a memory
@@ -181,6 +187,17 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
                 }
             }
         }
+    }
+    if (ksplit > 1) {                                     // block-uniform: all four wavefronts hold the same tile
+        if (ks > 0) {
+#pragma unroll
+            for (int t = 0; t < DX_TILE; ++t) partial[ks - 1][t][lane] = acc[t];
+        }
+        __syncthreads();
+        if (ks > 0) return;
+#pragma unroll
+        for (int t = 0; t < DX_TILE; ++t)
+            acc[t] = ((acc[t] + partial[0][t][lane]) + partial[1][t][lane]) + partial[2][t][lane];
     }
     if (lane_ok) {
         float* __restrict__ orow = dxpad + ((size_t)(a * H + h) * W) * C + c;
@@ -402,7 +419,8 @@ cv_grad_weight_narrow_kernel(const float* __restrict__ xpad, const float* __rest
 
 bool cv_grad_input_chan_supported(const ConvGeom& g) {
     // the staging buffer (four wavefronts, up to 2 * TILE + Kw patches) has to fit the default 64 KB of LDS
-    return g.C >= 32 && g.Kc % 16 == 0 && (2 * DX_TILE + g.Kw) * 64 * 8 * 4 <= 64 * 1024;
+    // (plus the 6 KB the output-channel split keeps for its partial sums)
+    return g.C >= 32 && g.Kc % 16 == 0 && (2 * DX_TILE + g.Kw) * 64 * 8 * 4 + 3 * DX_TILE * kWave * 4 <= 64 * 1024;
 }
 
 int launch_cv_grad_input_chan(const float* xpad, const float* w, const float* upm, const float* ym,
@@ -412,13 +430,17 @@ int launch_cv_grad_input_chan(const float* xpad, const float* w, const float* up
     const int tiles_w = (int)((g.W + span - 1) / span);
     const int c_blocks = halves == 2 ? 1 : (int)((g.C + kWave - 1) / kWave);
     const int64_t n_items = g.B * g.H * tiles_w * c_blocks;
-    const int64_t blocks = (n_items + 3) / 4;
+    const int kcb = g.Kc % 64 == 0 ? 64 : (g.Kc % 32 == 0 ? 32 : 16);
+    // small images with at least four chunks of output channels: split the channels over the
+    // wavefronts of a workgroup.  Decided by the layer's geometry alone, never by the batch: the
+    // order of the additions, and with it the last bits of dX, must not depend on the batch size.
+    const int ksplit = (halves == 1 && g.H * tiles_w * c_blocks <= 160 && g.Kc % (4 * kcb) == 0) ? 4 : 1;
+    const int64_t blocks = ksplit == 4 ? n_items : (n_items + 3) / 4;
     if (blocks > 0x7fffffffLL) return fail(SNNTC_ERR_TOO_LARGE, "conv backward: grid too large");
     dim3 grid((unsigned)blocks), block(256);
-    const int kcb = g.Kc % 64 == 0 ? 64 : (g.Kc % 32 == 0 ? 32 : 16);
     const size_t lds = (size_t)4 * 2 * (span + g.Kw) * kcb * sizeof(float);
     void (*kern)(const float*, const float*, const float*, const float*, float*, int, int, int, int, int, int, int,
-                 int, int, int, int, int, int64_t, float);
+                 int, int, int, int, int, int64_t, float, int);
     if (halves == 2)
         kern = kcb == 64 ? cv_grad_input_chan_kernel<64, 2> : kcb == 32 ? cv_grad_input_chan_kernel<32, 2>
                                                                          : cv_grad_input_chan_kernel<16, 2>;
@@ -429,7 +451,7 @@ int launch_cv_grad_input_chan(const float* xpad, const float* w, const float* up
         KernelTimerScope timer_("cv_grad_input", stream);
         hipLaunchKernelGGL(kern, grid, block, lds, stream, xpad, w, upm, ym, dxpad, (int)g.H, (int)g.W, (int)g.C,
                            (int)g.Kc, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.Nh, (int)g.Nw, tiles_w,
-                           c_blocks, n_items, np.max_cmp);
+                           c_blocks, n_items, np.max_cmp, ksplit);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
