@@ -35,6 +35,9 @@ sort_segments_kernel(SegmentSource src, float* __restrict__ sorted, int32_t* __r
     constexpr int NPAD = EPT * G;
     constexpr int SEGS = BLOCK / G;
     constexpr bool CROSS_WAVE = G > kWave;
+    // the exchange buffer below belongs to the block, not to a segment: a segment that spans several
+    // wavefronts must have the block to itself
+    static_assert(!CROSS_WAVE || SEGS == 1, "cross-wavefront segments need BLOCK == G");
     __shared__ u64 xchg[CROSS_WAVE ? NPAD : 1];
     __shared__ int wave_count[CROSS_WAVE ? G / kWave : 1];
 
