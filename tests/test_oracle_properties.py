@@ -105,3 +105,67 @@ def test_lowering_max_spike_time_only_removes_late_inputs(cut, seed, B, I, J, bi
     assert np.array_equal(y_cut[inside].view(np.uint32), y_ref[inside].view(np.uint32))
     assert np.array_equal(r_cut[inside].view(np.uint32), r_ref[inside].view(np.uint32))
     assert np.all(y_cut[~inside] == cutf) and np.all(r_cut[~inside] == 0) and np.all(k_cut[~inside] == -1)
+
+
+# ---------------------------------------------------------------------------------------------
+# backward
+# ---------------------------------------------------------------------------------------------
+def _backward(g, x, w, bias, out):
+    p = capi.fc_params(1.0 if bias else 0.0)
+    return capi.fc_backward_dev(g, x, w, p, out)
+
+
+def _fwd_out(x, w, bias):
+    return capi.fc_forward_dev(x, w, capi.fc_params(1.0 if bias else 0.0))
+
+
+@settings(max_examples=40, deadline=None)
+@given(m=st.integers(-3, 3), **CASES)
+def test_gradients_are_linear_in_the_upstream_gradient(m, seed, B, I, J, bias):
+    x, w = _case(seed, B, I, J, bias)
+    out = _fwd_out(x, w, bias)
+    g = np.zeros((2 * B, J), np.float32)
+    g[:B] = np.random.default_rng(seed + 3).standard_normal((B, J))
+    c = np.float32(2.0 ** m)
+    dx0, dw0, _ = _backward(g, x, w, bias, out)
+    dx1, dw1, _ = _backward(g * c, x, w, bias, out)
+    assert np.array_equal((dx0 * c).view(np.uint32), dx1.view(np.uint32))
+    assert np.array_equal((dw0 * c).view(np.uint32), dw1.view(np.uint32))
+
+
+@settings(max_examples=40, deadline=None)
+@given(**CASES)
+def test_samples_are_independent_in_dx_and_add_up_in_dw(seed, B, I, J, bias):
+    x, w = _case(seed, B + 1, I, J, bias)
+    Bt = B + 1
+    out = _fwd_out(x, w, bias)
+    g = np.zeros((2 * Bt, J), np.float32)
+    g[:Bt] = np.random.default_rng(seed + 4).standard_normal((Bt, J))
+    dx, dw, _ = _backward(g, x, w, bias, out)
+    dw_sum = np.zeros_like(dw, dtype=np.float64)
+    mag = np.zeros_like(dw, dtype=np.float64)
+    for b in range(Bt):
+        o1 = np.stack((out[b], out[Bt + b]))
+        g1 = np.stack((g[b], g[Bt + b]))
+        dx1, dw1, _ = _backward(g1, x[b:b + 1], w, bias, o1)
+        assert np.array_equal(dx1[0].view(np.uint32), dx[b].view(np.uint32))       # no other sample enters
+        dw_sum += dw1
+        mag += np.abs(dw1)
+    assert np.all(np.abs(dw - dw_sum) <= 1e-6 * np.maximum(mag, 1e-30) * Bt)       # fp32 sum over the batch
+
+
+@settings(max_examples=40, deadline=None)
+@given(extra=st.integers(1, 4), **CASES)
+def test_inputs_that_never_arrive_get_no_gradient(extra, seed, B, I, J, bias):
+    x, w = _case(seed, B, I, J, bias)
+    rng = np.random.default_rng(seed + 5)
+    x2 = np.concatenate([x, np.full((B, extra), 1e5, np.float32)], axis=1)
+    w2 = np.concatenate([w[:I], rng.standard_normal((extra, J)).astype(np.float32), w[I:]], axis=0)
+    out = _fwd_out(x2, w2, bias)
+    g = np.zeros((2 * B, J), np.float32)
+    g[:B] = rng.standard_normal((B, J))
+    dx, dw, _ = _backward(g, x2, w2, bias, out)
+    assert np.all(dx[:, I:I + extra] == 0) and np.all(dw[I:I + extra] == 0)
+    dx0, dw0, _ = _backward(g, x, w, bias, _fwd_out(x, w, bias))
+    assert np.array_equal(dx[:, :I].view(np.uint32), dx0.view(np.uint32))
+    assert np.array_equal(dw[:I].view(np.uint32), dw0[:I].view(np.uint32))
