@@ -221,7 +221,7 @@ __global__ void __launch_bounds__(256)
 cv_grad_weight_wide_kernel(const float* __restrict__ xpad, const float* __restrict__ upm,
                            const float* __restrict__ ym, float* __restrict__ dst, int S, int Kc, int rows,
                            int seg_per_slice, int H, int W, int C, int Kw, int Sh, int Sw, int Nh, int Nw,
-                           int bias_row, float biasvolt, int s_safe) {
+                           int bias_row, float biasvolt, int s_safe, float neg_s, float post) {
     __shared__ float red[3][DWW_RI + 1][kWave];
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -249,48 +249,40 @@ cv_grad_weight_wide_kernel(const float* __restrict__ xpad, const float* __restri
 
     if (s_lo < s_hi) {
         const int per_img = Nh * Nw;
-        int a = s_lo / per_img;
-        int r2 = s_lo - a * per_img;
+        const int a = s_lo / per_img;
+        const int r2 = s_lo - a * per_img;
         int nh = r2 / Nw, nw = r2 - nh * Nw;
-        const float* __restrict__ ycol = ym + jc;
-        const float* __restrict__ ucol = upm + jc;
-        if (FULL || n_rows == DWW_RI) {
-            for (int s = s_lo; s < s_hi; ++s) {
-                const float* __restrict__ xb =
-                    xpad + ((size_t)(a * H + nh * Sh + kh) * W + (size_t)(nw * Sw)) * C + q0;
-                const float yv = ycol[(size_t)s * Kc];
-                const float uv = ucol[(size_t)s * Kc];
+        // the block's first input of patch s_lo; the step to the next patch is one add, plus one more
+        // at the end of an output row and of an image
+        const float* xb = xpad + ((size_t)(a * H + nh * Sh + kh) * W + (size_t)(nw * Sw)) * C + q0;
+        const ptrdiff_t step_w = (ptrdiff_t)Sw * C;
+        const ptrdiff_t wrap_w = ((ptrdiff_t)Sh * W - (ptrdiff_t)Nw * Sw) * C;
+        const ptrdiff_t wrap_h = ((ptrdiff_t)H - (ptrdiff_t)Nh * Sh) * W * C;
+        // y and up of the next patch are requested before the current one is worked on
+        const float* yp = ym + (size_t)s_lo * Kc + jc;
+        const float* up = upm + (size_t)s_lo * Kc + jc;
+        float y_next = *yp, u_next = *up;
+        const int s_fast = (FULL || n_rows == DWW_RI) ? s_hi : min(s_hi, s_safe);
+        for (int s = s_lo; s < s_hi; ++s) {
+            const float yv = y_next * -neg_s, uv = u_next;
+            if (s + 1 < s_hi) { yp += Kc; up += Kc; }
+            y_next = *yp; u_next = *up;
+            if (FULL || s < s_fast) {
 #pragma unroll
-                for (int r = 0; r < DWW_RI; ++r) acc[r] = __fmaf_rn(fminf(xb[r] - yv, 0.0f), uv, acc[r]);
-                if (with_bias) acc_bias = __fmaf_rn(fminf(biasvolt - yv, 0.0f), uv, acc_bias);
-                if (++nw == Nw) { nw = 0; if (++nh == Nh) { nh = 0; ++a; } }
-            }
-        } else {
-            // a block at the end of a kernel row fetches past its rows (the values are discarded) ...
-            int s = s_lo;
-            const int s_fast = min(s_hi, s_safe);
-            for (; s < s_fast; ++s) {
-                const float* __restrict__ xb =
-                    xpad + ((size_t)(a * H + nh * Sh + kh) * W + (size_t)(nw * Sw)) * C + q0;
-                const float yv = ycol[(size_t)s * Kc];
-                const float uv = ucol[(size_t)s * Kc];
-#pragma unroll
-                for (int r = 0; r < DWW_RI; ++r) acc[r] = __fmaf_rn(fminf(xb[r] - yv, 0.0f), uv, acc[r]);
-                if (with_bias) acc_bias = __fmaf_rn(fminf(biasvolt - yv, 0.0f), uv, acc_bias);
-                if (++nw == Nw) { nw = 0; if (++nh == Nh) { nh = 0; ++a; } }
-            }
-            // ... except for the last few patches of the tensor, where that fetch could leave it: there
-            // the unused rows re-read the block's last row
-            for (; s < s_hi; ++s) {
-                const float* __restrict__ xb =
-                    xpad + ((size_t)(a * H + nh * Sh + kh) * W + (size_t)(nw * Sw)) * C + q0;
-                const float yv = ycol[(size_t)s * Kc];
-                const float uv = ucol[(size_t)s * Kc];
+                for (int r = 0; r < DWW_RI; ++r) acc[r] = __fmaf_rn(scaled_lead(xb[r], neg_s, yv), uv, acc[r]);
+            } else {
+                // A block at the end of a kernel row fetches past its rows (the values are discarded),
+                // except for the last few patches of the tensor, where that fetch could leave it: there
+                // the unused rows re-read the block's last row.
 #pragma unroll
                 for (int r = 0; r < DWW_RI; ++r)
-                    acc[r] = __fmaf_rn(fminf(xb[min(r, n_rows - 1)] - yv, 0.0f), uv, acc[r]);
-                if (with_bias) acc_bias = __fmaf_rn(fminf(biasvolt - yv, 0.0f), uv, acc_bias);
-                if (++nw == Nw) { nw = 0; if (++nh == Nh) { nh = 0; ++a; } }
+                    acc[r] = __fmaf_rn(scaled_lead(xb[min(r, n_rows - 1)], neg_s, yv), uv, acc[r]);
+            }
+            if (with_bias) acc_bias = __fmaf_rn(scaled_lead(biasvolt, neg_s, yv), uv, acc_bias);
+            xb += step_w;
+            if (++nw == Nw) {
+                nw = 0; xb += wrap_w;
+                if (++nh == Nh) { nh = 0; xb += wrap_h; }
             }
         }
     }
@@ -305,10 +297,11 @@ cv_grad_weight_wide_kernel(const float* __restrict__ xpad, const float* __restri
 #pragma unroll
         for (int r = 0; r < DWW_RI; ++r)
             if (r < n_rows)
-                out[(size_t)(i0 + r) * Kc + j] = ((acc[r] + red[0][r][lane]) + red[1][r][lane]) + red[2][r][lane];
+                out[(size_t)(i0 + r) * Kc + j] =
+                    (((acc[r] + red[0][r][lane]) + red[1][r][lane]) + red[2][r][lane]) * post;
         if (with_bias)
             out[(size_t)bias_row * Kc + j] =
-                ((acc_bias + red[0][DWW_RI][lane]) + red[1][DWW_RI][lane]) + red[2][DWW_RI][lane];
+                (((acc_bias + red[0][DWW_RI][lane]) + red[1][DWW_RI][lane]) + red[2][DWW_RI][lane]) * post;
     }
 }
 
@@ -346,7 +339,7 @@ __global__ void __launch_bounds__(256)
 cv_grad_weight_narrow_kernel(const float* __restrict__ xpad, const float* __restrict__ upm,
                              const float* __restrict__ ym, float* __restrict__ dst, int S, int Kc, int rows,
                              int seg_per_slice, int H, int W, int C, int Kw, int Sh, int Sw, int Nh, int Nw,
-                             int bias_row, float biasvolt, int /*s_safe*/) {
+                             int bias_row, float biasvolt, int /*s_safe*/, float /*neg_s*/, float /*post*/) {
     __shared__ float red[4][DWW_RI + 1][kWave];
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -488,11 +481,12 @@ int launch_cv_grad_weight_wide(const float* xpad, const float* upm, const float*
     {
         KernelTimerScope timer_("grad_weight", stream);
         const bool full = (g.Kw * g.C) % DWW_RI == 0;
+        const LeadScale ls = lead_scale(np.max_time);
         hipLaunchKernelGGL(g.Kc <= 32 ? cv_grad_weight_narrow_kernel
                            : full ? cv_grad_weight_wide_kernel<true> : cv_grad_weight_wide_kernel<false>, grid, dim3(256), 0,
                            stream, xpad, upm, ym, dst, (int)g.S, (int)g.Kc, (int)rows, seg_per_slice, (int)g.H,
                            (int)g.W, (int)g.C, (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.Nh, (int)g.Nw,
-                           np.bias ? (int)g.P : -1, np.biasvolt, (int)s_safe);
+                           np.bias ? (int)g.P : -1, np.biasvolt, (int)s_safe, ls.neg_s, ls.post);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;

@@ -157,7 +157,7 @@ constexpr int DW_UNROLL = 4;
 __global__ void __launch_bounds__(256)
 grad_weight_kernel(SegmentSource src, const float* __restrict__ upm, const float* __restrict__ ym,
                    float* __restrict__ dst, int S, int J, int rows, int row_start, int seg_per_slice,
-                   float biasvolt) {
+                   float biasvolt, float neg_s, float post) {
     __shared__ float red[3][DW_RI][kWave];
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -189,7 +189,7 @@ grad_weight_kernel(SegmentSource src, const float* __restrict__ upm, const float
             const float* xb[DW_UNROLL];
 #pragma unroll
             for (int u = 0; u < DW_UNROLL; ++u) {
-                yv[u] = ycol[(size_t)(s + u) * J];
+                yv[u] = ycol[(size_t)(s + u) * J] * -neg_s;
                 uv[u] = ucol[(size_t)(s + u) * J];
                 xb[u] = segment_base(src, s + u) + off0;
             }
@@ -197,14 +197,14 @@ grad_weight_kernel(SegmentSource src, const float* __restrict__ upm, const float
             for (int u = 0; u < DW_UNROLL; ++u) {
 #pragma unroll
                 for (int r = 0; r < DW_RI; ++r)
-                    acc[r] = __fmaf_rn(fminf(xb[u][r] - yv[u], 0.0f), uv[u], acc[r]);
+                    acc[r] = __fmaf_rn(scaled_lead(xb[u][r], neg_s, yv[u]), uv[u], acc[r]);
             }
         }
         for (; s < s_hi; ++s) {
-            const float yv = ycol[(size_t)s * J], uv = ucol[(size_t)s * J];
+            const float yv = ycol[(size_t)s * J] * -neg_s, uv = ucol[(size_t)s * J];
             const float* xb = segment_base(src, s) + off0;
 #pragma unroll
-            for (int r = 0; r < DW_RI; ++r) acc[r] = __fmaf_rn(fminf(xb[r] - yv, 0.0f), uv, acc[r]);
+            for (int r = 0; r < DW_RI; ++r) acc[r] = __fmaf_rn(scaled_lead(xb[r], neg_s, yv), uv, acc[r]);
         }
     } else {
         int off[DW_RI];
@@ -216,12 +216,12 @@ grad_weight_kernel(SegmentSource src, const float* __restrict__ upm, const float
             off[r] = row_offset(src, min(i, I - 1));
         }
         for (int s = s_lo; s < s_hi; ++s) {
-            const float yv = ycol[(size_t)s * J], uv = ucol[(size_t)s * J];
+            const float yv = ycol[(size_t)s * J] * -neg_s, uv = ucol[(size_t)s * J];
             const float* xb = segment_base(src, s);
 #pragma unroll
             for (int r = 0; r < DW_RI; ++r) {
                 const float xv = is_bias[r] ? biasvolt : xb[off[r]];
-                acc[r] = __fmaf_rn(fminf(xv - yv, 0.0f), uv, acc[r]);
+                acc[r] = __fmaf_rn(scaled_lead(xv, neg_s, yv), uv, acc[r]);
             }
         }
     }
@@ -235,7 +235,8 @@ grad_weight_kernel(SegmentSource src, const float* __restrict__ upm, const float
 #pragma unroll
         for (int r = 0; r < DW_RI; ++r) {
             if (i0 + r < rows)
-                out[(size_t)(i0 + r) * J + j] = ((acc[r] + red[0][r][lane]) + red[1][r][lane]) + red[2][r][lane];
+                out[(size_t)(i0 + r) * J + j] =
+                    (((acc[r] + red[0][r][lane]) + red[1][r][lane]) + red[2][r][lane]) * post;
         }
     }
 }
@@ -354,16 +355,25 @@ int launch_fc_grad_input(const float* x, const float* wt, const float* upm, cons
 }
 
 // Number of slices the segment range is cut into for dW: none when the (row-block x column-block)
-// grid alone fills the chip; otherwise enough for ~2048 blocks, at least 64 segments per slice, at
-// most 256 slices.
+// grid alone fills the chip; otherwise up to ~1536 blocks (six per CU, all resident at once), at
+// least 64 segments per slice, at most 256 slices.  Within the upper half of that range the count
+// is the one whose blocks spread most evenly over the 256 CUs: the launch lasts as long as the CU
+// with the most blocks, ceil(blocks / 256) of them, each 1/n of a column of work.
 int weight_grad_splits(int64_t S, int64_t base_blocks) {
     if (base_blocks >= 1024) return 1;
-    int64_t want = (1536 + base_blocks - 1) / (base_blocks > 0 ? base_blocks : 1);
+    if (base_blocks < 1) base_blocks = 1;
+    int64_t want = (1536 + base_blocks - 1) / base_blocks;
     int64_t cap = S / 64;
     if (want > cap) want = cap;
     if (want > 256) want = 256;
     if (want < 1) want = 1;
-    return (int)want;
+    int64_t best = want;
+    double best_cost = 1e30;
+    for (int64_t n = want; n >= 1 && 2 * n >= want; --n) {
+        const double cost = (double)((base_blocks * n + 255) / 256) / (double)n;
+        if (cost < best_cost * 0.995) { best_cost = cost; best = n; }
+    }
+    return (int)best;
 }
 
 int grad_weight_blocks(int64_t rows, int64_t J) {
@@ -383,8 +393,9 @@ int launch_grad_weight_rows(const SegmentSource& src, const float* upm, const fl
     if (grid.y > 65535u) return fail(SNNTC_ERR_TOO_LARGE, "weight gradient: too many weight rows");
     {
         KernelTimerScope timer_(row_start ? "grad_weight_tail" : "grad_weight", stream);
+        const LeadScale ls = lead_scale(np.max_time);
         hipLaunchKernelGGL(grad_weight_kernel, grid, dim3(256), 0, stream, src, upm, ym, dst, (int)S, (int)J,
-                           (int)rows, (int)row_start, seg_per_slice, np.biasvolt);
+                           (int)rows, (int)row_start, seg_per_slice, np.biasvolt, ls.neg_s, ls.post);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;

@@ -3,6 +3,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <math.h>
 #include <stddef.h>
 #include <stdint.h>
 
@@ -55,6 +56,29 @@ struct NeuronParams {
     float biasvolt;   // input value of the bias row
     int bias;         // biasvolt > 1e-8
 };
+
+// The weight-gradient kernels add up u * min(x - y, 0) over the segments.  They evaluate the second
+// factor as -clamp01((y - x) * s) / s with s a power of two: fma(x, -s, y*s) rounds exactly like
+// the difference itself, the [0, 1] clamp is an output modifier of the fma, and the factor -1/s is
+// applied once to the finished sum, so the result has the bits of the plain sub / min / fma
+// sequence at two vector instructions per term instead of three.  1/s is the power of two above
+// 2 * MAX_SPIKE_TIME: the clamp's upper end is never reached while inputs stay above
+// -MAX_SPIKE_TIME (outputs that take part are below MAX_SPIKE_TIME by construction).
+struct LeadScale {
+    float neg_s;      // -s
+    float post;       // -1/s
+};
+inline LeadScale lead_scale(float max_time) {
+    int e = 0;
+    if (max_time > 1.0f) {
+        if (max_time < 3e28f) frexpf(max_time, &e);      // max_time < 2^e
+        else e = 95;
+    }
+    return LeadScale{-ldexpf(1.0f, -(e + 1)), -ldexpf(1.0f, e + 1)};
+}
+__device__ __forceinline__ float scaled_lead(float x, float neg_s, float ys) {
+    return __builtin_amdgcn_fmed3f(__fmaf_rn(x, neg_s, ys), 0.0f, 1.0f);
+}
 
 // Where a segment's elements come from: rows of a dense matrix, or patches of an NHWC image
 // gathered on the fly (patch s=(a*Nh+nh)*Nw+nw, element i=(kh*Kw+kw)*C+c).
