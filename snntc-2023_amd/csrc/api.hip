@@ -159,7 +159,9 @@ int forward_chain(const SegmentSource& src, const FcFwdWs& ws, const float* w, f
 // area is sized for the worst case of 256 slices only when slicing can happen at all.
 struct BwdWs { float* upm; float* ym; float* wt; float* dxp; float* partial; int max_split; size_t bytes; };
 // patch_scratch: elements of the per-patch gradient of conv layers whose dX goes through patch space
-BwdWs bwd_ws(void* ws, int64_t S, int64_t rows, int64_t J, int64_t min_base_blocks, int64_t patch_scratch = 0) {
+// narrow_split: slices the one-launch backward of a narrow dense layer needs (0: not that path)
+BwdWs bwd_ws(void* ws, int64_t S, int64_t rows, int64_t J, int64_t min_base_blocks, int64_t patch_scratch = 0,
+             int narrow_split = 0) {
     Carver c(ws);
     BwdWs r;
     r.upm = c.take<float>(S * J);
@@ -167,6 +169,7 @@ BwdWs bwd_ws(void* ws, int64_t S, int64_t rows, int64_t J, int64_t min_base_bloc
     r.wt = c.take<float>(rows * J);
     r.dxp = c.take<float>(patch_scratch);
     r.max_split = weight_grad_splits(S, min_base_blocks);
+    if (narrow_split > r.max_split) r.max_split = narrow_split;
     r.partial = c.take<float>(r.max_split > 1 ? (int64_t)r.max_split * rows * J : 0);
     r.bytes = c.used;
     return r;
@@ -352,10 +355,16 @@ int snntc_fc_forward_workspace_bytes(int64_t B, int64_t I, int64_t J, size_t* by
     return SNNTC_OK;
 }
 
+// Slices of the one-launch backward pass for dense layers with few outputs; 0 when the layer takes
+// the general path.  Decided by the layer's shape alone.
+static int fc_narrow_split(int64_t B, int64_t I, int64_t J) {
+    return (I >= 1 && B >= 1 && fc_backward_narrow_supported(J)) ? fc_backward_narrow_splits(B) : 0;
+}
+
 int snntc_fc_backward_workspace_bytes(int64_t B, int64_t I, int64_t J, size_t* bytes) {
     if (!bytes || B < 0 || I < 0 || J < 0)
         return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_fc_backward_workspace_bytes: bad argument");
-    *bytes = bwd_ws(nullptr, B, I + 1, J, grad_weight_blocks(I, J)).bytes;
+    *bytes = bwd_ws(nullptr, B, I + 1, J, grad_weight_blocks(I, J), 0, fc_narrow_split(B, I, J)).bytes;
     return SNNTC_OK;
 }
 
@@ -390,10 +399,13 @@ int snntc_fc_backward(const float* grad, const float* x, const float* w, const f
         return dw ? launch_fill_zero(dw, w_rows * J, st) : SNNTC_OK;
     }
     if (!grad || !x || !w || !oldout) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_fc_backward: NULL tensor pointer");
-    BwdWs ws = bwd_ws(workspace, B, I + 1, J, grad_weight_blocks(I, J));
+    const int narrow = fc_narrow_split(B, I, J);
+    BwdWs ws = bwd_ws(workspace, B, I + 1, J, grad_weight_blocks(I, J), 0, narrow);
     rc = check_workspace(workspace, workspace_bytes, ws.bytes);
     if (rc) return rc;
     const NeuronParams np = neuron_params(params_host[0], params_host[2], params_host[5]);
+    if (narrow)                                          // a classifier head: everything in one launch
+        return launch_fc_backward_narrow(x, w, grad, oldout, oldout + B * J, dx, dw, ws.partial, B, I, J, np, st);
     rc = launch_prep_upstream(grad, oldout, oldout + B * J, ws.upm, ws.ym, B * J, np, st);
     if (rc) return rc;
     if (dx) {

@@ -241,6 +241,131 @@ grad_weight_kernel(SegmentSource src, const float* __restrict__ upm, const float
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Whole backward pass of a dense layer with few outputs (a classifier head: J <= 16) in one launch:
+// the masked upstream values, dX and dW.  A wavefront covers 16 weight rows i (the bias row is one
+// more row, with x = biasvolt and no dX) times four groups of JL adjacent columns: lane = (group,
+// row).  A block takes up to NARROW_SAMPLES samples, whose scaled output times and upstream values
+// it first puts into LDS; each of its wavefronts then walks every NARROW_WAVES-th sample.  dX[b, i]
+// is complete after a sample -- the four column groups are added in the order (0 + 1) + (2 + 3) --
+// and is stored at once; the dW sums of a lane run over the samples and are added across the
+// wavefronts in wavefront order at the end.  Both inputs of the comparison x <= y are scaled by
+// the same power of two, which does not change its outcome.  With more than one block of samples
+// the dW sums go to `dst` as slices for reduce_partials_kernel.
+// ---------------------------------------------------------------------------------------------
+constexpr int NARROW_GROUPS = 4;
+constexpr int NARROW_ROWS = kWave / NARROW_GROUPS;     // weight rows per block
+constexpr int NARROW_JMAX = 4 * NARROW_GROUPS;
+constexpr int NARROW_WAVES = 16;
+constexpr int NARROW_SAMPLES = 256;
+
+template <int JL>
+__global__ void __launch_bounds__(NARROW_WAVES * kWave)
+fc_backward_narrow_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                          const float* __restrict__ grad, const float* __restrict__ y,
+                          const float* __restrict__ rcp, float* __restrict__ dx, float* __restrict__ dst,
+                          int B, int I, int J, int rows, float max_cmp, float biasvolt, float neg_s, float post) {
+    constexpr int JP = JL * NARROW_GROUPS;
+    // one more row than samples: (-inf, 0), which adds nothing, for the turns of a wavefront past
+    // the block's last sample
+    __shared__ float ys[NARROW_SAMPLES + 1][JP];           // scaled output time, -inf where masked out
+    __shared__ float us[NARROW_SAMPLES + 1][JP];           // grad * 1/wsum, 0 where masked out
+    __shared__ float red[NARROW_WAVES - 1][JL][kWave];
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int group = lane / NARROW_ROWS;
+    const int i = blockIdx.x * NARROW_ROWS + lane % NARROW_ROWS;
+    const int j0 = group * JL;                             // first column of the lane
+    const int b0 = blockIdx.y * NARROW_SAMPLES;
+    const int n_s = min(NARROW_SAMPLES, B - b0);
+
+    for (int e = threadIdx.x; e < n_s * JP; e += NARROW_WAVES * kWave) {
+        const int bl = e / JP, j = e - bl * JP;
+        float yv = -INFINITY, uv = 0.0f;
+        if (j < J) {
+            const size_t t = (size_t)(b0 + bl) * J + j;
+            const float yt = y[t];
+            if (yt <= max_cmp) { yv = yt * -neg_s; uv = grad[t] * rcp[t]; }
+        }
+        ys[bl][j] = yv;
+        us[bl][j] = uv;
+    }
+    if (threadIdx.x < JP) {
+        ys[NARROW_SAMPLES][threadIdx.x] = -INFINITY;
+        us[NARROW_SAMPLES][threadIdx.x] = 0.0f;
+    }
+
+    const bool is_input = i < I;
+    const unsigned ic = (unsigned)min(i, I - 1);
+    // the lane's input of every sample its wavefront takes, requested before anything waits
+    constexpr int PER_WAVE = NARROW_SAMPLES / NARROW_WAVES;
+    const float* __restrict__ xcol = x + (size_t)b0 * I + ic;
+    float xs[PER_WAVE];
+#pragma unroll
+    for (int q = 0; q < PER_WAVE; ++q) {
+        const int bl = min(wave + q * NARROW_WAVES, n_s - 1);
+        xs[q] = is_input ? xcol[(size_t)bl * I] : biasvolt;
+    }
+    float wr[JL], acc[JL];
+#pragma unroll
+    for (int c = 0; c < JL; ++c) {
+        wr[c] = (dx && is_input && j0 + c < J) ? w[(size_t)ic * J + j0 + c] : 0.0f;
+        acc[c] = 0.0f;
+    }
+    __syncthreads();
+
+    // four samples at a time, without branches, so that their LDS reads and lane exchanges overlap
+    constexpr int BATCH = 4;
+    static_assert(PER_WAVE % BATCH == 0, "samples per wavefront must be a multiple of the batch");
+#pragma unroll
+    for (int q0 = 0; q0 < PER_WAVE; q0 += BATCH) {
+        float dxa[BATCH];
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+            const int bl = wave + (q0 + u) * NARROW_WAVES;
+            const int row = bl < n_s ? bl : NARROW_SAMPLES;
+            const float xq = xs[q0 + u] * -neg_s;
+            dxa[u] = 0.0f;
+#pragma unroll
+            for (int c = 0; c < JL; ++c) {
+                const float yv = ys[row][j0 + c], uv = us[row][j0 + c];
+                acc[c] = __fmaf_rn(__builtin_amdgcn_fmed3f(yv - xq, 0.0f, 1.0f), uv, acc[c]);
+                dxa[u] = __fmaf_rn(uv, xq <= yv ? wr[c] : 0.0f, dxa[u]);
+            }
+        }
+        if (dx) {                                           // block-uniform
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u) dxa[u] += __shfl_xor(dxa[u], NARROW_ROWS, kWave);      // (0 + 1), (2 + 3)
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u) dxa[u] += __shfl_xor(dxa[u], 2 * NARROW_ROWS, kWave);
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u) {
+                const int bl = wave + (q0 + u) * NARROW_WAVES;
+                if (group == 0 && is_input && bl < n_s) dx[(size_t)(b0 + bl) * I + i] = dxa[u];
+            }
+        }
+    }
+
+    if (!dst) return;
+    if (wave > 0) {
+#pragma unroll
+        for (int c = 0; c < JL; ++c) red[wave - 1][c][lane] = acc[c];
+    }
+    __syncthreads();
+    if (wave == 0 && i < rows) {
+        float* out = dst + (size_t)blockIdx.y * rows * J + (size_t)i * J + j0;
+#pragma unroll
+        for (int c = 0; c < JL; ++c) {
+            if (j0 + c < J) {
+                float sum = acc[c];
+#pragma unroll
+                for (int v = 0; v < NARROW_WAVES - 1; ++v) sum += red[v][c][lane];
+                out[c] = sum * post;
+            }
+        }
+    }
+}
+
 // A block adds up 32 elements: its eight groups of 32 threads each take a contiguous eighth of the
 // slices (two chains per thread keep loads in flight) and the eight sums are added in group order.
 // The order of additions depends only on nsplit, never on timing.
@@ -410,6 +535,35 @@ int launch_reduce_partials(const float* partial, float* dw, int64_t n, int nspli
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
+}
+
+bool fc_backward_narrow_supported(int64_t J) { return J >= 1 && J <= NARROW_JMAX; }
+
+int fc_backward_narrow_splits(int64_t B) { return (int)((B + NARROW_SAMPLES - 1) / NARROW_SAMPLES); }
+
+// dx and/or dw may be NULL.  With more than one block of samples `partial` takes the dW slices.
+int launch_fc_backward_narrow(const float* x, const float* w, const float* grad, const float* y, const float* rcp,
+                              float* dx, float* dw, float* partial, int64_t B, int64_t I, int64_t J,
+                              const NeuronParams& np, hipStream_t stream) {
+    const int64_t rows = I + np.bias;
+    const int nsplit = fc_backward_narrow_splits(B);
+    // without dW only the input rows are needed; the bias row has no dX
+    const int64_t lanes = dw ? rows : I;
+    dim3 grid((unsigned)((lanes + NARROW_ROWS - 1) / NARROW_ROWS), (unsigned)nsplit);
+    if (grid.y > 65535u) return fail(SNNTC_ERR_TOO_LARGE, "dense backward: batch %lld too large", (long long)B);
+    float* dst = dw ? (nsplit > 1 ? partial : dw) : nullptr;
+    {
+        KernelTimerScope timer_("fc_backward_narrow", stream);
+        const LeadScale ls = lead_scale(np.max_time);
+        const int jl = (int)((J + NARROW_GROUPS - 1) / NARROW_GROUPS);      // columns per lane
+        auto kern = jl == 1 ? fc_backward_narrow_kernel<1> : jl == 2 ? fc_backward_narrow_kernel<2>
+                  : jl == 3 ? fc_backward_narrow_kernel<3> : fc_backward_narrow_kernel<4>;
+        hipLaunchKernelGGL(kern, grid, dim3(NARROW_WAVES * kWave), 0, stream, x, w, grad, y, rcp, dx, dst, (int)B,
+                           (int)I, (int)J, (int)rows, np.max_cmp, np.biasvolt, ls.neg_s, ls.post);
+    }
+    SNNTC_HIP_CHECK(hipGetLastError());
+    if (!dw) return SNNTC_OK;
+    return launch_reduce_partials(partial, dw, rows * J, nsplit, stream);
 }
 
 // dxp: scratch of S * P floats (gradient per patch element)

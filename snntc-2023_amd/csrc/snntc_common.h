@@ -139,6 +139,15 @@ int launch_grad_weight_rows(const SegmentSource& src, const float* upm, const fl
                             hipStream_t stream);
 int launch_reduce_partials(const float* partial, float* dw, int64_t n, int nsplit, hipStream_t stream);
 
+// Dense layers with at most 16 outputs: masked upstream values, dX and dW in one launch (dx / dw
+// may be NULL).  `partial` (fc_backward_narrow_splits(B) x rows x J floats) is used when the batch
+// spans more than one block of samples.
+bool fc_backward_narrow_supported(int64_t J);
+int fc_backward_narrow_splits(int64_t B);
+int launch_fc_backward_narrow(const float* x, const float* w, const float* grad, const float* y, const float* rcp,
+                              float* dx, float* dw, float* partial, int64_t B, int64_t I, int64_t J,
+                              const NeuronParams& np, hipStream_t stream);
+
 // Conv layers with many channels: lane = channel (dX) / wide row blocks (dW), see cv_grad.hip.
 bool cv_grad_input_chan_supported(const ConvGeom& g);
 int launch_cv_grad_input_chan(const float* xpad, const float* w, const float* upm, const float* ym,
