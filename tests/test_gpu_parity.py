@@ -49,6 +49,13 @@ DENSE_CASES = [
     (6, 3, 1000, 70, True, "reftest"),
     (7, 4, 2048, 96, True, "baseline"),        # cross-wavefront sort
     (8, 2, 5000, 40, False, "reftest"),        # 8192-wide sort
+    # layers with at most 16 outputs take a backward pass of their own (one launch for the masked
+    # upstream values, dX and dW; 256 samples per block, 16 weight rows per wavefront)
+    (9, 256, 800, 10, True, "baseline"),       # the MLP's head at its batch
+    (10, 600, 95, 16, True, "reftest"),        # three blocks of samples, the last one partial
+    (11, 257, 17, 1, False, "reftest"),        # one output, no bias row, one sample past a block
+    (12, 33, 48, 13, True, "reftest"),         # bias row opens a block of its own
+    (13, 40, 64, 17, True, "reftest"),         # first width past that pass
 ]
 
 
@@ -80,6 +87,21 @@ def test_dense_forward_backward(seed, B, I, J, bias, dist):
     sdx, sdw, _ = capi.fc_backward_dev(g, x, w, p, ref_out)
     check_grad(sdx, rdx, adx * 8, "oracle fp32 dX")
     check_grad(sdw, rdw, adw * 8, "oracle fp32 dW")
+
+
+@pytest.mark.parametrize("B,I,J", [(300, 70, 10), (64, 100, 48)])
+def test_dense_backward_single_gradient_calls_match_the_joint_call(B, I, J):
+    """A NULL dX or dW output is simply not computed; the other one must not change by a bit."""
+    import snntc_amd as snn
+    x, w, p, g = dense_case(21, B, I, J, True, "reftest")
+    out = snn.snnfc(t(x), t(w), p)
+    dx, dw, _ = snn.snnfc_grad(t(g), t(x), t(w), p, out)
+    dx_only, none_w, _ = snn.snnfc_grad(t(g), t(x), t(w), p, out, want_dw=False)
+    none_x, dw_only, _ = snn.snnfc_grad(t(g), t(x), t(w), p, out, want_dx=False)
+    torch.cuda.synchronize()
+    assert none_w is None and none_x is None
+    assert torch.equal(dx_only, dx), "dX changes when dW is not asked for"
+    assert torch.equal(dw_only, dw), "dW changes when dX is not asked for"
 
 
 CONV_CASES = [
