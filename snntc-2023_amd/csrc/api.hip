@@ -497,7 +497,9 @@ int snntc_cv_backward(const float* grad, const float* xpad, const float* w, cons
     if (rc) return rc;
     if (dxpad) {
         if (cv_grad_input_chan_supported(g)) {
-            rc = launch_cv_grad_input_chan(xpad, w, ws.upm, ws.ym, dxpad, g, np, st);
+            rc = launch_cv_weight_regroup(w, ws.wt, g, st);
+            if (rc) return rc;
+            rc = launch_cv_grad_input_chan(xpad, ws.wt, ws.upm, ws.ym, dxpad, g, np, st);
         } else {
             rc = launch_transpose(w, ws.wt, g.P, Kc, st);   // wt[Kc, P]
             if (rc) return rc;

@@ -150,7 +150,10 @@ int launch_fc_backward_narrow(const float* x, const float* w, const float* grad,
 
 // Conv layers with many channels: lane = channel (dX) / wide row blocks (dW), see cv_grad.hip.
 bool cv_grad_input_chan_supported(const ConvGeom& g);
-int launch_cv_grad_input_chan(const float* xpad, const float* w, const float* upm, const float* ym,
+// launch_cv_grad_input_chan reads the weights from a copy regrouped as [tap][kc / 4][c][kc % 4]
+// (P * Kc floats), which launch_cv_weight_regroup writes.
+int launch_cv_weight_regroup(const float* w, float* wq, const ConvGeom& g, hipStream_t stream);
+int launch_cv_grad_input_chan(const float* xpad, const float* wq, const float* upm, const float* ym,
                               float* dxpad, const ConvGeom& g, const NeuronParams& np, hipStream_t stream);
 bool cv_grad_weight_wide_supported(const ConvGeom& g);
 int cv_grad_weight_wide_blocks(const ConvGeom& g);
