@@ -307,7 +307,7 @@ def account(torch, snn, layers):
       scan          : bytes 4*(2*S*I + (I+b)*J + 2*S*J)            flops 4*steps
       dX kernels    : bytes 4*(2*S*J + in + I*J + in)              flops 2*pairs
       grad_weight   : bytes 4*(2*S*J + in + (I+b)*J)               flops 3*pairs
-      prep_upstream : bytes 4*(3*S*J + 2*S*J)                      flops S*J
+      prep_upstream : bytes 4*(3*S*J + 2*S*J + 2*I*J)              flops S*J   (carries the weight copy dX reads)
     `in` is the op's input tensor (B*I dense, B*H*W*C padded image for conv)."""
     acc = {}
 
@@ -337,8 +337,7 @@ def account(torch, snn, layers):
         add("fc_grad_input" if kind == "dense" else "cv_grad_input", 2.0 * pairs,
             4.0 * (2.0 * S * J + 2.0 * n_in + I * J))
         add("grad_weight", 3.0 * pairs, 4.0 * (2.0 * S * J + n_in + (I + bias) * J))
-        add("prep_upstream", float(S * J), 4.0 * 5.0 * S * J)
-        add("transpose_w", 0.0, 4.0 * 2.0 * I * J)
+        add("prep_upstream", float(S * J), 4.0 * (5.0 * S * J + 2.0 * I * J))     # with the weight copy for dX
     return acc
 
 

@@ -406,11 +406,11 @@ int snntc_fc_backward(const float* grad, const float* x, const float* w, const f
     const NeuronParams np = neuron_params(params_host[0], params_host[2], params_host[5]);
     if (narrow)                                          // a classifier head: everything in one launch
         return launch_fc_backward_narrow(x, w, grad, oldout, oldout + B * J, dx, dw, ws.partial, B, I, J, np, st);
-    rc = launch_prep_upstream(grad, oldout, oldout + B * J, ws.upm, ws.ym, B * J, np, st);
+    // wt[J, I] for dX (the bias row is not needed) is written by the same launch
+    rc = launch_backward_prologue(grad, oldout, oldout + B * J, ws.upm, ws.ym, B * J, np, dx ? 1 : 0, w, ws.wt, I, J,
+                                  0, st);
     if (rc) return rc;
     if (dx) {
-        rc = launch_transpose(w, ws.wt, I, J, st);      // wt[J, I]: bias row not needed for dX
-        if (rc) return rc;
         rc = launch_fc_grad_input(x, ws.wt, ws.upm, ws.ym, dx, B, I, J, I, st);
         if (rc) return rc;
     }
@@ -493,16 +493,16 @@ int snntc_cv_backward(const float* grad, const float* xpad, const float* w, cons
     rc = check_workspace(workspace, workspace_bytes, ws.bytes);
     if (rc) return rc;
     const NeuronParams np = neuron_params(params_host[0], params_host[4], params_host[11]);
-    rc = launch_prep_upstream(grad, oldout, oldout + g.S * Kc, ws.upm, ws.ym, g.S * Kc, np, st);
+    // the weight copy dX reads from is written by the same launch: regrouped for the channel kernel,
+    // wt[Kc, P] for the generic one
+    const bool chan_dx = cv_grad_input_chan_supported(g);
+    rc = launch_backward_prologue(grad, oldout, oldout + g.S * Kc, ws.upm, ws.ym, g.S * Kc, np,
+                                  !dxpad ? 0 : chan_dx ? 2 : 1, w, ws.wt, g.P, Kc, g.C, st);
     if (rc) return rc;
     if (dxpad) {
-        if (cv_grad_input_chan_supported(g)) {
-            rc = launch_cv_weight_regroup(w, ws.wt, g, st);
-            if (rc) return rc;
+        if (chan_dx) {
             rc = launch_cv_grad_input_chan(xpad, ws.wt, ws.upm, ws.ym, dxpad, g, np, st);
         } else {
-            rc = launch_transpose(w, ws.wt, g.P, Kc, st);   // wt[Kc, P]
-            if (rc) return rc;
             rc = launch_cv_grad_input(conv_source(xpad, g), ws.wt, ws.upm, ws.ym, ws.dxp, dxpad, g, g.P, st);
         }
         if (rc) return rc;

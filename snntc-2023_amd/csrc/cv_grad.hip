@@ -15,7 +15,7 @@ namespace {
 // dX.  A wavefront owns TILE consecutive pixels of one image row and 64 (or 32) channels; lane =
 // channel.  For every kernel tap (kh, kw) the lane keeps its weight row W[(kh,kw,c), 0..KCB) in
 // registers and sweeps the tile: the patch under the tap is the same for all lanes.  The rows come
-// from a copy of W regrouped as [tap][kc / 4][c][kc % 4] (weight_regroup_kernel): read from W itself,
+// from a copy of W regrouped as [tap][kc / 4][c][kc % 4] (written by backward_prologue_kernel): read from W itself,
 // every 16-byte fetch of a wavefront touches 64 different cache lines instead of 8.  The ym / upm
 // rows of the TILE + Kw - 1 patches one kernel row can touch are staged in a wavefront-private
 // piece of LDS (lane = output channel while staging) and read back as broadcasts, four output
@@ -210,19 +210,6 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
         for (int t = 0; t < DX_TILE; ++t)
             if (p0 + t < W) orow[(size_t)(p0 + t) * C] = acc[t];
     }
-}
-
-// W[(tap, c), kc] -> wq[tap][kc / 4][c][kc % 4], one 16-byte piece per thread (Kc is a multiple of 4).
-__global__ void __launch_bounds__(256)
-weight_regroup_kernel(const float* __restrict__ w, float* __restrict__ wq, int C, int Kc, int64_t n4) {
-    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;     // over (tap, c, kc / 4), kc / 4 fastest
-    if (t >= n4) return;
-    const int k4 = Kc / 4;
-    const int64_t row = t / k4;                              // tap * C + c
-    const int q = (int)(t - row * k4);
-    const int64_t tap = row / C;
-    const int c = (int)(row - tap * C);
-    reinterpret_cast<float4*>(wq)[(tap * k4 + q) * C + c] = reinterpret_cast<const float4*>(w)[t];
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -428,25 +415,13 @@ cv_grad_weight_narrow_kernel(const float* __restrict__ xpad, const float* __rest
 
 }  // namespace
 
-int launch_cv_weight_regroup(const float* w, float* wq, const ConvGeom& g, hipStream_t stream) {
-    const int64_t n4 = g.Kh * g.Kw * g.C * (g.Kc / 4);
-    if (n4 <= 0) return SNNTC_OK;
-    {
-        KernelTimerScope timer_("weight_regroup", stream);
-        hipLaunchKernelGGL(weight_regroup_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, stream, w, wq,
-                           (int)g.C, (int)g.Kc, n4);
-    }
-    SNNTC_HIP_CHECK(hipGetLastError());
-    return SNNTC_OK;
-}
-
 bool cv_grad_input_chan_supported(const ConvGeom& g) {
     // the staging buffer (four wavefronts, up to 2 * TILE + Kw patches) has to fit the default 64 KB of LDS
     // (plus the 6 KB the output-channel split keeps for its partial sums)
     return g.C >= 32 && g.Kc % 16 == 0 && (2 * DX_TILE + g.Kw) * 64 * 8 * 4 + 3 * DX_TILE * kWave * 4 <= 64 * 1024;
 }
 
-// wq: the weights regrouped by launch_cv_weight_regroup
+// wq: the weights regrouped by launch_backward_prologue (mode 2)
 int launch_cv_grad_input_chan(const float* xpad, const float* wq, const float* upm, const float* ym,
                               float* dxpad, const ConvGeom& g, const NeuronParams& np, hipStream_t stream) {
     const int halves = g.C <= 32 ? 2 : 1;

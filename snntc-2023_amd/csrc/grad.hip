@@ -18,32 +18,51 @@
 namespace snntc {
 namespace {
 
+// First launch of a backward pass.  The elementwise pass over the layer's outputs,
+//   upm = valid ? grad * rcp : 0,  ym = valid ? y : -inf   (valid: y <= MAX - 0.1),
+// and the weight copy dX reads from do not depend on each other: one launch does both, the first
+// prep_blocks workgroups the former, the rest the latter.
+//   mode 1: wt[cols, rows] = w[rows, cols]^T, a 32 x 32 tile per workgroup
+//   mode 2: w[(tap, c), kc] -> wt[tap][kc / 4][c][kc % 4], one 16-byte piece per thread (cols = Kc, a
+//           multiple of 4; chan = C)
 __global__ void __launch_bounds__(256)
-prep_upstream_kernel(const float* __restrict__ grad, const float* __restrict__ y,
-                     const float* __restrict__ rcp, float* __restrict__ upm, float* __restrict__ ym,
-                     int64_t n, float max_cmp) {
-    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= n) return;
-    const float yv = y[t];
-    const bool valid = yv <= max_cmp;
-    upm[t] = valid ? grad[t] * rcp[t] : 0.0f;
-    ym[t] = valid ? yv : -INFINITY;
-}
-
-// 32x32 tile transpose through LDS (padded against bank conflicts).
-__global__ void __launch_bounds__(256)
-transpose_kernel(const float* __restrict__ in, float* __restrict__ out, int rows, int cols) {
+backward_prologue_kernel(const float* __restrict__ grad, const float* __restrict__ y,
+                         const float* __restrict__ rcp, float* __restrict__ upm, float* __restrict__ ym,
+                         int64_t n, float max_cmp, int prep_blocks, int mode, const float* __restrict__ w,
+                         float* __restrict__ wt, int rows, int cols, int chan) {
     __shared__ float tile[32][33];
-    const int tx = threadIdx.x % 32, ty = threadIdx.x / 32;       // 32 x 8
-    const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
-    for (int dy = ty; dy < 32; dy += 8) {
-        const int r = r0 + dy, c = c0 + tx;
-        tile[dy][tx] = (r < rows && c < cols) ? in[(size_t)r * cols + c] : 0.0f;
+    if ((int)blockIdx.x < prep_blocks) {
+        const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+        if (t >= n) return;
+        const float yv = y[t];
+        const bool valid = yv <= max_cmp;
+        upm[t] = valid ? grad[t] * rcp[t] : 0.0f;
+        ym[t] = valid ? yv : -INFINITY;
+        return;
     }
-    __syncthreads();
-    for (int dy = ty; dy < 32; dy += 8) {
-        const int c = c0 + dy, r = r0 + tx;
-        if (r < rows && c < cols) out[(size_t)c * rows + r] = tile[tx][dy];
+    const int blk = (int)blockIdx.x - prep_blocks;
+    if (mode == 1) {
+        const int tiles_x = (cols + 31) / 32;
+        const int tx = threadIdx.x % 32, ty = threadIdx.x / 32;       // 32 x 8
+        const int c0 = (blk % tiles_x) * 32, r0 = (blk / tiles_x) * 32;
+        for (int dy = ty; dy < 32; dy += 8) {
+            const int r = r0 + dy, c = c0 + tx;
+            tile[dy][tx] = (r < rows && c < cols) ? w[(size_t)r * cols + c] : 0.0f;
+        }
+        __syncthreads();
+        for (int dy = ty; dy < 32; dy += 8) {
+            const int c = c0 + dy, r = r0 + tx;
+            if (r < rows && c < cols) wt[(size_t)c * rows + r] = tile[tx][dy];
+        }
+    } else {
+        const int k4 = cols / 4;
+        const int64_t t = (int64_t)blk * blockDim.x + threadIdx.x;    // over (tap, c, kc / 4), kc / 4 fastest
+        if (t >= (int64_t)rows * k4) return;
+        const int64_t row = t / k4;                                   // tap * C + c
+        const int q = (int)(t - row * k4);
+        const int64_t tap = row / chan;
+        const int c = (int)(row - tap * chan);
+        reinterpret_cast<float4*>(wt)[(tap * k4 + q) * chan + c] = reinterpret_cast<const float4*>(w)[t];
     }
 }
 
@@ -433,22 +452,21 @@ int blocks_for(int64_t n, int block) { return (int)((n + block - 1) / block); }
 
 }  // namespace
 
-int launch_prep_upstream(const float* grad, const float* y, const float* rcp, float* upm, float* ym,
-                         int64_t n, const NeuronParams& np, hipStream_t stream) {
-    if (n <= 0) return SNNTC_OK;
-    { KernelTimerScope timer_("prep_upstream", stream);
-    hipLaunchKernelGGL(prep_upstream_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream, grad, y, rcp,
-                       upm, ym, n, np.max_cmp);
-    }
-    SNNTC_HIP_CHECK(hipGetLastError());
-    return SNNTC_OK;
-}
-
-int launch_transpose(const float* w, float* wt, int64_t rows, int64_t cols, hipStream_t stream) {
-    if (rows <= 0 || cols <= 0) return SNNTC_OK;
-    dim3 grid((unsigned)((cols + 31) / 32), (unsigned)((rows + 31) / 32));
-    { KernelTimerScope timer_("transpose_w", stream);
-    hipLaunchKernelGGL(transpose_kernel, grid, dim3(256), 0, stream, w, wt, (int)rows, (int)cols);
+int launch_backward_prologue(const float* grad, const float* y, const float* rcp, float* upm, float* ym,
+                             int64_t n, const NeuronParams& np, int mode, const float* w, float* wt, int64_t rows,
+                             int64_t cols, int64_t chan, hipStream_t stream) {
+    const int64_t prep_blocks = (n + 255) / 256;
+    int64_t copy_blocks = 0;
+    if (mode == 1) copy_blocks = ((cols + 31) / 32) * ((rows + 31) / 32);
+    else if (mode == 2) copy_blocks = (rows * (cols / 4) + 255) / 256;
+    if (mode != 0 && (rows <= 0 || cols <= 0)) { mode = 0; copy_blocks = 0; }
+    if (prep_blocks + copy_blocks <= 0) return SNNTC_OK;
+    if (prep_blocks + copy_blocks > 0x7fffffffLL) return fail(SNNTC_ERR_TOO_LARGE, "backward: grid too large");
+    {
+        KernelTimerScope timer_("prep_upstream", stream);
+        hipLaunchKernelGGL(backward_prologue_kernel, dim3((unsigned)(prep_blocks + copy_blocks)), dim3(256), 0, stream,
+                           grad, y, rcp, upm, ym, n, np.max_cmp, (int)prep_blocks, mode, w, wt, (int)rows, (int)cols,
+                           (int)chan);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;

@@ -120,12 +120,13 @@ int launch_scan(const float* sorted, const int32_t* perm, const int32_t* n_real,
                 float* rcp, int32_t* causal_k, int64_t S, int64_t I, int64_t stride, int64_t J,
                 const NeuronParams& np, hipStream_t stream);
 
-// upm = valid ? grad*rcp : 0 ; ym = valid ? y : -inf   (valid: y <= MAX-0.1), n elements each.
-int launch_prep_upstream(const float* grad, const float* y, const float* rcp, float* upm, float* ym,
-                         int64_t n, const NeuronParams& np, hipStream_t stream);
-
-// wt[cols, rows] = w[rows, cols]^T
-int launch_transpose(const float* w, float* wt, int64_t rows, int64_t cols, hipStream_t stream);
+// upm = valid ? grad*rcp : 0 ; ym = valid ? y : -inf   (valid: y <= MAX-0.1), n elements each, and,
+// in the same launch, the weight copy dX reads from: mode 0 none, mode 1
+// wt[cols, rows] = w[rows, cols]^T, mode 2 the regrouped copy of a conv layer's weights
+// (wt[tap][cols / 4][chan][cols % 4] from w[(tap, chan), cols], rows = taps * chan).
+int launch_backward_prologue(const float* grad, const float* y, const float* rcp, float* upm, float* ym,
+                             int64_t n, const NeuronParams& np, int mode, const float* w, float* wt, int64_t rows,
+                             int64_t cols, int64_t chan, hipStream_t stream);
 
 int launch_fc_grad_input(const float* x, const float* wt, const float* upm, const float* ym, float* dx,
                          int64_t B, int64_t I, int64_t J, int64_t wt_stride, hipStream_t stream);
@@ -150,9 +151,7 @@ int launch_fc_backward_narrow(const float* x, const float* w, const float* grad,
 
 // Conv layers with many channels: lane = channel (dX) / wide row blocks (dW), see cv_grad.hip.
 bool cv_grad_input_chan_supported(const ConvGeom& g);
-// launch_cv_grad_input_chan reads the weights from a copy regrouped as [tap][kc / 4][c][kc % 4]
-// (P * Kc floats), which launch_cv_weight_regroup writes.
-int launch_cv_weight_regroup(const float* w, float* wq, const ConvGeom& g, hipStream_t stream);
+// launch_cv_grad_input_chan reads the weights from the copy regrouped by launch_backward_prologue (mode 2).
 int launch_cv_grad_input_chan(const float* xpad, const float* wq, const float* upm, const float* ym,
                               float* dxpad, const ConvGeom& g, const NeuronParams& np, hipStream_t stream);
 bool cv_grad_weight_wide_supported(const ConvGeom& g);
