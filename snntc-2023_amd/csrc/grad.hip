@@ -261,6 +261,111 @@ grad_weight_kernel(SegmentSource src, const float* __restrict__ upm, const float
 }
 
 // ---------------------------------------------------------------------------------------------
+// dW of a dense layer.  Same mapping as grad_weight_kernel (lane = output j, DW_RI weight rows per
+// block, the block's samples shared out over its four wavefronts), arranged so that a wavefront
+// waits for memory a few times instead of once per four samples -- at a batch of a few hundred
+// samples the wavefronts are short-lived and there are too few of them to hide those waits:
+//  * the x values of the block's rows, 256 samples at a time, are staged in LDS by all threads (the
+//    tile after the current one is already on its way) and read back as broadcasts; rows past the
+//    inputs read biasvolt, so the bias row needs no code of its own;
+//  * the ym / upm values of DWD_BATCH samples are requested together before the first one is used.
+// ---------------------------------------------------------------------------------------------
+#ifndef SNNTC_DWD_BATCH
+#define SNNTC_DWD_BATCH 16
+#endif
+constexpr int DWD_BATCH = SNNTC_DWD_BATCH;
+constexpr int DWD_TILE = 256;                              // samples per staged tile: 64 per wavefront
+static_assert(DW_RI == 8, "the staging below moves eight rows per sample");
+
+__global__ void __launch_bounds__(256)
+grad_weight_dense_kernel(const float* __restrict__ x, const float* __restrict__ upm, const float* __restrict__ ym,
+                         float* __restrict__ dst, int S, int I, int J, int rows, int seg_per_slice, float biasvolt,
+                         float neg_s, float post) {
+    __shared__ __align__(16) float xt[2][DWD_TILE][DW_RI];
+    __shared__ float red[3][DW_RI][kWave];
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int j = blockIdx.x * kWave + lane;
+    const unsigned jc = (unsigned)min(j, J - 1);
+    const int i0 = blockIdx.y * DW_RI;
+    const int s_begin = blockIdx.z * seg_per_slice;
+    const int s_end = min(S, s_begin + seg_per_slice);
+    const float* __restrict__ ycol = ym + jc;
+    const float* __restrict__ ucol = upm + jc;
+
+    float acc[DW_RI];
+#pragma unroll
+    for (int r = 0; r < DW_RI; ++r) acc[r] = 0.0f;
+
+    // element e = threadIdx.x + 256 * k of a tile: sample e / 8, row e % 8
+    const int st_row = threadIdx.x % DW_RI;
+    const int st_smp = threadIdx.x / DW_RI;                 // + 32 * k
+    const bool st_input = i0 + st_row < I;
+    const float* __restrict__ st_src = x + (st_input ? i0 + st_row : 0);
+    float pending[DW_RI];
+    auto fetch_tile = [&](int c0) {
+#pragma unroll
+        for (int k = 0; k < DW_RI; ++k) {
+            const int s = min(c0 + st_smp + 32 * k, s_end - 1);
+            pending[k] = st_input ? st_src[(size_t)s * I] : biasvolt;
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int k = 0; k < DW_RI; ++k) xt[buf][st_smp + 32 * k][st_row] = pending[k];
+    };
+
+    if (s_begin < s_end) {
+        fetch_tile(s_begin);
+        store_tile(0);
+        int buf = 0;
+        for (int c0 = s_begin; c0 < s_end; c0 += DWD_TILE, buf ^= 1) {
+            __syncthreads();                                // tile `buf` is complete; the other one is free
+            const bool more = c0 + DWD_TILE < s_end;
+            if (more) fetch_tile(c0 + DWD_TILE);
+            const int w0 = c0 + wave * (DWD_TILE / 4);
+#pragma unroll 1
+            for (int h = 0; h < DWD_TILE / 4; h += DWD_BATCH) {
+                const int sb = w0 + h;
+                if (sb >= s_end) break;                     // wavefront-uniform
+                float yv[DWD_BATCH], uv[DWD_BATCH];
+#pragma unroll
+                for (int q = 0; q < DWD_BATCH; ++q) {
+                    const int sc = min(sb + q, s_end - 1);
+                    yv[q] = ycol[(size_t)sc * J];
+                    uv[q] = ucol[(size_t)sc * J];
+                }
+#pragma unroll
+                for (int q = 0; q < DWD_BATCH; ++q) {
+                    const float4* xq = reinterpret_cast<const float4*>(&xt[buf][wave * (DWD_TILE / 4) + h + q][0]);
+                    const float4 xa = xq[0], xb = xq[1];
+                    const float xr[DW_RI] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+                    const float ys = yv[q] * -neg_s;
+                    const float u = sb + q < s_end ? uv[q] : 0.0f;
+#pragma unroll
+                    for (int r = 0; r < DW_RI; ++r) acc[r] = __fmaf_rn(scaled_lead(xr[r], neg_s, ys), u, acc[r]);
+                }
+            }
+            if (more) store_tile(buf ^ 1);
+        }
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int r = 0; r < DW_RI; ++r) red[wave - 1][r][lane] = acc[r];
+    }
+    __syncthreads();
+    if (wave == 0 && j < J) {
+        float* out = dst + (size_t)blockIdx.z * rows * J;
+#pragma unroll
+        for (int r = 0; r < DW_RI; ++r) {
+            if (i0 + r < rows)
+                out[(size_t)(i0 + r) * J + j] =
+                    (((acc[r] + red[0][r][lane]) + red[1][r][lane]) + red[2][r][lane]) * post;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // Whole backward pass of a dense layer with few outputs (a classifier head: J <= 16) in one launch:
 // the masked upstream values, dX and dW.  A wavefront covers 16 weight rows i (the bias row is one
 // more row, with x = biasvolt and no dX) times four groups of JL adjacent columns: lane = (group,
@@ -537,8 +642,12 @@ int launch_grad_weight_rows(const SegmentSource& src, const float* upm, const fl
     {
         KernelTimerScope timer_(row_start ? "grad_weight_tail" : "grad_weight", stream);
         const LeadScale ls = lead_scale(np.max_time);
-        hipLaunchKernelGGL(grad_weight_kernel, grid, dim3(256), 0, stream, src, upm, ym, dst, (int)S, (int)J,
-                           (int)rows, (int)row_start, seg_per_slice, np.biasvolt, ls.neg_s, ls.post);
+        if (!src.conv && row_start == 0)
+            hipLaunchKernelGGL(grad_weight_dense_kernel, grid, dim3(256), 0, stream, src.base, upm, ym, dst, (int)S,
+                               (int)src.I, (int)J, (int)rows, seg_per_slice, np.biasvolt, ls.neg_s, ls.post);
+        else
+            hipLaunchKernelGGL(grad_weight_kernel, grid, dim3(256), 0, stream, src, upm, ym, dst, (int)S, (int)J,
+                               (int)rows, (int)row_start, seg_per_slice, np.biasvolt, ls.neg_s, ls.post);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
