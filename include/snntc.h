@@ -107,6 +107,9 @@ SNNTC_API int snntc_fc_forward_ex(const float* x, const float* w, const float* p
  * grad_rows still declared as 2B), oldout[2B,J] = the forward output.
  * dx[B,I], dw[w_rows,J], dparams[6] (device; written with zeros).  Any of the three outputs may be
  * NULL: that gradient is then not computed (the reference always computes all of them).
+ * Domain: inputs are spike times; dw is exact for x >= -MAX_SPIKE_TIME (it is formed from the
+ * differences y - x, which the kernels keep within 2 * MAX_SPIKE_TIME; the same holds for
+ * snntc_cv_backward).
  * Errors: grad_rows != 2B -> DIM_MISMATCH (snntc/snnfcgrad_kernels.cc:119-120); sizes as above. */
 SNNTC_API int snntc_fc_backward(const float* grad, const float* x, const float* w, const float* params_host,
                       const float* oldout, float* dx, float* dw, float* dparams,

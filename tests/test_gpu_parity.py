@@ -338,6 +338,37 @@ def test_dense_non_default_parameters_and_sentinel_inputs(biasvolt, theta, max_t
                               lambda out: snn.snnfc_grad(t(g), t(x), t(w), p, t(out)), g, B)
 
 
+@pytest.mark.parametrize("max_time", [1.0, 12.0, 1e5, 3e6])
+@pytest.mark.parametrize("J", [9, 70])
+def test_dense_weight_gradient_over_the_whole_range_of_time_differences(max_time, J):
+    """The dW kernels evaluate min(x - y, 0) through a scaled, clamped difference that is exact while
+    y - x stays below 2 * MAX.  Inputs here run from -0.9 * MAX up to the sentinel, outputs up to
+    MAX - 0.1, so the differences cover (almost) that whole range, for MAX below, at and far above
+    the default, and for both dW kernels (narrow head and general)."""
+    import snntc_amd as snn
+    rng = np.random.default_rng(int(max_time) % 1000 + J)
+    B, I = 70, 40
+    x = ((rng.random((B, I)) * 1.85 - 0.9) * max_time).astype(np.float32)
+    x[rng.random((B, I)) < 0.1] = np.float32(max_time)
+    w = rng.standard_normal((I + 1, J)).astype(np.float32)
+    p = capi.fc_params(1.0, max_time=max_time)
+    # a forward output written by hand: spike times anywhere in [0, MAX - 0.1], a few never-fired
+    out = np.zeros((2 * B, J), np.float32)
+    out[:B] = (rng.random((B, J)) * (np.float32(max_time) - np.float32(0.1))).astype(np.float32)
+    out[B:] = rng.standard_normal((B, J)).astype(np.float32)
+    dead = rng.random((B, J)) < 0.1
+    out[:B][dead] = np.float32(max_time); out[B:][dead] = 0.0
+    g = np.zeros((2 * B, J), np.float32); g[:B] = rng.standard_normal((B, J))
+    dx, dw, _ = snn.snnfc_grad(t(g), t(x), t(w), p, t(out))
+    torch.cuda.synchronize()
+    rdx, rdw, _ = capi.fc_backward_dev(g, x, w, p, out, wide=True)
+    ao = out.copy(); ao[B:] = np.abs(ao[B:])
+    adx, adw, _ = capi.fc_backward_dev(np.abs(g), x, np.abs(w), p, ao, wide=True)
+    check_grad(dx.cpu().numpy(), rdx, adx, "dX")
+    check_grad(dw.cpu().numpy(), rdw, adw, "dW")
+    assert np.isfinite(dw.cpu().numpy()).all()
+
+
 @pytest.mark.parametrize("biasvolt,theta,max_time", PARAM_SWEEP)
 @pytest.mark.parametrize("C,Kc", [(32, 32), (64, 16), (5, 9)])
 def test_conv_non_default_parameters_and_sentinel_inputs(biasvolt, theta, max_time, C, Kc):
