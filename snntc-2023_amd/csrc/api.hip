@@ -392,9 +392,10 @@ int snntc_fc_backward(const float* grad, const float* x, const float* w, const f
         return fail(SNNTC_ERR_DIM_MISMATCH, "snntc_fc_backward: Grad/Oldout batch should be 2 * batch (got %lld for batch %lld)",
                     (long long)grad_rows, (long long)B);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (dparams) { rc = launch_fill_zero(dparams, 6, st); if (rc) return rc; }
-    if (!dx && !dw) return SNNTC_OK;                     // a NULL gradient output is simply not computed
+    // dparams is all zeros; where a backward launch follows, its first workgroup writes them
+    if (!dx && !dw) return dparams ? launch_fill_zero(dparams, 6, st) : SNNTC_OK;   // a NULL gradient output is simply not computed
     if (B == 0 || J == 0) {
+        if (dparams) { rc = launch_fill_zero(dparams, 6, st); if (rc) return rc; }
         if (dx) { rc = launch_fill_zero(dx, B * I, st); if (rc) return rc; }
         return dw ? launch_fill_zero(dw, w_rows * J, st) : SNNTC_OK;
     }
@@ -405,10 +406,11 @@ int snntc_fc_backward(const float* grad, const float* x, const float* w, const f
     if (rc) return rc;
     const NeuronParams np = neuron_params(params_host[0], params_host[2], params_host[5]);
     if (narrow)                                          // a classifier head: everything in one launch
-        return launch_fc_backward_narrow(x, w, grad, oldout, oldout + B * J, dx, dw, ws.partial, B, I, J, np, st);
+        return launch_fc_backward_narrow(x, w, grad, oldout, oldout + B * J, dx, dw, ws.partial, dparams, 6, B, I, J,
+                                         np, st);
     // wt[J, I] for dX (the bias row is not needed) is written by the same launch
     rc = launch_backward_prologue(grad, oldout, oldout + B * J, ws.upm, ws.ym, B * J, np, dx ? 1 : 0, w, ws.wt, I, J,
-                                  0, st);
+                                  0, dparams, 6, st);
     if (rc) return rc;
     if (dx) {
         rc = launch_fc_grad_input(x, ws.wt, ws.upm, ws.ym, dx, B, I, J, I, st);
@@ -481,9 +483,9 @@ int snntc_cv_backward(const float* grad, const float* xpad, const float* w, cons
         return fail(SNNTC_ERR_DIM_MISMATCH, "snntc_cv_backward: Grad/Oldout batch should be 2 * batch (got %lld for batch %lld)",
                     (long long)grad_rows, (long long)B);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (dparams) { rc = launch_fill_zero(dparams, 12, st); if (rc) return rc; }
-    if (!dxpad && !dw) return SNNTC_OK;                  // a NULL gradient output is simply not computed
+    if (!dxpad && !dw) return dparams ? launch_fill_zero(dparams, 12, st) : SNNTC_OK;   // a NULL gradient output is simply not computed
     if (g.S == 0 || Kc == 0) {
+        if (dparams) { rc = launch_fill_zero(dparams, 12, st); if (rc) return rc; }
         if (dxpad) { rc = launch_fill_zero(dxpad, B * H * W * C, st); if (rc) return rc; }
         return dw ? launch_fill_zero(dw, w_rows * Kc, st) : SNNTC_OK;
     }
@@ -497,7 +499,7 @@ int snntc_cv_backward(const float* grad, const float* xpad, const float* w, cons
     // wt[Kc, P] for the generic one
     const bool chan_dx = cv_grad_input_chan_supported(g);
     rc = launch_backward_prologue(grad, oldout, oldout + g.S * Kc, ws.upm, ws.ym, g.S * Kc, np,
-                                  !dxpad ? 0 : chan_dx ? 2 : 1, w, ws.wt, g.P, Kc, g.C, st);
+                                  !dxpad ? 0 : chan_dx ? 2 : 1, w, ws.wt, g.P, Kc, g.C, dparams, 12, st);
     if (rc) return rc;
     if (dxpad) {
         if (chan_dx) {

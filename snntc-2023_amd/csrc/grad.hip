@@ -29,8 +29,10 @@ __global__ void __launch_bounds__(256)
 backward_prologue_kernel(const float* __restrict__ grad, const float* __restrict__ y,
                          const float* __restrict__ rcp, float* __restrict__ upm, float* __restrict__ ym,
                          int64_t n, float max_cmp, int prep_blocks, int mode, const float* __restrict__ w,
-                         float* __restrict__ wt, int rows, int cols, int chan) {
+                         float* __restrict__ wt, int rows, int cols, int chan, float* __restrict__ zeros,
+                         int n_zeros) {
     __shared__ float tile[32][33];
+    if (blockIdx.x == 0 && (int)threadIdx.x < n_zeros) zeros[threadIdx.x] = 0.0f;    // the dParams output
     if ((int)blockIdx.x < prep_blocks) {
         const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
         if (t >= n) return;
@@ -388,8 +390,10 @@ __global__ void __launch_bounds__(NARROW_WAVES * kWave)
 fc_backward_narrow_kernel(const float* __restrict__ x, const float* __restrict__ w,
                           const float* __restrict__ grad, const float* __restrict__ y,
                           const float* __restrict__ rcp, float* __restrict__ dx, float* __restrict__ dst,
-                          int B, int I, int J, int rows, float max_cmp, float biasvolt, float neg_s, float post) {
+                          int B, int I, int J, int rows, float max_cmp, float biasvolt, float neg_s, float post,
+                          float* __restrict__ zeros, int n_zeros) {
     constexpr int JP = JL * NARROW_GROUPS;
+    if (blockIdx.x == 0 && blockIdx.y == 0 && (int)threadIdx.x < n_zeros) zeros[threadIdx.x] = 0.0f;   // dParams
     // one more row than samples: (-inf, 0), which adds nothing, for the turns of a wavefront past
     // the block's last sample
     __shared__ float ys[NARROW_SAMPLES + 1][JP];           // scaled output time, -inf where masked out
@@ -559,19 +563,20 @@ int blocks_for(int64_t n, int block) { return (int)((n + block - 1) / block); }
 
 int launch_backward_prologue(const float* grad, const float* y, const float* rcp, float* upm, float* ym,
                              int64_t n, const NeuronParams& np, int mode, const float* w, float* wt, int64_t rows,
-                             int64_t cols, int64_t chan, hipStream_t stream) {
+                             int64_t cols, int64_t chan, float* zeros, int n_zeros, hipStream_t stream) {
+    if (!zeros) n_zeros = 0;
     const int64_t prep_blocks = (n + 255) / 256;
     int64_t copy_blocks = 0;
     if (mode == 1) copy_blocks = ((cols + 31) / 32) * ((rows + 31) / 32);
     else if (mode == 2) copy_blocks = (rows * (cols / 4) + 255) / 256;
     if (mode != 0 && (rows <= 0 || cols <= 0)) { mode = 0; copy_blocks = 0; }
-    if (prep_blocks + copy_blocks <= 0) return SNNTC_OK;
+    if (prep_blocks + copy_blocks <= 0) return n_zeros > 0 ? launch_fill_zero(zeros, n_zeros, stream) : SNNTC_OK;
     if (prep_blocks + copy_blocks > 0x7fffffffLL) return fail(SNNTC_ERR_TOO_LARGE, "backward: grid too large");
     {
         KernelTimerScope timer_("prep_upstream", stream);
         hipLaunchKernelGGL(backward_prologue_kernel, dim3((unsigned)(prep_blocks + copy_blocks)), dim3(256), 0, stream,
                            grad, y, rcp, upm, ym, n, np.max_cmp, (int)prep_blocks, mode, w, wt, (int)rows, (int)cols,
-                           (int)chan);
+                           (int)chan, zeros, n_zeros);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
@@ -670,8 +675,9 @@ int fc_backward_narrow_splits(int64_t B) { return (int)((B + NARROW_SAMPLES - 1)
 
 // dx and/or dw may be NULL.  With more than one block of samples `partial` takes the dW slices.
 int launch_fc_backward_narrow(const float* x, const float* w, const float* grad, const float* y, const float* rcp,
-                              float* dx, float* dw, float* partial, int64_t B, int64_t I, int64_t J,
-                              const NeuronParams& np, hipStream_t stream) {
+                              float* dx, float* dw, float* partial, float* zeros, int n_zeros, int64_t B, int64_t I,
+                              int64_t J, const NeuronParams& np, hipStream_t stream) {
+    if (!zeros) n_zeros = 0;
     const int64_t rows = I + np.bias;
     const int nsplit = fc_backward_narrow_splits(B);
     // without dW only the input rows are needed; the bias row has no dX
@@ -686,7 +692,7 @@ int launch_fc_backward_narrow(const float* x, const float* w, const float* grad,
         auto kern = jl == 1 ? fc_backward_narrow_kernel<1> : jl == 2 ? fc_backward_narrow_kernel<2>
                   : jl == 3 ? fc_backward_narrow_kernel<3> : fc_backward_narrow_kernel<4>;
         hipLaunchKernelGGL(kern, grid, dim3(NARROW_WAVES * kWave), 0, stream, x, w, grad, y, rcp, dx, dst, (int)B,
-                           (int)I, (int)J, (int)rows, np.max_cmp, np.biasvolt, ls.neg_s, ls.post);
+                           (int)I, (int)J, (int)rows, np.max_cmp, np.biasvolt, ls.neg_s, ls.post, zeros, n_zeros);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     if (!dw) return SNNTC_OK;

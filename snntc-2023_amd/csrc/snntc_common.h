@@ -123,10 +123,11 @@ int launch_scan(const float* sorted, const int32_t* perm, const int32_t* n_real,
 // upm = valid ? grad*rcp : 0 ; ym = valid ? y : -inf   (valid: y <= MAX-0.1), n elements each, and,
 // in the same launch, the weight copy dX reads from: mode 0 none, mode 1
 // wt[cols, rows] = w[rows, cols]^T, mode 2 the regrouped copy of a conv layer's weights
-// (wt[tap][cols / 4][chan][cols % 4] from w[(tap, chan), cols], rows = taps * chan).
+// (wt[tap][cols / 4][chan][cols % 4] from w[(tap, chan), cols], rows = taps * chan).  `zeros`, if not
+// NULL, are n_zeros (<= 256) floats the launch clears: the op's all-zero dParams output.
 int launch_backward_prologue(const float* grad, const float* y, const float* rcp, float* upm, float* ym,
                              int64_t n, const NeuronParams& np, int mode, const float* w, float* wt, int64_t rows,
-                             int64_t cols, int64_t chan, hipStream_t stream);
+                             int64_t cols, int64_t chan, float* zeros, int n_zeros, hipStream_t stream);
 
 int launch_fc_grad_input(const float* x, const float* wt, const float* upm, const float* ym, float* dx,
                          int64_t B, int64_t I, int64_t J, int64_t wt_stride, hipStream_t stream);
@@ -146,8 +147,8 @@ int launch_reduce_partials(const float* partial, float* dw, int64_t n, int nspli
 bool fc_backward_narrow_supported(int64_t J);
 int fc_backward_narrow_splits(int64_t B);
 int launch_fc_backward_narrow(const float* x, const float* w, const float* grad, const float* y, const float* rcp,
-                              float* dx, float* dw, float* partial, int64_t B, int64_t I, int64_t J,
-                              const NeuronParams& np, hipStream_t stream);
+                              float* dx, float* dw, float* partial, float* zeros, int n_zeros, int64_t B, int64_t I,
+                              int64_t J, const NeuronParams& np, hipStream_t stream);
 
 // Conv layers with many channels: lane = channel (dX) / wide row blocks (dW), see cv_grad.hip.
 bool cv_grad_input_chan_supported(const ConvGeom& g);
