@@ -399,6 +399,37 @@ def test_conv_non_default_parameters_and_sentinel_inputs(biasvolt, theta, max_ti
                               lambda out: snn.snncv_grad(t(g), t(xpad), t(w), p, t(out)), g, B)
 
 
+@pytest.mark.parametrize("max_time", [2.0, 1e5, 3e6])
+@pytest.mark.parametrize("C,Kc", [(32, 64), (8, 48), (32, 16)])
+def test_conv_weight_gradient_over_the_whole_range_of_time_differences(max_time, C, Kc):
+    """As the dense test of the same name, for the conv dW kernels (wide: Kc > 32, narrow: Kc <= 32)
+    and the generic one (C = 8): pixel times from -0.9 * MAX up to the sentinel, spike times written
+    by hand anywhere in [0, MAX - 0.1]."""
+    import snntc_amd as snn
+    rng = np.random.default_rng(int(max_time) % 1000 + C + Kc)
+    B, H, W, K = 2, 9, 10, 3
+    P = K * K * C
+    xpad = ((rng.random((B, H + 2, W + 2, C)) * 1.85 - 0.9) * max_time).astype(np.float32)
+    xpad[rng.random(xpad.shape) < 0.1] = np.float32(max_time)
+    w = rng.standard_normal((P + 1, Kc)).astype(np.float32)
+    p = capi.cv_params(K, K, 1, 1, same=True, biasvolt=1.0, max_time=max_time)
+    Nh, Nw, _ = capi.cv_dims(xpad.shape, p)
+    out = np.zeros((2 * B, Nh, Nw, Kc), np.float32)
+    out[:B] = (rng.random((B, Nh, Nw, Kc)) * (np.float32(max_time) - np.float32(0.1))).astype(np.float32)
+    out[B:] = rng.standard_normal((B, Nh, Nw, Kc)).astype(np.float32)
+    dead = rng.random((B, Nh, Nw, Kc)) < 0.1
+    out[:B][dead] = np.float32(max_time); out[B:][dead] = 0.0
+    g = np.zeros((2 * B, Nh, Nw, Kc), np.float32); g[:B] = rng.standard_normal((B, Nh, Nw, Kc))
+    dx, dw, _ = snn.snncv_grad(t(g), t(xpad), t(w), p, t(out))
+    torch.cuda.synchronize()
+    rdx, rdw, _ = capi.cv_backward_dev(g, xpad, w, p, out, wide=True)
+    ao = out.copy(); ao[B:] = np.abs(ao[B:])
+    adx, adw, _ = capi.cv_backward_dev(np.abs(g), xpad, np.abs(w), p, ao, wide=True)
+    check_grad(dx.cpu().numpy(), rdx, adx, "dX")
+    check_grad(dw.cpu().numpy(), rdw, adw, "dW")
+    assert np.isfinite(dw.cpu().numpy()).all()
+
+
 def test_empty_batch_and_single_elements():
     """B = 0 yields empty outputs and an all-zero weight gradient; 1x1x1 shapes work."""
     import snntc_amd as snn
