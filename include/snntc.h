@@ -164,6 +164,28 @@ SNNTC_API int snntc_softmax_time_loss(const float* times, const float* label, fl
                             int64_t B, int64_t J, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Earliest-spike pooling of NHWC spike times, SNN_maxpool2d (SNN_TC_Modules.py:215-246: pad with
+ * padvalue = 1e5, then -maxpool(-x) with VALID windows).  The padding is implicit here:
+ *   y[b,nh,nw,c] = min over kh < Kh, kw < Kw of x[b, nh*Sh - pad_top + kh, nw*Sw - pad_left + kw, c],
+ * where positions outside the H x W image count as pad_value.  The caller passes the layer's
+ * geometry: pad_top / pad_left (0 for VALID; the reference's SAME split puts int(total/2) before)
+ * and Nh, Nw = the number of whole windows of the padded image.
+ *   arg[b,nh,nw,c]  int32, kh*Kw + kw of the first window position (kh-major order) that attains
+ *                   the minimum -- the position a max pooling of -x that replaces its running
+ *                   maximum only on a strictly greater value ends on.  May be NULL (no backward).
+ * Backward: dx[b,h,w,c] = sum of grad_y over the windows whose recorded position is pixel (h,w)
+ * (a window whose minimum lies in the padding passes nothing on), added in (kh, kw) order.
+ * No workspace.  Errors: a size < 0, Kh/Kw/Sh/Sw < 1, a pad < 0 or >= the kernel size, a window
+ * that does not fit the padded image -> BAD_ARGUMENT; more than INT32_MAX elements -> TOO_LARGE.
+ * ------------------------------------------------------------------------------------------- */
+SNNTC_API int snntc_min_pool_forward(const float* x, float* y, int32_t* arg, int64_t B, int64_t H, int64_t W,
+                           int64_t C, int64_t Kh, int64_t Kw, int64_t Sh, int64_t Sw, int64_t pad_top,
+                           int64_t pad_left, int64_t Nh, int64_t Nw, float pad_value, void* stream);
+SNNTC_API int snntc_min_pool_backward(const float* grad_y, const int32_t* arg, float* dx, int64_t B, int64_t H,
+                            int64_t W, int64_t C, int64_t Kh, int64_t Kw, int64_t Sh, int64_t Sw,
+                            int64_t pad_top, int64_t pad_left, int64_t Nh, int64_t Nw, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * SGD update of a training step: w[t][e] -= lr * dw[t][e] for e in [0, n[t]), t in [0, count).
  * The reference leaves the update to the framework's optimizer (snntc/snntc-mnist.py:70,92-93);
  * here all weight tensors of a network are updated by one launch (per 32 tensors).

@@ -15,6 +15,9 @@ Test infrastructure only.  Nothing here shares code with ``snntc_oracle.c``:
   of value 1.0 and never fires while sum(w) < 1.
 * ``analytic_grads`` are the textbook derivatives of y = sum_C(w x) / (sum_C w - theta) over the
   causal set C; ``fd_grads`` are central finite differences of the float64 forward.
+* ``min_pool`` / ``min_pool_grad`` restate SNN_maxpool2d (SNN_TC_Modules.py:215-246) literally:
+  pad with padvalue, negate, VALID max pooling, negate; the gradient goes to the first position of
+  the padded window (row-major) that holds the maximum of -x.
 * ``same_pad`` is the SAME-padding split of SNN_conv (SNN_TC_Modules.py:147-161), which the
   reference's test recomputes independently (snntc/test-snn-cv-forward.py:70-75,126-131).
 """
@@ -178,3 +181,50 @@ def softmax_time_loss(times, label):
     sample = -(y * logp).sum(axis=1)
     grad = (y - np.exp(logp) * y.sum(axis=1, keepdims=True)) / t.shape[0]
     return sample, grad
+
+
+def min_pool(x, Kh, Kw, Sh, Sw, same=True, pad_value=1e5):
+    """SNN_maxpool2d (SNN_TC_Modules.py:215-246) on NHWC x, written as the reference writes it: pad
+    with pad_value (SAME split as same_pad), then -maxpool(-xpad) over VALID windows.
+    Returns (y[B,Nh,Nw,C], arg[B,Nh,Nw,C], (top, left)); arg = kh*Kw + kw of the first position of the
+    padded window, in row-major order, that holds the maximum of -x."""
+    x = np.asarray(x, np.float32)
+    B, H, W, C = x.shape
+    (top, bottom), (left, right) = (same_pad(H, Kh, Sh), same_pad(W, Kw, Sw)) if same else ((0, 0), (0, 0))
+    xpad = np.pad(x, ((0, 0), (top, bottom), (left, right), (0, 0)), constant_values=np.float32(pad_value))
+    Nh = (xpad.shape[1] - Kh) // Sh + 1
+    Nw = (xpad.shape[2] - Kw) // Sw + 1
+    neg = -xpad
+    best = np.full((B, Nh, Nw, C), -np.inf, np.float32)
+    arg = np.zeros((B, Nh, Nw, C), np.int32)
+    for kh in range(Kh):
+        for kw in range(Kw):
+            v = neg[:, kh:kh + (Nh - 1) * Sh + 1:Sh, kw:kw + (Nw - 1) * Sw + 1:Sw, :]
+            better = v > best                                  # strictly greater: the first maximum stays
+            arg[better] = kh * Kw + kw
+            best = np.where(better, v, best)
+    return -best, arg, (top, left)
+
+
+def min_pool_grad(grad_y, arg, in_shape, Kh, Kw, Sh, Sw, pad):
+    """Gradient of min_pool: each window's gradient goes to the padded-window position arg names;
+    what lands in the padding is dropped.  Contributions to a pixel are added in (kh, kw) order."""
+    B, H, W, C = in_shape
+    top, left = pad
+    gy = np.asarray(grad_y, np.float32)
+    Nh, Nw = gy.shape[1], gy.shape[2]
+    dx = np.zeros((B, H, W, C), np.float32)
+    for kh in range(Kh):
+        for kw in range(Kw):
+            hit = arg == kh * Kw + kw
+            for nh in range(Nh):
+                h = nh * Sh - top + kh
+                if h < 0 or h >= H:
+                    continue
+                for nw in range(Nw):
+                    w = nw * Sw - left + kw
+                    if w < 0 or w >= W:
+                        continue
+                    dx[:, h, w, :] += np.where(hit[:, nh, nw, :], gy[:, nh, nw, :], np.float32(0))
+    return dx
+

@@ -309,6 +309,47 @@ int snntc_softmax_time_loss(const float* times, const float* label, float* sampl
     return launch_softmax_time_loss(times, label, sample_loss, dtimes, B, J, static_cast<hipStream_t>(stream));
 }
 
+// Geometry checks shared by the two pooling entry points.
+static int pool_geom(int64_t B, int64_t H, int64_t W, int64_t C, int64_t Kh, int64_t Kw, int64_t Sh, int64_t Sw,
+                     int64_t pad_top, int64_t pad_left, int64_t Nh, int64_t Nw, const char* who, PoolGeom* g) {
+    if (B < 0 || H < 0 || W < 0 || C < 0 || Nh < 0 || Nw < 0)
+        return fail(SNNTC_ERR_BAD_ARGUMENT, "%s: negative size", who);
+    if (Kh < 1 || Kw < 1 || Sh < 1 || Sw < 1) return fail(SNNTC_ERR_BAD_ARGUMENT, "%s: kernel and stride must be >= 1", who);
+    if (pad_top < 0 || pad_left < 0 || pad_top >= Kh || pad_left >= Kw)
+        return fail(SNNTC_ERR_BAD_ARGUMENT, "%s: padding %lld x %lld outside [0, kernel)", who, (long long)pad_top,
+                    (long long)pad_left);
+    // every window has to reach into the image (a window wholly inside the padding has no meaning)
+    if (Nh > 0 && (Nh - 1) * Sh - pad_top >= H) return fail(SNNTC_ERR_BAD_ARGUMENT, "%s: Nh %lld does not fit", who, (long long)Nh);
+    if (Nw > 0 && (Nw - 1) * Sw - pad_left >= W) return fail(SNNTC_ERR_BAD_ARGUMENT, "%s: Nw %lld does not fit", who, (long long)Nw);
+    if (B * H * W * C > kInt32Max || B * Nh * Nw * C > kInt32Max)
+        return fail(SNNTC_ERR_TOO_LARGE, "%s: more than INT32_MAX elements", who);
+    *g = PoolGeom{B, H, W, C, Kh, Kw, Sh, Sw, pad_top, pad_left, Nh, Nw};
+    return SNNTC_OK;
+}
+
+int snntc_min_pool_forward(const float* x, float* y, int32_t* arg, int64_t B, int64_t H, int64_t W, int64_t C,
+                           int64_t Kh, int64_t Kw, int64_t Sh, int64_t Sw, int64_t pad_top, int64_t pad_left,
+                           int64_t Nh, int64_t Nw, float pad_value, void* stream) {
+    PoolGeom g;
+    int rc = pool_geom(B, H, W, C, Kh, Kw, Sh, Sw, pad_top, pad_left, Nh, Nw, "snntc_min_pool_forward", &g);
+    if (rc) return rc;
+    if (B * Nh * Nw * C == 0) return SNNTC_OK;
+    if (!y || (!x && B * H * W * C > 0)) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_min_pool_forward: NULL tensor pointer");
+    return launch_min_pool_forward(x, y, arg, g, pad_value, static_cast<hipStream_t>(stream));
+}
+
+int snntc_min_pool_backward(const float* grad_y, const int32_t* arg, float* dx, int64_t B, int64_t H, int64_t W,
+                            int64_t C, int64_t Kh, int64_t Kw, int64_t Sh, int64_t Sw, int64_t pad_top,
+                            int64_t pad_left, int64_t Nh, int64_t Nw, void* stream) {
+    PoolGeom g;
+    int rc = pool_geom(B, H, W, C, Kh, Kw, Sh, Sw, pad_top, pad_left, Nh, Nw, "snntc_min_pool_backward", &g);
+    if (rc) return rc;
+    if (B * H * W * C == 0) return SNNTC_OK;
+    if (!dx || ((!grad_y || !arg) && B * Nh * Nw * C > 0))
+        return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_min_pool_backward: NULL tensor pointer");
+    return launch_min_pool_backward(grad_y, arg, dx, g, static_cast<hipStream_t>(stream));
+}
+
 int snntc_sgd_update(float* const* w, const float* const* dw, const int64_t* n, int64_t count, float lr,
                      void* stream) {
     if (count < 0 || count > INT32_MAX) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_sgd_update: bad tensor count");

@@ -166,6 +166,16 @@ int launch_cv_grad_input(const SegmentSource& src, const float* wt, const float*
 
 int launch_fill_zero(float* p, int64_t n, hipStream_t stream);
 
+// Earliest-spike pooling (pool.hip).  Window (nh, nw) starts at pixel (nh*Sh - pad_top, nw*Sw - pad_left);
+// pixels outside the image count as pad_value.  arg (may be NULL in the forward pass) records kh*Kw+kw
+// of the first window position that attains the minimum.
+struct PoolGeom {
+    int64_t B, H, W, C, Kh, Kw, Sh, Sw, pad_top, pad_left, Nh, Nw;
+};
+int launch_min_pool_forward(const float* x, float* y, int32_t* arg, const PoolGeom& g, float pad_value,
+                            hipStream_t stream);
+int launch_min_pool_backward(const float* gy, const int32_t* arg, float* dx, const PoolGeom& g, hipStream_t stream);
+
 // w[t] -= lr * dw[t] for `count` tensors of n[t] elements (host arrays of device pointers).
 int launch_sgd_update(float* const* w, const float* const* dw, const int64_t* n, int count, float lr,
                       hipStream_t stream);

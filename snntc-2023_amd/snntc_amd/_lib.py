@@ -27,6 +27,7 @@ EXPORTS = (
     "snntc_cv_output_dims", "snntc_cv_forward_workspace_bytes", "snntc_cv_backward_workspace_bytes",
     "snntc_cv_forward", "snntc_cv_forward_ex", "snntc_cv_backward",
     "snntc_softmax_time_loss", "snntc_sgd_update",
+    "snntc_min_pool_forward", "snntc_min_pool_backward",
     "snntc_profile_enable", "snntc_profile_collect", "snntc_profile_entry",
 )
 
@@ -89,6 +90,8 @@ def load():
                                       vp, sz, vp]
     lib.snntc_softmax_time_loss.argtypes = [vp, vp, vp, vp, i64, i64, vp]
     lib.snntc_sgd_update.argtypes = [c.POINTER(vp), c.POINTER(vp), c.POINTER(i64), i64, c.c_float, vp]
+    lib.snntc_min_pool_forward.argtypes = [vp, vp, vp] + [i64] * 12 + [c.c_float, vp]
+    lib.snntc_min_pool_backward.argtypes = [vp, vp, vp] + [i64] * 12 + [vp]
     lib.snntc_profile_enable.argtypes = [c.c_int]
     lib.snntc_profile_collect.argtypes = []
     lib.snntc_profile_entry.argtypes = [c.c_int, c.POINTER(c.c_char_p), c.POINTER(i64), c.POINTER(c.c_double)]

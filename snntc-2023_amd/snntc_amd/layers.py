@@ -12,7 +12,7 @@ import numpy as np
 import torch
 import torch.nn.functional as F
 
-from .ops import SnnCvTimes, SnnFcTimes, SoftmaxTimeLoss
+from .ops import SnnCvTimes, SnnFcTimes, SnnMinPool, SoftmaxTimeLoss
 
 # Mirrors the reference's module-level switch (SNN_TC_Modules.py:11): when True the layers keep
 # the largest batch and element count they have seen in ``maxD`` (every tensor must stay below
@@ -187,7 +187,20 @@ class SNN_maxpool2d(_Pool2d):
     """Earliest-spike pooling: pad with 1e5, then -maxpool(-x), VALID (SNN_TC_Modules.py:215-246)."""
 
     def forward(self, input):
-        x = self._padded_nchw(input)
+        if input.is_cuda and input.dtype == torch.float32 and input.dim() == 4:
+            # one kernel each way: the padding is implicit and the minimum is taken directly
+            H, W = input.shape[1], input.shape[2]
+            top = bottom = left = right = 0
+            if self.padding == 'SAME':
+                top, bottom = _same_pad(H, self.Kh, self.Sh)
+                left, right = _same_pad(W, self.Kw, self.Sw)
+                if min(top, bottom, left, right) < 0:
+                    raise ValueError("negative SAME padding: kernel smaller than stride is not supported")
+            nh = (H + top + bottom - self.Kh) // self.Sh + 1
+            nw = (W + left + right - self.Kw) // self.Sw + 1
+            return SnnMinPool.apply(input.contiguous(), (self.Kh, self.Kw), (self.Sh, self.Sw), (top, left), (nh, nw),
+                                    float(self.padvalue))
+        x = self._padded_nchw(input)                         # host tensors: the reference's formula itself
         y = -F.max_pool2d(-x, (self.Kh, self.Kw), (self.Sh, self.Sw))
         return y.permute(0, 2, 3, 1)
 

@@ -316,3 +316,58 @@ class SoftmaxTimeLoss(torch.autograd.Function):
             return None, None
         (grad,) = ctx.saved_tensors
         return grad * upstream, None
+
+
+def min_pool(x, kernel, stride, pad, out_hw, pad_value=1e5, want_arg=True):
+    """Earliest-spike pooling of NHWC spike times x[B,H,W,C] -> (y[B,Nh,Nw,C], arg or None).
+    kernel = (Kh, Kw), stride = (Sh, Sw), pad = (top, left), out_hw = (Nh, Nw); pixels outside the
+    image count as pad_value.  arg records, per output, the window position that attained the minimum."""
+    lib = _lib.load()
+    x = _dev_f32(x, "x", 4)
+    B, H, W, C = x.shape
+    with torch.cuda.device(x.device):
+        y = torch.empty((B, out_hw[0], out_hw[1], C), dtype=torch.float32, device=x.device)
+        arg = torch.empty(y.shape, dtype=torch.int32, device=x.device) if want_arg else None
+        _lib.check(lib.snntc_min_pool_forward(_ptr(x), _ptr(y), _ptr(arg), B, H, W, C, kernel[0], kernel[1], stride[0],
+                                              stride[1], pad[0], pad[1], out_hw[0], out_hw[1], float(pad_value),
+                                              _stream(x.device)))
+    return y, arg
+
+
+def min_pool_grad(grad_y, arg, in_shape, kernel, stride, pad):
+    """Gradient of min_pool with respect to its input: every pixel adds the gradients of the windows
+    that recorded it."""
+    lib = _lib.load()
+    grad_y = _dev_f32(grad_y, "grad_y", 4)
+    B, H, W, C = in_shape
+    Nh, Nw = grad_y.shape[1], grad_y.shape[2]
+    if tuple(arg.shape) != tuple(grad_y.shape) or arg.dtype != torch.int32 or not arg.is_contiguous():
+        raise ValueError("arg must be the contiguous int32 tensor min_pool returned")
+    with torch.cuda.device(grad_y.device):
+        dx = torch.empty((B, H, W, C), dtype=torch.float32, device=grad_y.device)
+        _lib.check(lib.snntc_min_pool_backward(_ptr(grad_y), _ptr(arg), _ptr(dx), B, H, W, C, kernel[0], kernel[1],
+                                               stride[0], stride[1], pad[0], pad[1], Nh, Nw, _stream(grad_y.device)))
+    return dx
+
+
+class SnnMinPool(torch.autograd.Function):
+    """SNN_maxpool2d on device tensors: min over the (implicitly padded) window, gradient to the
+    position that attained it."""
+
+    @staticmethod
+    def forward(ctx, x, kernel, stride, pad, out_hw, pad_value):
+        y, arg = min_pool(x, kernel, stride, pad, out_hw, pad_value, want_arg=x.requires_grad)
+        ctx.geom = (tuple(x.shape), tuple(kernel), tuple(stride), tuple(pad))
+        if arg is not None:
+            ctx.save_for_backward(arg)
+        ctx.has_arg = arg is not None
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        if not ctx.has_arg:
+            return (None,) * 6
+        (arg,) = ctx.saved_tensors
+        in_shape, kernel, stride, pad = ctx.geom
+        return (min_pool_grad(grad_y.contiguous(), arg, in_shape, kernel, stride, pad),) + (None,) * 5
+
