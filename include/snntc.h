@@ -186,6 +186,19 @@ SNNTC_API int snntc_min_pool_backward(const float* grad_y, const int32_t* arg, f
                             int64_t pad_top, int64_t pad_left, int64_t Nh, int64_t Nw, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * SAME padding of SNN_conv (SNN_TC_Modules.py:147-161: tf.pad with MAX_SPIKE_TIME) in one pass:
+ *   xpad[b,hp,wp,c] = x[b, hp - top, wp - left, c] inside the H x W image, `value` outside,
+ * xpad being [B,Hp,Wp,C] with Hp >= top + H, Wp >= left + W.  snntc_pad_time_backward is the
+ * gradient: dx[b,h,w,c] = dxpad[b, h + top, w + left, c].  No workspace.
+ * Errors: a negative size or offset, Hp < top + H, Wp < left + W -> BAD_ARGUMENT; more than
+ * INT32_MAX elements -> TOO_LARGE.
+ * ------------------------------------------------------------------------------------------- */
+SNNTC_API int snntc_pad_time_forward(const float* x, float* xpad, int64_t B, int64_t H, int64_t W, int64_t C,
+                           int64_t top, int64_t left, int64_t Hp, int64_t Wp, float value, void* stream);
+SNNTC_API int snntc_pad_time_backward(const float* dxpad, float* dx, int64_t B, int64_t H, int64_t W, int64_t C,
+                            int64_t top, int64_t left, int64_t Hp, int64_t Wp, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * SGD update of a training step: w[t][e] -= lr * dw[t][e] for e in [0, n[t]), t in [0, count).
  * The reference leaves the update to the framework's optimizer (snntc/snntc-mnist.py:70,92-93);
  * here all weight tensors of a network are updated by one launch (per 32 tensors).

@@ -350,6 +350,38 @@ int snntc_min_pool_backward(const float* grad_y, const int32_t* arg, float* dx, 
     return launch_min_pool_backward(grad_y, arg, dx, g, static_cast<hipStream_t>(stream));
 }
 
+static int pad_geom(int64_t B, int64_t H, int64_t W, int64_t C, int64_t top, int64_t left, int64_t Hp, int64_t Wp,
+                    const char* who, PadGeom* g) {
+    if (B < 0 || H < 0 || W < 0 || C < 0 || top < 0 || left < 0)
+        return fail(SNNTC_ERR_BAD_ARGUMENT, "%s: negative size or offset", who);
+    if (Hp < top + H || Wp < left + W)
+        return fail(SNNTC_ERR_BAD_ARGUMENT, "%s: padded size %lld x %lld does not hold the image", who, (long long)Hp,
+                    (long long)Wp);
+    if (B * Hp * Wp * C > kInt32Max) return fail(SNNTC_ERR_TOO_LARGE, "%s: more than INT32_MAX elements", who);
+    *g = PadGeom{B, H, W, C, top, left, Hp, Wp};
+    return SNNTC_OK;
+}
+
+int snntc_pad_time_forward(const float* x, float* xpad, int64_t B, int64_t H, int64_t W, int64_t C, int64_t top,
+                           int64_t left, int64_t Hp, int64_t Wp, float value, void* stream) {
+    PadGeom g;
+    int rc = pad_geom(B, H, W, C, top, left, Hp, Wp, "snntc_pad_time_forward", &g);
+    if (rc) return rc;
+    if (B * Hp * Wp * C == 0) return SNNTC_OK;
+    if (!xpad || (!x && B * H * W * C > 0)) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_pad_time_forward: NULL tensor pointer");
+    return launch_pad_time(x, xpad, g, value, static_cast<hipStream_t>(stream));
+}
+
+int snntc_pad_time_backward(const float* dxpad, float* dx, int64_t B, int64_t H, int64_t W, int64_t C, int64_t top,
+                            int64_t left, int64_t Hp, int64_t Wp, void* stream) {
+    PadGeom g;
+    int rc = pad_geom(B, H, W, C, top, left, Hp, Wp, "snntc_pad_time_backward", &g);
+    if (rc) return rc;
+    if (B * H * W * C == 0) return SNNTC_OK;
+    if (!dxpad || !dx) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_pad_time_backward: NULL tensor pointer");
+    return launch_crop_time(dxpad, dx, g, static_cast<hipStream_t>(stream));
+}
+
 int snntc_sgd_update(float* const* w, const float* const* dw, const int64_t* n, int64_t count, float lr,
                      void* stream) {
     if (count < 0 || count > INT32_MAX) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_sgd_update: bad tensor count");

@@ -7,6 +7,9 @@
 // the first one in (kh, kw) order, as a max pooling that replaces its running maximum only on a
 // strictly greater value does -- so the backward pass is a gather: every input pixel adds the
 // gradients of the windows that recorded it, in (kh, kw) order, with no atomics.
+//
+// Also here: the SAME padding of SNN_conv (SNN_TC_Modules.py:147-161, tf.pad with MAX_SPIKE_TIME) as
+// one pass that writes every element of the padded tensor once, and the matching crop of the gradient.
 #include "snntc_common.h"
 
 namespace snntc {
@@ -84,7 +87,89 @@ min_pool_backward_kernel(const float* __restrict__ gy, const int32_t* __restrict
     dx[(size_t)row * W * C + e] = sum;
 }
 
+// xpad[b, hp, wp, c] = x[b, hp - top, wp - left, c] inside the image, `value` outside.
+// blockIdx.x = padded row (b, hp); VEC floats per thread (VEC = 4 when C is a multiple of 4 and both
+// tensors are 16-byte aligned: a group of four then never straddles a pixel).
+template <int VEC>
+__global__ void __launch_bounds__(256)
+pad_time_kernel(const float* __restrict__ x, float* __restrict__ xpad, int H, int W, int C, int top, int left,
+                int Hp, int Wp, float value, FastDiv by_c) {
+    const unsigned e = (blockIdx.y * 256u + threadIdx.x) * VEC;            // (wp, c) within the padded row
+    if (e >= (unsigned)(Wp * C)) return;
+    const unsigned b = blockIdx.x / (unsigned)Hp;
+    const int hp = (int)(blockIdx.x - b * (unsigned)Hp);
+    const int wp = (int)fast_div(e, by_c), c = (int)e - wp * C;
+    const int h = hp - top, w = wp - left;
+    const bool inside = h >= 0 && h < H && w >= 0 && w < W;
+    float* out = xpad + (size_t)blockIdx.x * Wp * C + e;
+    const float* in = x + (((size_t)b * H + (inside ? h : 0)) * W + (inside ? w : 0)) * C + c;
+    if (VEC == 4) {
+        float4 v = make_float4(value, value, value, value);
+        if (inside) v = *reinterpret_cast<const float4*>(in);
+        *reinterpret_cast<float4*>(out) = v;
+    } else {
+        *out = inside ? *in : value;
+    }
+}
+
+// dx[b, h, w, c] = dxpad[b, h + top, w + left, c]
+template <int VEC>
+__global__ void __launch_bounds__(256)
+crop_time_kernel(const float* __restrict__ dxpad, float* __restrict__ dx, int H, int W, int C, int top, int left,
+                 int Hp, int Wp) {
+    const unsigned e = (blockIdx.y * 256u + threadIdx.x) * VEC;            // (w, c) within the row
+    if (e >= (unsigned)(W * C)) return;
+    const unsigned b = blockIdx.x / (unsigned)H;
+    const int h = (int)(blockIdx.x - b * (unsigned)H);
+    const float* in = dxpad + (((size_t)b * Hp + h + top) * Wp + left) * C + e;
+    float* out = dx + (size_t)blockIdx.x * W * C + e;
+    if (VEC == 4) *reinterpret_cast<float4*>(out) = *reinterpret_cast<const float4*>(in);
+    else *out = *in;
+}
+
 }  // namespace
+
+int launch_pad_time(const float* x, float* xpad, const PadGeom& g, float value, hipStream_t stream) {
+    const int64_t rows = g.B * g.Hp, per_row = g.Wp * g.C;
+    if (rows <= 0 || per_row <= 0) return SNNTC_OK;
+    const bool vec = g.C % 4 == 0 && ((uintptr_t)x % 16 == 0) && ((uintptr_t)xpad % 16 == 0);
+    const int64_t threads = vec ? per_row / 4 : per_row;
+    dim3 grid((unsigned)rows, (unsigned)((threads + 255) / 256));
+    if (grid.y > 65535u) return fail(SNNTC_ERR_TOO_LARGE, "padding: row of %lld elements too long", (long long)per_row);
+    {
+        KernelTimerScope timer_("pad_time", stream);
+        const FastDiv by_c = make_fast_div(g.C, per_row);
+        if (vec)
+            hipLaunchKernelGGL(pad_time_kernel<4>, grid, dim3(256), 0, stream, x, xpad, (int)g.H, (int)g.W, (int)g.C,
+                               (int)g.top, (int)g.left, (int)g.Hp, (int)g.Wp, value, by_c);
+        else
+            hipLaunchKernelGGL(pad_time_kernel<1>, grid, dim3(256), 0, stream, x, xpad, (int)g.H, (int)g.W, (int)g.C,
+                               (int)g.top, (int)g.left, (int)g.Hp, (int)g.Wp, value, by_c);
+    }
+    SNNTC_HIP_CHECK(hipGetLastError());
+    return SNNTC_OK;
+}
+
+int launch_crop_time(const float* dxpad, float* dx, const PadGeom& g, hipStream_t stream) {
+    const int64_t rows = g.B * g.H, per_row = g.W * g.C;
+    if (rows <= 0 || per_row <= 0) return SNNTC_OK;
+    // a group of four starts at ((..) * Wp + left) * C + e floats: a multiple of 4 when C is
+    const bool vec = g.C % 4 == 0 && ((uintptr_t)dx % 16 == 0) && ((uintptr_t)dxpad % 16 == 0);
+    const int64_t threads = vec ? per_row / 4 : per_row;
+    dim3 grid((unsigned)rows, (unsigned)((threads + 255) / 256));
+    if (grid.y > 65535u) return fail(SNNTC_ERR_TOO_LARGE, "padding: row of %lld elements too long", (long long)per_row);
+    {
+        KernelTimerScope timer_("crop_time", stream);
+        if (vec)
+            hipLaunchKernelGGL(crop_time_kernel<4>, grid, dim3(256), 0, stream, dxpad, dx, (int)g.H, (int)g.W, (int)g.C,
+                               (int)g.top, (int)g.left, (int)g.Hp, (int)g.Wp);
+        else
+            hipLaunchKernelGGL(crop_time_kernel<1>, grid, dim3(256), 0, stream, dxpad, dx, (int)g.H, (int)g.W, (int)g.C,
+                               (int)g.top, (int)g.left, (int)g.Hp, (int)g.Wp);
+    }
+    SNNTC_HIP_CHECK(hipGetLastError());
+    return SNNTC_OK;
+}
 
 int launch_min_pool_forward(const float* x, float* y, int32_t* arg, const PoolGeom& g, float pad_value,
                             hipStream_t stream) {

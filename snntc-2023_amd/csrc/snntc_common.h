@@ -176,6 +176,14 @@ int launch_min_pool_forward(const float* x, float* y, int32_t* arg, const PoolGe
                             hipStream_t stream);
 int launch_min_pool_backward(const float* gy, const int32_t* arg, float* dx, const PoolGeom& g, hipStream_t stream);
 
+// SAME padding of a conv layer's input with a constant (pool.hip): xpad[B,Hp,Wp,C] holds x[B,H,W,C]
+// at row offset top, column offset left, `value` elsewhere; launch_crop_time is the reverse copy.
+struct PadGeom {
+    int64_t B, H, W, C, top, left, Hp, Wp;
+};
+int launch_pad_time(const float* x, float* xpad, const PadGeom& g, float value, hipStream_t stream);
+int launch_crop_time(const float* dxpad, float* dx, const PadGeom& g, hipStream_t stream);
+
 // w[t] -= lr * dw[t] for `count` tensors of n[t] elements (host arrays of device pointers).
 int launch_sgd_update(float* const* w, const float* const* dw, const int64_t* n, int count, float lr,
                       hipStream_t stream);

@@ -28,6 +28,7 @@ EXPORTS = (
     "snntc_cv_forward", "snntc_cv_forward_ex", "snntc_cv_backward",
     "snntc_softmax_time_loss", "snntc_sgd_update",
     "snntc_min_pool_forward", "snntc_min_pool_backward",
+    "snntc_pad_time_forward", "snntc_pad_time_backward",
     "snntc_profile_enable", "snntc_profile_collect", "snntc_profile_entry",
 )
 
@@ -92,6 +93,8 @@ def load():
     lib.snntc_sgd_update.argtypes = [c.POINTER(vp), c.POINTER(vp), c.POINTER(i64), i64, c.c_float, vp]
     lib.snntc_min_pool_forward.argtypes = [vp, vp, vp] + [i64] * 12 + [c.c_float, vp]
     lib.snntc_min_pool_backward.argtypes = [vp, vp, vp] + [i64] * 12 + [vp]
+    lib.snntc_pad_time_forward.argtypes = [vp, vp] + [i64] * 8 + [c.c_float, vp]
+    lib.snntc_pad_time_backward.argtypes = [vp, vp] + [i64] * 8 + [vp]
     lib.snntc_profile_enable.argtypes = [c.c_int]
     lib.snntc_profile_collect.argtypes = []
     lib.snntc_profile_entry.argtypes = [c.c_int, c.POINTER(c.c_char_p), c.POINTER(i64), c.POINTER(c.c_double)]

@@ -12,7 +12,7 @@ import numpy as np
 import torch
 import torch.nn.functional as F
 
-from .ops import SnnCvTimes, SnnFcTimes, SnnMinPool, SoftmaxTimeLoss
+from .ops import SnnCvTimes, SnnFcTimes, SnnMinPool, SnnPadTime, SoftmaxTimeLoss
 
 # Mirrors the reference's module-level switch (SNN_TC_Modules.py:11): when True the layers keep
 # the largest batch and element count they have seen in ``maxD`` (every tensor must stay below
@@ -50,6 +50,8 @@ def _pad_hw(x, kh, kw, sh, sw, value):
     if min(top, bottom, left, right) < 0:
         raise ValueError("negative SAME padding: kernel smaller than stride is not supported")
     if top or bottom or left or right:
+        if x.is_cuda and x.dtype == torch.float32 and x.dim() == 4:
+            return SnnPadTime.apply(x.contiguous(), top, bottom, left, right, float(value))    # one pass
         x = F.pad(x, (0, 0, left, right, top, bottom), mode="constant", value=float(value))
     return x
 

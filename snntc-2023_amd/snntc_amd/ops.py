@@ -371,3 +371,42 @@ class SnnMinPool(torch.autograd.Function):
         in_shape, kernel, stride, pad = ctx.geom
         return (min_pool_grad(grad_y.contiguous(), arg, in_shape, kernel, stride, pad),) + (None,) * 5
 
+
+def pad_time(x, top, bottom, left, right, value):
+    """x[B,H,W,C] -> [B, top+H+bottom, left+W+right, C], the border filled with `value` (one pass)."""
+    lib = _lib.load()
+    x = _dev_f32(x, "x", 4)
+    B, H, W, C = x.shape
+    Hp, Wp = top + H + bottom, left + W + right
+    with torch.cuda.device(x.device):
+        xpad = torch.empty((B, Hp, Wp, C), dtype=torch.float32, device=x.device)
+        _lib.check(lib.snntc_pad_time_forward(_ptr(x), _ptr(xpad), B, H, W, C, top, left, Hp, Wp, float(value),
+                                              _stream(x.device)))
+    return xpad
+
+
+def pad_time_grad(dxpad, in_shape, top, left):
+    """The gradient of pad_time: the H x W interior of dxpad."""
+    lib = _lib.load()
+    dxpad = _dev_f32(dxpad, "dxpad", 4)
+    B, H, W, C = in_shape
+    with torch.cuda.device(dxpad.device):
+        dx = torch.empty((B, H, W, C), dtype=torch.float32, device=dxpad.device)
+        _lib.check(lib.snntc_pad_time_backward(_ptr(dxpad), _ptr(dx), B, H, W, C, top, left, dxpad.shape[1],
+                                               dxpad.shape[2], _stream(dxpad.device)))
+    return dx
+
+
+class SnnPadTime(torch.autograd.Function):
+    """SAME padding of a conv layer's input with MAX_SPIKE_TIME, one kernel each way."""
+
+    @staticmethod
+    def forward(ctx, x, top, bottom, left, right, value):
+        ctx.geom = (tuple(x.shape), top, left)
+        return pad_time(x, top, bottom, left, right, value)
+
+    @staticmethod
+    def backward(ctx, dxpad):
+        in_shape, top, left = ctx.geom
+        return (pad_time_grad(dxpad.contiguous(), in_shape, top, left),) + (None,) * 5
+

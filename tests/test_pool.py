@@ -86,3 +86,25 @@ def test_pooling_argument_errors():
         snn.min_pool(x, (2, 2), (2, 2), (0, 0), (4, 2))              # a window wholly outside the image
     with pytest.raises(ValueError):
         snn.min_pool(x, (0, 2), (2, 2), (0, 0), (2, 2))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,H,W,C,pads", [(2, 5, 7, 3, (1, 1, 1, 1)), (3, 8, 8, 32, (0, 1, 0, 1)),
+                                          (2, 32, 32, 64, (1, 1, 1, 1)), (1, 224, 224, 3, (2, 3, 2, 3)),
+                                          (2, 4, 6, 8, (3, 0, 0, 2))])
+def test_hip_padding_matches_constant_pad(B, H, W, C, pads):
+    """SAME padding with MAX_SPIKE_TIME in one pass, and its gradient (the interior of the upstream)."""
+    import snntc_amd as snn
+    top, bottom, left, right = pads
+    rng = np.random.default_rng(H + C)
+    x = torch.from_numpy(rng.random((B, H, W, C)).astype(np.float32)).to("cuda:0").requires_grad_(True)
+    ref = F.pad(x.detach(), (0, 0, left, right, top, bottom), value=1e5)
+    out = snn.SnnPadTime.apply(x, top, bottom, left, right, 1e5)
+    assert torch.equal(out, ref)
+    g = torch.from_numpy(rng.standard_normal(tuple(ref.shape)).astype(np.float32)).to("cuda:0")
+    out.backward(g)
+    assert torch.equal(x.grad, g[:, top:top + H, left:left + W, :])
+    # the layer takes the same path
+    conv = snn.SNN_conv(C, 4, 3, 1, 'SAME')
+    assert torch.equal(conv.prepare_input(x.detach()), F.pad(x.detach(), (0, 0, 1, 1, 1, 1), value=1e5))
+
