@@ -30,40 +30,63 @@ FastDiv make_fast_div(int64_t d, int64_t max_n) {
     return f;
 }
 
-// blockIdx.x = output row (b, nh), blockIdx.y * 256 + threadIdx.x = (nw, c) within the row: 32-bit index
+// blockIdx.x = output row (b, nh); a thread takes VEC consecutive channels of one (nw, c) position of
+// the row (VEC = 4 when C is a multiple of 4 and the tensors are 16-byte aligned): 32-bit index
 // arithmetic only, consecutive lanes on consecutive channels.
+template <int VEC>
 __global__ void __launch_bounds__(256)
 min_pool_forward_kernel(const float* __restrict__ x, float* __restrict__ y, int32_t* __restrict__ arg, int H, int W,
                         int C, int Kh, int Kw, int Sh, int Sw, int pad_top, int pad_left, int Nh, int Nw,
                         float pad_value, FastDiv by_c) {
-    const unsigned e = blockIdx.y * 256u + threadIdx.x;
+    const unsigned e = (blockIdx.y * 256u + threadIdx.x) * VEC;
     if (e >= (unsigned)(Nw * C)) return;
     const unsigned nw = fast_div(e, by_c), c = e - nw * (unsigned)C;
     const unsigned row = blockIdx.x;
     const unsigned b = row / (unsigned)Nh, nh = row - b * (unsigned)Nh;                    // scalar: once per block
     const int h0 = (int)nh * Sh - pad_top, w0 = (int)nw * Sw - pad_left;
     const float* __restrict__ img = x + (size_t)b * H * W * C + c;
-    float best = INFINITY;
-    int where = 0;
+    float best[VEC];
+    int where[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) { best[v] = INFINITY; where[v] = 0; }
     for (int kh = 0; kh < Kh; ++kh) {
         const int h = h0 + kh;
         for (int kw = 0; kw < Kw; ++kw) {
             const int w = w0 + kw;
-            const float v = (h >= 0 && h < H && w >= 0 && w < W) ? img[((size_t)h * W + w) * C] : pad_value;
-            if (v < best) { best = v; where = kh * Kw + kw; }
+            float val[VEC];
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) val[v] = pad_value;
+            if (h >= 0 && h < H && w >= 0 && w < W) {
+                const float* p = img + ((size_t)h * W + w) * C;
+                if (VEC == 4) {
+                    const float4 q = *reinterpret_cast<const float4*>(p);
+                    val[0] = q.x; val[1] = q.y; val[2] = q.z; val[3] = q.w;
+                } else {
+                    val[0] = *p;
+                }
+            }
+#pragma unroll
+            for (int v = 0; v < VEC; ++v)
+                if (val[v] < best[v]) { best[v] = val[v]; where[v] = kh * Kw + kw; }
         }
     }
     const size_t t = (size_t)row * Nw * C + e;
-    y[t] = best;
-    if (arg) arg[t] = where;
+    if (VEC == 4) {
+        *reinterpret_cast<float4*>(y + t) = make_float4(best[0], best[1], best[2], best[3]);
+        if (arg) *reinterpret_cast<int4*>(arg + t) = make_int4(where[0], where[1], where[2], where[3]);
+    } else {
+        y[t] = best[0];
+        if (arg) arg[t] = where[0];
+    }
 }
 
-// blockIdx.x = input row (b, h), blockIdx.y * 256 + threadIdx.x = (w, c) within the row.
+// blockIdx.x = input row (b, h); a thread takes VEC consecutive channels of one (w, c) position.
+template <int VEC>
 __global__ void __launch_bounds__(256)
 min_pool_backward_kernel(const float* __restrict__ gy, const int32_t* __restrict__ arg, float* __restrict__ dx,
                          int H, int W, int C, int Kh, int Kw, int Sh, int Sw, int pad_top, int pad_left, int Nh,
                          int Nw, FastDiv by_c, FastDiv by_sw) {
-    const unsigned e = blockIdx.y * 256u + threadIdx.x;
+    const unsigned e = (blockIdx.y * 256u + threadIdx.x) * VEC;
     if (e >= (unsigned)(W * C)) return;
     const int w = (int)fast_div(e, by_c), c = (int)e - w * C;
     const unsigned row = blockIdx.x;
@@ -75,16 +98,34 @@ min_pool_backward_kernel(const float* __restrict__ gy, const int32_t* __restrict
     const int nh_hi = min(Nh - 1, hp / Sh), nh_lo = hp - Kh + 1 <= 0 ? 0 : (hp - Kh + Sh) / Sh;   // scalar
     const int nw_hi = min(Nw - 1, (int)fast_div((unsigned)wp, by_sw));
     const int nw_lo = wp - Kw + 1 <= 0 ? 0 : (int)fast_div((unsigned)(wp - Kw + Sw), by_sw);
-    float sum = 0.0f;
+    float sum[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) sum[v] = 0.0f;
     for (int nh = nh_hi; nh >= nh_lo; --nh) {
         const int kh = hp - nh * Sh;
         for (int nw = nw_hi; nw >= nw_lo; --nw) {
-            const int kw = wp - nw * Sw;
+            const int pos = kh * Kw + (wp - nw * Sw);
             const size_t o = (((size_t)b * Nh + nh) * Nw + nw) * C + c;
-            if (arg[o] == kh * Kw + kw) sum += gy[o];
+            // both values are requested at once: a gradient fetched only after the position has
+            // been looked at would cost a second trip to memory
+            int where[VEC];
+            float g[VEC];
+            if (VEC == 4) {
+                const int4 a4 = *reinterpret_cast<const int4*>(arg + o);
+                const float4 g4 = *reinterpret_cast<const float4*>(gy + o);
+                where[0] = a4.x; where[1] = a4.y; where[2] = a4.z; where[3] = a4.w;
+                g[0] = g4.x; g[1] = g4.y; g[2] = g4.z; g[3] = g4.w;
+            } else {
+                where[0] = arg[o];
+                g[0] = gy[o];
+            }
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) sum[v] += where[v] == pos ? g[v] : 0.0f;
         }
     }
-    dx[(size_t)row * W * C + e] = sum;
+    float* out = dx + (size_t)row * W * C + e;
+    if (VEC == 4) *reinterpret_cast<float4*>(out) = make_float4(sum[0], sum[1], sum[2], sum[3]);
+    else *out = sum[0];
 }
 
 // xpad[b, hp, wp, c] = x[b, hp - top, wp - left, c] inside the image, `value` outside.
@@ -171,17 +212,22 @@ int launch_crop_time(const float* dxpad, float* dx, const PadGeom& g, hipStream_
     return SNNTC_OK;
 }
 
+static bool aligned16(const void* p) { return (uintptr_t)p % 16 == 0; }
+
 int launch_min_pool_forward(const float* x, float* y, int32_t* arg, const PoolGeom& g, float pad_value,
                             hipStream_t stream) {
     const int64_t rows = g.B * g.Nh, per_row = g.Nw * g.C;
     if (rows <= 0 || per_row <= 0) return SNNTC_OK;
-    dim3 grid((unsigned)rows, (unsigned)((per_row + 255) / 256));
+    const bool vec = g.C % 4 == 0 && aligned16(x) && aligned16(y) && aligned16(arg);
+    const int64_t threads = vec ? per_row / 4 : per_row;
+    dim3 grid((unsigned)rows, (unsigned)((threads + 255) / 256));
     if (grid.y > 65535u) return fail(SNNTC_ERR_TOO_LARGE, "pooling: output row of %lld elements too long", (long long)per_row);
     {
         KernelTimerScope timer_("min_pool", stream);
-        hipLaunchKernelGGL(min_pool_forward_kernel, grid, dim3(256), 0, stream, x, y, arg, (int)g.H, (int)g.W, (int)g.C,
-                           (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.pad_top, (int)g.pad_left, (int)g.Nh,
-                           (int)g.Nw, pad_value, make_fast_div(g.C, per_row));
+        auto kern = vec ? min_pool_forward_kernel<4> : min_pool_forward_kernel<1>;
+        hipLaunchKernelGGL(kern, grid, dim3(256), 0, stream, x, y, arg, (int)g.H, (int)g.W, (int)g.C, (int)g.Kh,
+                           (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.pad_top, (int)g.pad_left, (int)g.Nh, (int)g.Nw,
+                           pad_value, make_fast_div(g.C, per_row));
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
@@ -190,13 +236,16 @@ int launch_min_pool_forward(const float* x, float* y, int32_t* arg, const PoolGe
 int launch_min_pool_backward(const float* gy, const int32_t* arg, float* dx, const PoolGeom& g, hipStream_t stream) {
     const int64_t rows = g.B * g.H, per_row = g.W * g.C;
     if (rows <= 0 || per_row <= 0) return SNNTC_OK;
-    dim3 grid((unsigned)rows, (unsigned)((per_row + 255) / 256));
+    const bool vec = g.C % 4 == 0 && aligned16(gy) && aligned16(arg) && aligned16(dx);
+    const int64_t threads = vec ? per_row / 4 : per_row;
+    dim3 grid((unsigned)rows, (unsigned)((threads + 255) / 256));
     if (grid.y > 65535u) return fail(SNNTC_ERR_TOO_LARGE, "pooling: input row of %lld elements too long", (long long)per_row);
     {
         KernelTimerScope timer_("min_pool_grad", stream);
-        hipLaunchKernelGGL(min_pool_backward_kernel, grid, dim3(256), 0, stream, gy, arg, dx, (int)g.H, (int)g.W,
-                           (int)g.C, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.pad_top, (int)g.pad_left,
-                           (int)g.Nh, (int)g.Nw, make_fast_div(g.C, per_row), make_fast_div(g.Sw, g.W + g.Kw + g.Sw));
+        auto kern = vec ? min_pool_backward_kernel<4> : min_pool_backward_kernel<1>;
+        hipLaunchKernelGGL(kern, grid, dim3(256), 0, stream, gy, arg, dx, (int)g.H, (int)g.W, (int)g.C, (int)g.Kh,
+                           (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.pad_top, (int)g.pad_left, (int)g.Nh, (int)g.Nw,
+                           make_fast_div(g.C, per_row), make_fast_div(g.Sw, g.W + g.Kw + g.Sw));
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
