@@ -197,8 +197,9 @@ int launch_sort(const SegmentSource& src, int64_t S, float* sorted, int32_t* per
     if (I <= 128)  return launch_sort_t<2, 64>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
     if (I <= 256)  return launch_sort_t<4, 64>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
     if (I <= 512)  return launch_sort_t<8, 64>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
-    // few long segments (a dense batch): four wavefronts per segment instead of one fill the chip
-    if (I <= 1024 && I > 512 && S < 2048) return launch_sort_t<4, 256>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
+    // few long segments (a dense batch): eight wavefronts per segment instead of one fill the chip
+    // (B = 256 rows of 800: 10.7 us against 11.6 us with four, 11.8 us with sixteen)
+    if (I <= 1024 && I > 512 && S < 2048) return launch_sort_t<2, 512>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
     if (I <= 1024) return launch_sort_t<16, 64>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
     if (I <= 2048) return launch_sort_t<8, 256>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
     if (I <= 4096) return launch_sort_t<8, 512>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
