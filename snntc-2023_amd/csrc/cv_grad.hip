@@ -221,13 +221,16 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
 constexpr int DWW_RI = 32;
 
 // FULL: every block has all DWW_RI rows (Kw*C is a multiple of it); the partial-block code is left out.
-template <bool FULL>
+// R: rows a block works on (DWW_RI, or the multiple of 8 above Kw*C for layers whose kernel rows are
+// shorter than that, e.g. 24 for a 7x7 stem on 3 channels: rows past the block's last one cost
+// instructions like any other).
+template <bool FULL, int R>
 __global__ void __launch_bounds__(256)
 cv_grad_weight_wide_kernel(const float* __restrict__ xpad, const float* __restrict__ upm,
                            const float* __restrict__ ym, float* __restrict__ dst, int S, int Kc, int rows,
                            int seg_per_slice, int H, int W, int C, int Kw, int Sh, int Sw, int Nh, int Nw,
                            int bias_row, float biasvolt, int s_safe, float neg_s, float post) {
-    __shared__ float red[3][DWW_RI + 1][kWave];
+    __shared__ float red[3][R + 1][kWave];
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int j = blockIdx.x * kWave + lane;
@@ -245,9 +248,9 @@ cv_grad_weight_wide_kernel(const float* __restrict__ xpad, const float* __restri
     const int s_lo = s_begin + wave * per_wave;
     const int s_hi = min(s_end, s_lo + per_wave);
 
-    float acc[DWW_RI];
+    float acc[R];
 #pragma unroll
-    for (int r = 0; r < DWW_RI; ++r) acc[r] = 0.0f;
+    for (int r = 0; r < R; ++r) acc[r] = 0.0f;
     // the block of rows 0..31 also carries the bias row (x = biasvolt for every patch)
     const bool with_bias = bias_row >= 0 && blockIdx.y == 0;
     float acc_bias = 0.0f;
@@ -267,20 +270,20 @@ cv_grad_weight_wide_kernel(const float* __restrict__ xpad, const float* __restri
         const float* yp = ym + (size_t)s_lo * Kc + jc;
         const float* up = upm + (size_t)s_lo * Kc + jc;
         float y_next = *yp, u_next = *up;
-        const int s_fast = (FULL || n_rows == DWW_RI) ? s_hi : min(s_hi, s_safe);
+        const int s_fast = (FULL || n_rows == R) ? s_hi : min(s_hi, s_safe);
         for (int s = s_lo; s < s_hi; ++s) {
             const float yv = y_next * -neg_s, uv = u_next;
             if (s + 1 < s_hi) { yp += Kc; up += Kc; }
             y_next = *yp; u_next = *up;
             if (FULL || s < s_fast) {
 #pragma unroll
-                for (int r = 0; r < DWW_RI; ++r) acc[r] = __fmaf_rn(scaled_lead(xb[r], neg_s, yv), uv, acc[r]);
+                for (int r = 0; r < R; ++r) acc[r] = __fmaf_rn(scaled_lead(xb[r], neg_s, yv), uv, acc[r]);
             } else {
                 // A block at the end of a kernel row fetches past its rows (the values are discarded),
                 // except for the last few patches of the tensor, where that fetch could leave it: there
                 // the unused rows re-read the block's last row.
 #pragma unroll
-                for (int r = 0; r < DWW_RI; ++r)
+                for (int r = 0; r < R; ++r)
                     acc[r] = __fmaf_rn(scaled_lead(xb[min(r, n_rows - 1)], neg_s, yv), uv, acc[r]);
             }
             if (with_bias) acc_bias = __fmaf_rn(scaled_lead(biasvolt, neg_s, yv), uv, acc_bias);
@@ -293,20 +296,20 @@ cv_grad_weight_wide_kernel(const float* __restrict__ xpad, const float* __restri
     }
     if (wave > 0) {
 #pragma unroll
-        for (int r = 0; r < DWW_RI; ++r) red[wave - 1][r][lane] = acc[r];
-        red[wave - 1][DWW_RI][lane] = acc_bias;
+        for (int r = 0; r < R; ++r) red[wave - 1][r][lane] = acc[r];
+        red[wave - 1][R][lane] = acc_bias;
     }
     __syncthreads();
     if (wave == 0 && j < Kc) {
         float* out = dst + (size_t)blockIdx.z * rows * Kc;
 #pragma unroll
-        for (int r = 0; r < DWW_RI; ++r)
+        for (int r = 0; r < R; ++r)
             if (r < n_rows)
                 out[(size_t)(i0 + r) * Kc + j] =
                     (((acc[r] + red[0][r][lane]) + red[1][r][lane]) + red[2][r][lane]) * post;
         if (with_bias)
             out[(size_t)bias_row * Kc + j] =
-                (((acc_bias + red[0][DWW_RI][lane]) + red[1][DWW_RI][lane]) + red[2][DWW_RI][lane]) * post;
+                (((acc_bias + red[0][R][lane]) + red[1][R][lane]) + red[2][R][lane]) * post;
     }
 }
 
@@ -386,7 +389,7 @@ cv_grad_weight_narrow_kernel(const float* __restrict__ xpad, const float* __rest
             const float yv = ym[(size_t)sc * Kc + jc];
             const float uv = have ? upm[(size_t)sc * Kc + jc] : 0.0f;
             dw_rows16(acc, 0, x0, yv, uv);
-            dw_rows16(acc, 16, x1, yv, uv);
+            if (n_rows > 16) dw_rows16(acc, 16, x1, yv, uv);     // block-uniform
             if (with_bias) acc_bias = __fmaf_rn(fminf(biasvolt - yv, 0.0f), uv, acc_bias);
             s += 2;
             if (s < s_hi) {                               // a lane past its last patch keeps pointing at it
@@ -488,8 +491,13 @@ int launch_cv_grad_weight_wide(const float* xpad, const float* upm, const float*
         KernelTimerScope timer_("grad_weight", stream);
         const bool full = (g.Kw * g.C) % DWW_RI == 0;
         const LeadScale ls = lead_scale(np.max_time);
-        hipLaunchKernelGGL(g.Kc <= 32 ? cv_grad_weight_narrow_kernel
-                           : full ? cv_grad_weight_wide_kernel<true> : cv_grad_weight_wide_kernel<false>, grid, dim3(256), 0,
+        // layers whose kernel rows are shorter than a block: work on the multiple of 8 rows above Kw*C
+        const int64_t kwc = g.Kw * g.C;
+        auto wide = full ? cv_grad_weight_wide_kernel<true, DWW_RI> : cv_grad_weight_wide_kernel<false, DWW_RI>;
+        if (kwc <= 8) wide = cv_grad_weight_wide_kernel<false, 8>;
+        else if (kwc <= 16) wide = cv_grad_weight_wide_kernel<false, 16>;
+        else if (kwc <= 24) wide = cv_grad_weight_wide_kernel<false, 24>;
+        hipLaunchKernelGGL(g.Kc <= 32 ? cv_grad_weight_narrow_kernel : wide, grid, dim3(256), 0,
                            stream, xpad, upm, ym, dst, (int)g.S, (int)g.Kc, (int)rows, seg_per_slice, (int)g.H,
                            (int)g.W, (int)g.C, (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.Nh, (int)g.Nw,
                            np.bias ? (int)g.P : -1, np.biasvolt, (int)s_safe, ls.neg_s, ls.post);
