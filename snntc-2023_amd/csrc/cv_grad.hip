@@ -119,18 +119,22 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
             for (int kc0 = ks * kc_share; kc0 < (ks + 1) * kc_share; kc0 += KCB) {
                 // stage the patch row: slots whose patch does not exist are never read
                 __builtin_amdgcn_wave_barrier();
-                // loads of STAGE slots are issued together: one slot at a time would cost a memory
-                // latency per slot, and nothing of this wavefront overlaps with it
-                constexpr int STAGE = 6;
-                for (int d0 = 0; d0 < n_slots; d0 += STAGE) {
+                // The loads of a round are issued together: one slot at a time would cost a memory
+                // latency per slot, and nothing of this wavefront overlaps with it.  A round covers
+                // STAGE * (64 / KCB) slots -- with fewer than 64 output channels per slot the lanes
+                // share out neighbouring slots -- which is the whole row for a 3-wide kernel.
+                constexpr int STAGE = 10, PER = kWave / KCB;
+                const int sub = lane / KCB, kcl = lane - sub * KCB;
+                for (int d0 = 0; d0 < n_slots; d0 += STAGE * PER) {
                     float yv[STAGE], uv[STAGE];
                     bool have[STAGE];
 #pragma unroll
                     for (int k = 0; k < STAGE; ++k) {
-                        const int ww = w0 - Kw + 1 + d0 + k;
-                        have[k] = d0 + k < n_slots && ww >= 0 && ww % Sw == 0 && ww / Sw < Nw && lane < KCB;
+                        const int d = d0 + k * PER + sub;
+                        const int ww = w0 - Kw + 1 + d;
+                        have[k] = d < n_slots && ww >= 0 && ww % Sw == 0 && ww / Sw < Nw;
                         if (have[k]) {
-                            const size_t so = (row0 + ww / Sw) * Kc + kc0 + lane;
+                            const size_t so = (row0 + ww / Sw) * Kc + kc0 + kcl;
                             yv[k] = ym[so];
                             uv[k] = upm[so];
                         }
@@ -138,8 +142,9 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
 #pragma unroll
                     for (int k = 0; k < STAGE; ++k) {
                         if (have[k]) {
-                            ys[(d0 + k) * KCB + lane] = yv[k];
-                            us[(d0 + k) * KCB + lane] = uv[k];
+                            const int d = d0 + k * PER + sub;
+                            ys[d * KCB + kcl] = yv[k];
+                            us[d * KCB + kcl] = uv[k];
                         }
                     }
                 }
