@@ -75,6 +75,16 @@ SNNTC_API const char* snntc_last_error(void);
 SNNTC_API const char* snntc_status_string(int status);
 
 /* ---------------------------------------------------------------------------------------------
+ * One-time set-up of a device (no counterpart in the reference, whose kernels need none).  Raises the
+ * dynamic-LDS limit of every kernel instantiation and looks up the device's copy of the library's
+ * static scratch array.  device < 0 means the current device.  Optional: every entry point performs
+ * the same set-up on its first call on a device -- but that first call must then not happen while a
+ * stream is being captured into a HIP graph (hipFuncSetAttribute is not allowed there).  A caller
+ * that captures graphs calls snntc_init() once per device beforehand, or runs one un-captured call.
+ * ------------------------------------------------------------------------------------------- */
+SNNTC_API int snntc_init(int device);
+
+/* ---------------------------------------------------------------------------------------------
  * Dense layer (SNN_dense).   x[B,I]   w[w_rows,J] with w_rows == I + (biasvolt > 1e-8)
  * ------------------------------------------------------------------------------------------- */
 
@@ -102,6 +112,20 @@ SNNTC_API int snntc_fc_forward_ex(const float* x, const float* w, const float* p
                         float* sorted_z, int32_t* perm, int32_t* causal_k,
                         int64_t B, int64_t I, int64_t J, int64_t w_rows,
                         void* workspace, size_t workspace_bytes, void* stream);
+
+/* snntc_fc_forward for callers that cannot allocate device memory or carry a workspace: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart
+ * in the reference (whose ops allocate their temporaries through the framework on every call).
+ * Same results as snntc_fc_forward, bit for bit; the scratch (sorted rows, permutation, counts)
+ * lives in a static device array of SNNTC_STATIC_SCRATCH_BYTES inside the library, which every GPU
+ * the library runs on holds until the process ends.  The call allocates and frees nothing.
+ * Limits: snntc_fc_forward_workspace_bytes(B, I, J) must not exceed SNNTC_STATIC_SCRATCH_BYTES
+ * (e.g. B = 1024 rows of I = 784), else SNNTC_ERR_WORKSPACE.  All calls on one GPU share that GPU's
+ * array: calls that overlap in time on the same GPU (two streams, two threads) race; serialise them. */
+#define SNNTC_STATIC_SCRATCH_BYTES (8u << 20)
+SNNTC_API size_t snntc_static_scratch_bytes(void);
+SNNTC_API int snntc_fc_forward_static(const float* x, const float* w, const float* params_host, float* out,
+                            int64_t B, int64_t I, int64_t J, int64_t w_rows, void* stream);
 
 /* grad[grad_rows,J] (only rows [0,B) are read, so a buffer holding just those rows may be passed with
  * grad_rows still declared as 2B), oldout[2B,J] = the forward output.

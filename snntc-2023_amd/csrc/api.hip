@@ -12,6 +12,11 @@
 
 #include "snntc_common.h"
 
+// Library-owned scratch of snntc_fc_forward_static (the entry point that allocates nothing): held by
+// every GPU the library runs on until the process ends.  Host code never passes this name to a
+// kernel; it asks hipGetSymbolAddress for the device's copy once (prepare_device below).
+static __device__ __align__(256) unsigned char scratch[SNNTC_STATIC_SCRATCH_BYTES];
+
 namespace snntc {
 
 static thread_local char g_last_error[512] = "";
@@ -275,6 +280,35 @@ int cv_forward_impl(const float* xpad, const float* w, const float* params, floa
                        st);
 }
 
+
+// ---- per-device one-time set-up and the library-owned scratch of snntc_fc_forward_static ----------
+// `scratch` is the forward workspace of the allocation-free entry point.  In host code the array's
+// name is only a handle for hipGetSymbolAddress: the device address (each GPU holds its own copy)
+// is looked up once per device and kept in g_scratch_ptr; host code uses that pointer, never the name.
+constexpr size_t kStaticScratchBytes = SNNTC_STATIC_SCRATCH_BYTES;
+
+std::mutex g_init_mutex;
+void* g_scratch_ptr[kMaxDevices];          // device address of `scratch` on each device, NULL until set up
+
+// Set-up of the current device `dev`: dynamic-LDS limits of all kernels and the address of `scratch`.
+int prepare_device(int dev, void** scratch_out) {
+    if (dev < 0 || dev >= kMaxDevices)
+        return fail(SNNTC_ERR_UNSUPPORTED, "snntc_init: device index %d not supported", dev);
+    std::lock_guard<std::mutex> lock(g_init_mutex);
+    if (!g_scratch_ptr[dev]) {
+        int rc = scan_prepare_device(dev, nullptr);
+        if (!rc) rc = merge_prepare_device(dev);
+        if (rc) return rc;
+        void* ptr = nullptr;
+        SNNTC_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(::scratch)));
+        if (!ptr || reinterpret_cast<uintptr_t>(ptr) % kAlign != 0)
+            return fail(SNNTC_ERR_HIP, "snntc_init: the static scratch array has no usable device address");
+        g_scratch_ptr[dev] = ptr;
+    }
+    if (scratch_out) *scratch_out = g_scratch_ptr[dev];
+    return SNNTC_OK;
+}
+
 }  // namespace
 }  // namespace snntc
 
@@ -453,6 +487,39 @@ int snntc_fc_forward_ex(const float* x, const float* w, const float* params_host
                         int64_t w_rows, void* workspace, size_t workspace_bytes, void* stream) {
     return fc_forward_impl(x, w, params_host, out, sorted_z, perm, causal_k, B, I, J, w_rows, workspace,
                            workspace_bytes, stream);
+}
+
+int snntc_init(int device) {
+    int current = 0;
+    SNNTC_HIP_CHECK(hipGetDevice(&current));
+    if (device < 0 || device == current) return prepare_device(current, nullptr);
+    SNNTC_HIP_CHECK(hipSetDevice(device));                 // the set-up needs its device current
+    const int rc = prepare_device(device, nullptr);
+    SNNTC_HIP_CHECK(hipSetDevice(current));
+    return rc;
+}
+
+size_t snntc_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int snntc_fc_forward_static(const float* x, const float* w, const float* params_host, float* out, int64_t B,
+                            int64_t I, int64_t J, int64_t w_rows, void* stream) {
+    int rc = fc_check(B, I, J, w_rows, params_host, "snntc_fc_forward_static");
+    if (rc) return rc;
+    const size_t need = fc_fwd_ws(nullptr, B, I).bytes;
+    if (need > kStaticScratchBytes)
+        return fail(SNNTC_ERR_WORKSPACE,
+                    "snntc_fc_forward_static: B=%lld, I=%lld needs %zu bytes of scratch, the library holds %zu "
+                    "(use snntc_fc_forward with a workspace of your own)",
+                    (long long)B, (long long)I, need, kStaticScratchBytes);
+    int dev = 0;
+    SNNTC_HIP_CHECK(hipGetDevice(&dev));
+    void* ws = nullptr;
+    rc = prepare_device(dev, &ws);           // first call on a device: look up this device's copy of the array
+    if (rc) return rc;
+    // every byte of the workspace the scan reads is written by the sort of this call (padding entries
+    // of the rows included), so nothing needs clearing between calls
+    return fc_forward_impl(x, w, params_host, out, nullptr, nullptr, nullptr, B, I, J, w_rows, ws,
+                           kStaticScratchBytes, stream);
 }
 
 int snntc_fc_backward(const float* grad, const float* x, const float* w, const float* params_host,

@@ -298,6 +298,22 @@ bool merge_sort_supported(const ConvGeom& g) {
     return merge_lds_bytes((int)g.C, (int)g.Kh, (int)g.Kw, (int)g.Sw, tw) <= MERGE_LDS_CAP && tw >= 2;
 }
 
+// One-time set-up on device `dev` (the current device): the dynamic-LDS limit of every
+// instantiation, so that no later launch calls hipFuncSetAttribute (not allowed during capture).
+int merge_prepare_device(int dev) {
+    static std::atomic<bool> done[kMaxDevices];
+    if (dev < 0 || dev >= kMaxDevices) return fail(SNNTC_ERR_UNSUPPORTED, "patch merge: device index %d not supported", dev);
+    if (done[dev].load(std::memory_order_acquire)) return SNNTC_OK;
+    const void* kernels[] = {reinterpret_cast<const void*>(merge_patches_kernel<1>),
+                             reinterpret_cast<const void*>(merge_patches_kernel<2>),
+                             reinterpret_cast<const void*>(merge_patches_kernel<3>),
+                             reinterpret_cast<const void*>(merge_patches_kernel<4>)};
+    for (const void* k : kernels)
+        SNNTC_HIP_CHECK(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)MERGE_LDS_CAP));
+    done[dev].store(true, std::memory_order_release);
+    return SNNTC_OK;
+}
+
 int launch_merge_patches(const float* pix_z, const int32_t* pix_c, int64_t Cs, float* sorted, int32_t* perm,
                          int32_t* n_real, const ConvGeom& g, int64_t stride, float max_cmp,
                          hipStream_t stream) {
@@ -311,15 +327,10 @@ int launch_merge_patches(const float* pix_z, const int32_t* pix_c, int64_t Cs, f
     const int eb = per_lane >= 4 ? 4 : (int)per_lane;
     auto kern = eb == 1 ? merge_patches_kernel<1> : eb == 2 ? merge_patches_kernel<2>
               : eb == 3 ? merge_patches_kernel<3> : merge_patches_kernel<4>;
-    static std::atomic<bool> lds_limit_raised[kMaxDevices][5];     // once per device and instantiation
     int dev = 0;
     SNNTC_HIP_CHECK(hipGetDevice(&dev));
-    if (dev < 0 || dev >= kMaxDevices) return fail(SNNTC_ERR_UNSUPPORTED, "patch merge: device index %d not supported", dev);
-    if (!lds_limit_raised[dev][eb].load(std::memory_order_acquire)) {
-        SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)MERGE_LDS_CAP));
-        lds_limit_raised[dev][eb].store(true, std::memory_order_release);
-    }
+    const int prep = merge_prepare_device(dev);
+    if (prep) return prep;
     {
         KernelTimerScope timer_("merge_patches", stream);
         hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(MERGE_THREADS), lds, stream, pix_z, pix_c, (int)Cs,

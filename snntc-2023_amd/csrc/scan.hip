@@ -904,22 +904,57 @@ unpad_rows_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ 
 
 }  // namespace
 
+namespace {
+template <int COLS>
+int raise_scan_lds_limits() {
+    const void* whole[] = {
+        reinterpret_cast<const void*>(scan_lds_kernel<COLS, true, true>),
+        reinterpret_cast<const void*>(scan_lds_kernel<COLS, false, true>),
+        reinterpret_cast<const void*>(scan_lds_kernel<COLS, true, false>),
+        reinterpret_cast<const void*>(scan_lds_kernel<COLS, false, false>),
+        reinterpret_cast<const void*>(scan_lds_multi_kernel<COLS, 2, true>),
+        reinterpret_cast<const void*>(scan_lds_multi_kernel<COLS, 2, false>)};
+    for (const void* k : whole)
+        SNNTC_HIP_CHECK(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_SCAN_BYTES));
+    const void* split[] = {reinterpret_cast<const void*>(scan_lds_split_kernel<COLS, true>),
+                           reinterpret_cast<const void*>(scan_lds_split_kernel<COLS, false>)};
+    for (const void* k : split)
+        SNNTC_HIP_CHECK(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                            LDS_SCAN_BYTES - SPLIT_STATIC_LDS));
+    return SNNTC_OK;
+}
+}  // namespace
+
+// One-time set-up of the scan on device `dev` (which must be the current device): the CU count and
+// the dynamic-LDS limit of EVERY instantiation, so that no later launch, whatever its shape, has
+// to call hipFuncSetAttribute (which is not allowed while a stream is being captured).
+int scan_prepare_device(int dev, int* cu_count_out) {
+    static std::atomic<int> cu_count[kMaxDevices];
+    if (dev < 0 || dev >= kMaxDevices) return fail(SNNTC_ERR_UNSUPPORTED, "scan: device index %d not supported", dev);
+    int cus = cu_count[dev].load(std::memory_order_acquire);
+    if (cus == 0) {
+        hipDeviceProp_t prop;
+        SNNTC_HIP_CHECK(hipGetDeviceProperties(&prop, dev));
+        int rc = raise_scan_lds_limits<64>();
+        if (!rc) rc = raise_scan_lds_limits<32>();
+        if (!rc) rc = raise_scan_lds_limits<16>();
+        if (!rc) rc = raise_scan_lds_limits<8>();
+        if (rc) return rc;
+        cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+        cu_count[dev].store(cus, std::memory_order_release);
+    }
+    if (cu_count_out) *cu_count_out = cus;
+    return SNNTC_OK;
+}
+
 template <int COLS>
 int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_real, const float* w, float* y,
                     float* rcp, int32_t* causal_k, int64_t S, int64_t I, int64_t stride, int64_t J,
                     const NeuronParams& np, size_t lds_bytes, hipStream_t stream) {
-    // per device: CU count, and whether the dynamic-LDS limit of the instantiations was raised
-    static std::atomic<int> cu_count[kMaxDevices];
-    int dev = 0;
+    int dev = 0, cus = 0;
     SNNTC_HIP_CHECK(hipGetDevice(&dev));
-    if (dev < 0 || dev >= kMaxDevices) return fail(SNNTC_ERR_UNSUPPORTED, "scan: device index %d not supported", dev);
-    int cus = cu_count[dev].load(std::memory_order_relaxed);
-    if (cus == 0) {
-        hipDeviceProp_t prop;
-        SNNTC_HIP_CHECK(hipGetDeviceProperties(&prop, dev));
-        cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-        cu_count[dev].store(cus, std::memory_order_relaxed);
-    }
+    const int prep = scan_prepare_device(dev, &cus);
+    if (prep) return prep;
     constexpr int SEGS = kWave / COLS;
     const int n_slices = (int)((J + COLS - 1) / COLS);
     const int64_t items = (S + SEGS - 1) / SEGS;
@@ -961,18 +996,6 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     auto kern = split ? scan_lds_split_kernel<COLS, false>
                 : low_latency ? scan_lds_kernel<COLS, false, true>
                 : multi ? scan_lds_multi_kernel<COLS, CH, false> : scan_lds_kernel<COLS, false, false>;
-    // raise the dynamic-LDS limit of both instantiations once (not per launch: the call is not
-    // allowed while a stream is being captured into a graph)
-    static std::atomic<bool> lds_limit_raised[kMaxDevices][4];
-    const int variant = split ? 3 : low_latency ? 1 : (multi ? 2 : 0);
-    const int lds_limit = split ? LDS_SCAN_BYTES - SPLIT_STATIC_LDS : LDS_SCAN_BYTES;
-    if (!lds_limit_raised[dev][variant].load(std::memory_order_acquire)) {
-        SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern_k),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_limit));
-        SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_limit));
-        lds_limit_raised[dev][variant].store(true, std::memory_order_release);
-    }
     dim3 grid((unsigned)(n_slices * n_groups)), block((unsigned)(split ? LOW_LATENCY_THREADS : WAVES * kWave));
     {
         KernelTimerScope timer_("scan", stream);

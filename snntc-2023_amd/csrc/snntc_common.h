@@ -120,6 +120,12 @@ int launch_scan(const float* sorted, const int32_t* perm, const int32_t* n_real,
                 float* rcp, int32_t* causal_k, int64_t S, int64_t I, int64_t stride, int64_t J,
                 const NeuronParams& np, hipStream_t stream);
 
+// One-time set-up on device `dev`, which must be the current device: the dynamic-LDS limits of every
+// scan / merge instantiation (and the CU count the scan sizes its launches with).  The launchers call
+// them on their first use of a device; snntc_init() calls them ahead of time.
+int scan_prepare_device(int dev, int* cu_count_out);
+int merge_prepare_device(int dev);
+
 // upm = valid ? grad*rcp : 0 ; ym = valid ? y : -inf   (valid: y <= MAX-0.1), n elements each, and,
 // in the same launch, the weight copy dX reads from: mode 0 none, mode 1
 // wt[cols, rows] = w[rows, cols]^T, mode 2 the regrouped copy of a conv layer's weights

@@ -21,7 +21,8 @@ ERR_HIP = 6
 
 #: every symbol include/snntc.h declares
 EXPORTS = (
-    "snntc_version", "snntc_last_error", "snntc_status_string",
+    "snntc_version", "snntc_last_error", "snntc_status_string", "snntc_init",
+    "snntc_static_scratch_bytes", "snntc_fc_forward_static",
     "snntc_fc_forward_workspace_bytes", "snntc_fc_backward_workspace_bytes",
     "snntc_fc_forward", "snntc_fc_forward_ex", "snntc_fc_backward",
     "snntc_cv_output_dims", "snntc_cv_forward_workspace_bytes", "snntc_cv_backward_workspace_bytes",
@@ -77,6 +78,9 @@ def load():
     lib.snntc_last_error.restype = c.c_char_p
     lib.snntc_status_string.restype = c.c_char_p
     lib.snntc_status_string.argtypes = [c.c_int]
+    lib.snntc_init.argtypes = [c.c_int]
+    lib.snntc_static_scratch_bytes.argtypes = []
+    lib.snntc_fc_forward_static.argtypes = [vp, vp, fparams, vp, i64, i64, i64, i64, vp]
     lib.snntc_fc_forward_workspace_bytes.argtypes = [i64, i64, i64, c.POINTER(sz)]
     lib.snntc_fc_backward_workspace_bytes.argtypes = [i64, i64, i64, c.POINTER(sz)]
     lib.snntc_fc_forward.argtypes = [vp, vp, fparams, vp, i64, i64, i64, i64, vp, sz, vp]
@@ -99,8 +103,9 @@ def load():
     lib.snntc_profile_collect.argtypes = []
     lib.snntc_profile_entry.argtypes = [c.c_int, c.POINTER(c.c_char_p), c.POINTER(i64), c.POINTER(c.c_double)]
     for name in EXPORTS:
-        if name not in ("snntc_version", "snntc_last_error", "snntc_status_string"):
+        if name not in ("snntc_version", "snntc_last_error", "snntc_status_string", "snntc_static_scratch_bytes"):
             getattr(lib, name).restype = c.c_int
+    lib.snntc_static_scratch_bytes.restype = sz
     _lib = lib
     return lib
 

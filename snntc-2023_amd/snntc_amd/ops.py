@@ -85,6 +85,37 @@ def snnfc(X, W, Params, return_aux=False):
     return out
 
 
+def init(device=None):
+    """One-time set-up of a device (kernel attributes, the library's static scratch): call it before
+    capturing library calls into a HIP graph.  device=None means the current device."""
+    lib = _lib.load()
+    if device is None:
+        index = -1
+    else:
+        index = torch.device(device).index
+        index = torch.cuda.current_device() if index is None else index
+    _lib.check(lib.snntc_init(index))
+
+
+def snnfc_static(X, W, Params, out=None):
+    """snnfc through the entry point that allocates nothing: the scratch is a static device array
+    inside the library (snntc_static_scratch_bytes()).  `out` may be a preallocated [2B,J] tensor.
+    Calls on one GPU share that array: do not overlap them."""
+    lib = _lib.load()
+    X = _dev_f32(X, "X", 2)
+    W = _dev_f32(W, "W", 2)
+    p, pp = _params(Params, 6)
+    B, I = X.shape
+    w_rows, J = W.shape
+    with torch.cuda.device(X.device):
+        if out is None:
+            out = torch.empty((2 * B, J), dtype=torch.float32, device=X.device)
+        elif tuple(out.shape) != (2 * B, J) or out.dtype != torch.float32 or not out.is_contiguous():
+            raise ValueError(f"out must be a contiguous float32 [{2 * B},{J}] tensor")
+        _lib.check(lib.snntc_fc_forward_static(_ptr(X), _ptr(W), pp, _ptr(out), B, I, J, w_rows, _stream(X.device)))
+    return out
+
+
 def snnfc_grad(grad, X, W, Params, Y, want_dparams=True, want_dx=True, want_dw=True, first_half_grad=False):
     """Dense backward.  grad[2B,J], Y[2B,J] = forward output -> (dX[B,I], dW like W, dParams[6]).
     dParams is all zeros (Params is a constant).  A want_* flag set to False skips that gradient

@@ -19,7 +19,7 @@ def lib():
 
 def _declared_symbols():
     text = open(os.path.join(ROOT, "include", "snntc.h")).read()
-    return re.findall(r"SNNTC_API\s+(?:const\s+char\s*\*|int)\s+(snntc_\w+)\s*\(", text)
+    return re.findall(r"SNNTC_API\s+(?:const\s+char\s*\*|int|size_t)\s+(snntc_\w+)\s*\(", text)
 
 
 def test_header_and_loader_list_the_same_symbols():
