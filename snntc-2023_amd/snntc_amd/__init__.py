@@ -8,10 +8,12 @@ from . import _lib
 from ._lib import SnntcError, SnntcLibraryError
 from .ops import SnnCv, SnnCvTimes, SnnFc, SnnFcTimes, SnnMinPool, SnnPadTime, SoftmaxTimeLoss, min_pool, min_pool_grad, pad_time, pad_time_grad, sgd_update, softmax_time_loss, snncv, snncv_grad, snncv_output_dims, snnfc, snnfc_grad, snnfc_static, init
 from . import train
-from .layers import (SNN_LRN, SNN_avgpool2d, SNN_conv, SNN_dense, SNN_maxpool2d, init_weight, loss_func)
+from . import networks
+from .layers import (SNN_LRN, SNN_avgpool2d, SNN_conv, SNN_dense, SNN_flatten, SNN_globalminpool2d, SNN_maxpool2d,
+                     init_weight, loss_func)
 
 __all__ = [
     "snnfc", "snnfc_grad", "snnfc_static", "init", "snncv", "snncv_grad", "snncv_output_dims", "SnnFc", "SnnCv", "SnnFcTimes", "SnnCvTimes", "SoftmaxTimeLoss", "softmax_time_loss", "sgd_update", "SnnMinPool", "min_pool", "min_pool_grad", "SnnPadTime", "pad_time", "pad_time_grad",
-    "SNN_dense", "SNN_conv", "SNN_maxpool2d", "SNN_avgpool2d", "SNN_LRN", "init_weight", "loss_func",
-    "SnntcError", "SnntcLibraryError", "train",
+    "SNN_dense", "SNN_conv", "SNN_maxpool2d", "SNN_avgpool2d", "SNN_globalminpool2d", "SNN_flatten", "SNN_LRN", "init_weight", "loss_func",
+    "SnntcError", "SnntcLibraryError", "train", "networks",
 ]

@@ -207,6 +207,33 @@ class SNN_maxpool2d(_Pool2d):
         return y.permute(0, 2, 3, 1)
 
 
+class SNN_globalminpool2d(torch.nn.Module):
+    """Global earliest-spike pooling, [B,H,W,C] -> [B,C]: every channel keeps its first spike over the
+    whole image.  It is SNN_maxpool2d with one VALID window the size of the image; the reference's
+    ImageNet example reduces with a stock global pooling layer at this place
+    (snntc-imagenet-example/snntc-imagenet.py:125)."""
+
+    def __init__(self, padvalue=1e5, name=None):
+        super().__init__()
+        self.padvalue = padvalue
+        self.name = name
+
+    def forward(self, input):
+        B, H, W, C = input.shape
+        if input.is_cuda and input.dtype == torch.float32:
+            y = SnnMinPool.apply(input.contiguous(), (H, W), (H, W), (0, 0), (1, 1), float(self.padvalue))
+            return y.reshape(B, C)
+        return input.amin(dim=(1, 2))                       # host tensors: the definition itself
+
+
+class SNN_flatten(torch.nn.Module):
+    """[B,H,W,C] -> [B,H*W*C] in NHWC order, what Keras' Flatten does between the reference's conv and
+    dense layers (tf.reshape in snntc-cifar10.py:105)."""
+
+    def forward(self, input):
+        return input.reshape(input.shape[0], -1)
+
+
 class SNN_avgpool2d(_Pool2d):
     """Average pooling after padding with 1e5 (SNN_TC_Modules.py:251-281)."""
 

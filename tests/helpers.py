@@ -66,3 +66,11 @@ def assert_close(actual, expected, rtol=1e-5, atol=1e-6, what=""):
         idx = np.unravel_index(np.argmax(err - lim), err.shape)
         raise AssertionError(f"{what}: {bad.sum()} of {bad.size} elements out of tolerance; worst at {idx}: "
                              f"got {a[idx]!r}, want {e[idx]!r}, |diff| {err[idx]:.3e} > {lim[idx]:.3e}")
+
+
+def grad_band(ref, ref_abs, depth=1):
+    """Tolerance of a gradient entry that is an fp32 sum: rel 1e-5 / abs 1e-6 of the value, plus
+    5e-7 (about 8 ulp) of the sum of the magnitudes of its summands, `ref_abs` -- two fp32 summation
+    orders of the same terms differ by a multiple of that, whatever the size of the sum itself.
+    `depth` widens the band for errors carried through that many layers."""
+    return depth * (1e-5 * np.abs(ref) + 1e-6 * np.maximum(1.0, 0.5 * np.abs(ref_abs)))

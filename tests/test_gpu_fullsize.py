@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import conv_case, dense_case
+from helpers import conv_case, dense_case, grad_band
 from oracle import capi
 
 pytestmark = pytest.mark.gpu
@@ -68,9 +68,12 @@ def test_dense_north_star_layer_full_batch():
     oabs = out.clone(); oabs[256:] = oabs[256:].abs()
     _, dw_mag, _ = snn.snnfc_grad(G.abs(), X, W, p, oabs)               # = -sum |x - y| |up|
     assert torch.all((dwa + dwb - dw).abs() <= 1e-5 * dw.abs() + 1e-6 * dw_mag.abs().clamp(min=1.0))
-    rdx, _, _ = capi.fc_backward_dev(np.concatenate((g[:8], g[256:264])), x[:8], w, p,
-                                     np.concatenate((out[:8].cpu().numpy(), out[256:264].cpu().numpy())), wide=True)
-    assert np.all(np.abs(dx[:8].cpu().numpy() - rdx) <= 1e-5 * np.abs(rdx) + 1e-5)
+    g8 = np.concatenate((g[:8], g[256:264]))
+    o8 = np.concatenate((out[:8].cpu().numpy(), out[256:264].cpu().numpy()))
+    rdx, _, _ = capi.fc_backward_dev(g8, x[:8], w, p, o8, wide=True)
+    o8a = o8.copy(); o8a[8:] = np.abs(o8a[8:])
+    adx, _, _ = capi.fc_backward_dev(np.abs(g8), x[:8], np.abs(w), p, o8a, wide=True)     # sums of |summands|
+    assert np.all(np.abs(dx[:8].cpu().numpy() - rdx) <= grad_band(rdx, adx))
 
 
 def test_conv_north_star_layer_full_batch():
@@ -100,8 +103,10 @@ def test_conv_north_star_layer_full_batch():
     dx1, dw1, _ = snn.snncv_grad(g1, X[:1], W, p, o1)
     assert torch.equal(dx1[0], dx[0])
     rdx, rdw, _ = capi.cv_backward_dev(g1.cpu().numpy(), xpad[:1], w, p, o1.cpu().numpy(), wide=True)
-    assert np.all(np.abs(dx1.cpu().numpy() - rdx) <= 1e-5 * np.abs(rdx) + 1e-5)
-    assert np.all(np.abs(dw1.cpu().numpy() - rdw) <= 1e-5 * np.abs(rdw) + 1e-4)
+    o1a = o1.cpu().numpy().copy(); o1a[1] = np.abs(o1a[1])
+    adx, adw, _ = capi.cv_backward_dev(np.abs(g1.cpu().numpy()), xpad[:1], np.abs(w), p, o1a, wide=True)
+    assert np.all(np.abs(dx1.cpu().numpy() - rdx) <= grad_band(rdx, adx))
+    assert np.all(np.abs(dw1.cpu().numpy() - rdw) <= grad_band(rdw, adw))
     # dW of the batch = sum of per-image dW (computed by the same kernels on single images)
     acc = torch.zeros_like(dw, dtype=torch.float64)
     for b in range(0, B, 8):
@@ -119,12 +124,15 @@ LAYER_SHAPES = [
     ("cifar conv 3->32 @32",   128, 32,  32,  3,   32,  3, 1),
     ("cifar conv 32->32 @32",  128, 32,  32,  32,  32,  3, 1),
     ("cifar conv 32->64 @16",  128, 16,  16,  32,  64,  3, 1),
+    ("cifar conv 64->64 @16",  128, 16,  16,  64,  64,  3, 1),
     ("cifar conv 64->128 @8",  128, 8,   8,   64,  128, 3, 1),
     ("resnet stem 7x7/2",      32,  224, 224, 3,   64,  7, 2),
     ("resnet 64->64 @56",      32,  56,  56,  64,  64,  3, 1),
     ("resnet 64->128 @28",     32,  28,  28,  64,  128, 3, 1),
     ("resnet 128->128 @28",    32,  28,  28,  128, 128, 3, 1),
+    ("resnet 128->256 @14",    32,  14,  14,  128, 256, 3, 1),
     ("resnet 256->256 @14",    32,  14,  14,  256, 256, 3, 1),
+    ("resnet 256->512 @7",     32,  7,   7,   256, 512, 3, 1),
     ("resnet 512->512 @7",     32,  7,   7,   512, 512, 3, 1),
 ]
 
@@ -158,7 +166,63 @@ def test_conv_layer_shapes_of_the_baseline_networks(name, B, H, W, C, Kc, K, S):
     rdx, rdw, _ = capi.cv_backward_dev(g1.cpu().numpy(), xpad[b:b + 1], w, p, o1.cpu().numpy(), wide=True)
     o1a = o1.clone(); o1a[1] = o1a[1].abs()
     mdx, mdw, _ = snn.snncv_grad(g1.abs(), X[b:b + 1], Wt.abs(), p, o1a)      # sums of |summands|
-    tol_dx = 1e-5 * np.abs(rdx) + 1e-6 * np.maximum(1.0, np.abs(mdx.cpu().numpy()))
-    tol_dw = 1e-5 * np.abs(rdw) + 1e-6 * np.maximum(1.0, np.abs(mdw.cpu().numpy()))
+    tol_dx = grad_band(rdx, mdx.cpu().numpy())
+    tol_dw = grad_band(rdw, mdw.cpu().numpy())
     assert np.all(np.abs(dx1.cpu().numpy() - rdx) <= tol_dx)
     assert np.all(np.abs(dw1.cpu().numpy() - rdw) <= tol_dw)
+
+
+def literal_bar_statistics(actual, ref):
+    """Share of elements outside the literal bar |a - e| <= 1e-5 * |e| + 1e-6, and the worst ratio of
+    the error to that bar."""
+    a = np.asarray(actual, np.float64); e = np.asarray(ref, np.float64)
+    ratio = np.abs(a - e) / (1e-5 * np.abs(e) + 1e-6)
+    return float((ratio > 1.0).mean()), float(ratio.max())
+
+
+LITERAL_BAR_CASES = [
+    # name, kind, shape
+    ("dense 784->800 B=128 (config 1)", "dense", (128, 784, 800)),
+    ("conv 3x3 64->64 @32x32 B=16 (config 3 layer, a quarter of its batch)", "conv", (16, 32, 32, 64, 64)),
+]
+
+
+@pytest.mark.parametrize("name,kind,shape", LITERAL_BAR_CASES, ids=["config1", "config3"])
+def test_gradients_against_the_literal_tolerance(name, kind, shape):
+    """How the gradients stand against the literal bar rel 1e-5 / abs 1e-6 (no scaling by the size of the
+    sums), with the float64-accumulated oracle as the reference value: for the HIP result and for the
+    oracle run in the reference kernels' own fp32 sequential order.  Long fp32 sums cannot all meet the
+    literal bar in any order; the HIP result must not be worse than the reference's order on either count
+    (share of elements outside up to a factor of 1.5 and a floor of one element in a thousand, worst
+    excess up to a factor of 2)."""
+    import json
+    import os
+    import snntc_amd as snn
+    if kind == "dense":
+        B, I, J = shape
+        x, w, p, g = dense_case(0, B, I, J, True, "baseline")
+        out = capi.fc_forward_dev(x, w, p)
+        wide = capi.fc_backward_dev(g, x, w, p, out, wide=True)
+        seq = capi.fc_backward_dev(g, x, w, p, out)
+        dx, dw, _ = snn.snnfc_grad(t(g), t(x), t(w), p, t(out))
+    else:
+        B, H, C, Kc = shape[0], shape[1], shape[3], shape[4]
+        _, x, w, p, g = conv_case(0, B, H, H, C, Kc, 3, 3, 1, 1, True, True, "baseline")
+        out = capi.cv_forward_dev(x, w, p)
+        wide = capi.cv_backward_dev(g, x, w, p, out, wide=True)
+        seq = capi.cv_backward_dev(g, x, w, p, out)
+        dx, dw, _ = snn.snncv_grad(t(g), t(x), t(w), p, t(out))
+    torch.cuda.synchronize()
+    stats = {"case": name}
+    for label, got, ref, ref_seq in (("dX", dx, wide[0], seq[0]), ("dW", dw, wide[1], seq[1])):
+        share_hip, worst_hip = literal_bar_statistics(got.cpu().numpy(), ref)
+        share_seq, worst_seq = literal_bar_statistics(ref_seq, ref)
+        stats[label] = {"hip_share_outside": share_hip, "hip_worst_ratio": worst_hip,
+                        "fp32_sequential_share_outside": share_seq, "fp32_sequential_worst_ratio": worst_seq,
+                        "max_abs_ref": float(np.abs(ref).max())}
+        assert share_hip <= max(1.5 * share_seq, 1e-3), (label, stats[label])
+        assert worst_hip <= max(2.0 * worst_seq, 1.0), (label, stats[label])
+    print(json.dumps(stats))
+    if os.path.isdir("gpurun_out"):
+        with open(os.path.join("gpurun_out", f"literal_bar_{kind}.json"), "w") as f:
+            json.dump(stats, f, indent=1)

@@ -2,7 +2,7 @@
 kernel sizes, strides, SAME / VALID), non-default biasvolt / threshold / MAX, quantised inputs (heavy
 ties) and MAX sentinels among the inputs.  Same bars as test_gpu_parity: sorted values, permutations,
 causal-set sizes, spike times and reciprocals bit-exact against the oracle; gradients within
-1e-5 * |ref| + 1e-6 * max(1, sum of |summands|)."""
+1e-5 * |ref| + 1e-6 * max(1, half the sum of |summands|) (helpers.grad_band)."""
 import numpy as np
 import pytest
 import torch

@@ -65,6 +65,43 @@ def test_costs():
     assert abs(float(l.l2_cost().detach()) - float(np.mean(w ** 2))) < 1e-7
 
 
+def _cost_gradient_check(dev):
+    """Gradients of the weight-constraint costs against their closed forms (SNN_TC_Modules.py:77-84,
+    snntc-mnist.py:55-59): d/dw_ij mean_j max(0, theta - sum_i w_ij) = -1/J on columns whose sum lies
+    below the threshold and 0 elsewhere; d/dw mean(w^2) = 2 w / n; the constraint cost is
+    K * sum_l (first) + K2 * sum_l (second) over the layers of a model."""
+    from snntc_amd import train
+    rng = np.random.default_rng(11)
+    dense = snn.SNN_dense(40, 12, Spike_Threshold=1.5, weight=(rng.standard_normal((41, 12)) * 0.2 + 0.03).astype(np.float32))
+    conv = snn.SNN_conv(3, 7, 3, 1, 'SAME', weight=(rng.standard_normal((28, 7)) * 0.2 + 0.04).astype(np.float32))
+    model = torch.nn.Sequential(conv, dense).to(dev)
+    for layer, theta in ((dense, 1.5), (conv, 1.0)):
+        w = layer.weight.detach().cpu().numpy().astype(np.float64)
+        below = w.sum(0) < theta
+        assert below.any() and (~below).any(), "the draw should hold columns on both sides of the threshold"
+        (gw,) = torch.autograd.grad(layer.w_sum_cost(), layer.weight)
+        want = np.where(below, -1.0 / w.shape[1], 0.0)[None, :].repeat(w.shape[0], 0)
+        assert np.allclose(gw.cpu().numpy(), want, rtol=0, atol=1e-7)
+        (gl,) = torch.autograd.grad(layer.l2_cost(), layer.weight)
+        assert np.allclose(gl.cpu().numpy(), 2.0 * w / w.size, rtol=1e-6, atol=1e-9)
+    K, K2 = 100.0, 1e-2
+    grads = torch.autograd.grad(train.constraint_cost(model, K, K2), [conv.weight, dense.weight])
+    for layer, g in zip((conv, dense), grads):
+        w = layer.weight.detach().cpu().numpy().astype(np.float64)
+        below = w.sum(0) < 1.0                                  # constraint_cost uses 1.0 (snntc-mnist.py:57)
+        want = K * np.where(below, -1.0 / w.shape[1], 0.0)[None, :] + K2 * 2.0 * w / w.size
+        assert np.allclose(g.cpu().numpy(), want, rtol=1e-5, atol=1e-7)
+
+
+def test_cost_gradients_against_closed_forms():
+    _cost_gradient_check("cpu")
+
+
+@pytest.mark.gpu
+def test_cost_gradients_against_closed_forms_on_the_gpu():
+    _cost_gradient_check("cuda:0")
+
+
 def test_min_time_pool_and_avg_pool():
     x = torch.rand(2, 5, 7, 3) + 1
     mp = snn.SNN_maxpool2d(2, 2, 'SAME')

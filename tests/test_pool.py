@@ -76,6 +76,40 @@ def test_hip_pooling_matches_the_oracle(B, H, W, C, Kh, Kw, Sh, Sw, same):
     assert np.array_equal(arg2.cpu().numpy(), arg) and np.array_equal(y2.cpu().numpy(), y)
 
 
+def test_global_min_pool_on_the_host_is_the_definition():
+    """Host tensors take the definition itself: the minimum over the image, per channel."""
+    from snntc_amd.layers import SNN_globalminpool2d
+    rng = np.random.default_rng(1)
+    x = np.exp(rng.random((3, 5, 4, 6))).astype(np.float32)
+    y, _, _ = cf.min_pool(x, 5, 4, 5, 4, same=False)
+    got = SNN_globalminpool2d()(torch.from_numpy(x))
+    assert tuple(got.shape) == (3, 6) and np.array_equal(got.numpy(), y.reshape(3, 6))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,H,W,C", [(32, 7, 7, 512), (3, 5, 9, 7), (2, 1, 1, 4), (1, 14, 14, 256)])
+def test_hip_global_min_pool_matches_the_oracle(B, H, W, C):
+    """SNN_globalminpool2d = one VALID window the size of the image (the ImageNet-shaped net's head):
+    values and the routed gradient against the pooling oracle, bit for bit; never-fired channels
+    (all pixels at 1e5) and ties included."""
+    import snntc_amd as snn
+    rng = np.random.default_rng(H * 31 + C)
+    x = np.exp(rng.random((B, H, W, C))).astype(np.float32)
+    x[rng.random(x.shape) < 0.1] = np.float32(1e5)
+    x[0, :, :, 0] = np.float32(1e5)                                  # a channel without any spike
+    x[-1, :, :, -1] = np.float32(2.5)                                # every pixel ties: the first one wins
+    y, arg, pad = cf.min_pool(x, H, W, H, W, same=False)
+    xt = torch.from_numpy(x).to("cuda:0").requires_grad_(True)
+    yt = snn.SNN_globalminpool2d()(xt)
+    assert tuple(yt.shape) == (B, C)
+    assert np.array_equal(yt.detach().cpu().numpy(), y.reshape(B, C))
+    assert np.array_equal(yt.detach().cpu().numpy(), x.min(axis=(1, 2)))
+    g = rng.standard_normal((B, C)).astype(np.float32)
+    yt.backward(torch.from_numpy(g).to("cuda:0"))
+    dx = cf.min_pool_grad(g.reshape(B, 1, 1, C), arg, x.shape, H, W, H, W, pad)
+    assert np.array_equal(xt.grad.cpu().numpy(), dx)
+
+
 @pytest.mark.gpu
 def test_pooling_argument_errors():
     import snntc_amd as snn
