@@ -42,13 +42,25 @@ def _dev_f32(t, name, ndim):
 
 
 def _workspace(device, nbytes):
-    """Grow-only scratch buffer per (device, stream); contents never outlive one op call."""
+    """Scratch for one op call.  Eager calls share a grow-only buffer per (device, stream), whose
+    contents never outlive the call.  While the stream is being captured into a HIP graph the buffer
+    is allocated per call instead: its address is baked into the graph, so it has to belong to the
+    graph's own memory pool (which keeps it alive exactly as long as the graph) and must not be a
+    cached tensor that a later, larger request would replace and free."""
+    nbytes = max(int(nbytes), 256)
+    if torch.cuda.is_current_stream_capturing():
+        return torch.empty(nbytes, dtype=torch.uint8, device=device)
     key = (device.index, torch.cuda.current_stream(device).cuda_stream)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
-        buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+        buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
         _workspaces[key] = buf
     return buf
+
+
+def release_workspaces():
+    """Drops the cached eager scratch buffers (they are re-created on demand)."""
+    _workspaces.clear()
 
 
 def _stream(device):

@@ -87,3 +87,37 @@ def test_optional_gradient_outputs():
     none_x, dw2, _ = snn.snnfc_grad(G, X, W, p, y, want_dparams=False, want_dx=False)
     assert none_w is None and none_p is None and none_x is None
     assert torch.equal(dx, dx2) and torch.equal(dw, dw2) and torch.all(dp == 0)
+
+
+def test_workspace_of_a_captured_graph_survives_a_later_larger_capture():
+    """Two graphs that share one memory pool: the second needs a larger scratch buffer than the first.
+    The first graph's scratch must stay its own, so replaying it after the second capture (and after
+    the second graph has run) still gives the eager result."""
+    import snntc_amd as snn
+    xs, ws, ps, _ = dense_case(3, 8, 100, 40, True, "baseline")
+    xl, wl, pl, _ = dense_case(4, 96, 900, 120, True, "baseline")
+    Xs, Ws, Xl, Wl = t(xs), t(ws), t(xl), t(wl)
+    ref_s = snn.snnfc(Xs, Ws, ps).clone()
+    ref_l = snn.snnfc(Xl, Wl, pl).clone()
+    torch.cuda.synchronize()
+
+    pool = torch.cuda.graph_pool_handle()
+    g1 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g1, pool=pool):
+        out_s = snn.snnfc(Xs, Ws, ps)
+    g2 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g2, pool=pool):
+        out_l = snn.snnfc(Xl, Wl, pl)
+        keep = [torch.full((1 << 16,), 7.0, device=DEV) for _ in range(4)]   # more tensors from the shared pool
+    torch.cuda.synchronize()
+    for i in range(3):
+        g2.replay()
+        g1.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_s, ref_s), f"round {i}: the first graph's result changed"
+        g2.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_l, ref_l), f"round {i}: the second graph's result changed"
+        assert all(bool((k == 7.0).all()) for k in keep), "scratch of the first graph overwrote live tensors"
+        snn.snnfc(Xl, Wl, pl)                                                 # eager work between replays
+        torch.cuda.synchronize()
