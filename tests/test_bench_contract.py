@@ -19,9 +19,19 @@ def test_more_than_one_gpu_is_refused():
 def test_workload_table_covers_the_baseline_configs():
     sys.path.insert(0, ROOT)
     import bench
-    assert set(bench.WORKLOADS) == {"mlp", "dense", "conv", "cifar", "imagenet"}
-    # BASELINE config 2 is the default workload
-    assert "784-800-800-10" in bench.MlpTrainStep.name and "B=256" in bench.MlpTrainStep.name
+    # one workload per BASELINE configuration plus the north-star dense layer; the default run times all of
+    # them and puts the largest single-GPU configuration on the top level of the line
+    assert set(bench.WORKLOADS) == {"cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "dense"}
+    assert set(bench.ALL_ORDER) == set(bench.WORKLOADS) and bench.HEADLINE == "cfg5"
+    assert bench.ALIASES == {"mlp": "cfg2", "conv": "cfg3", "cifar": "cfg4", "imagenet": "cfg5", "dense128": "cfg1"}
+
+
+def test_carried_counters_name_their_source():
+    sys.path.insert(0, ROOT)
+    import bench
+    c = bench.carried_counters("cfg3", "scan")
+    assert c["hbm_bytes_per_launch"] > 0 and 0 < c["valu_busy"] <= 1.1 and "commit" in c["source"]
+    assert bench.carried_counters("cfg3", "no_such_kernel") == {}
 
 
 def test_roofline_picks_the_binding_side():
