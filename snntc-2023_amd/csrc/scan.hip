@@ -7,13 +7,20 @@
 // sequential fp32 accumulation with a fused multiply-add for ysum, the division-free firing test
 // |ysum| > x*|wsum| with the product rounded on its own, and y = ysum * (1/wsum).
 //
-// Mapping: one wavefront per (segment, block of 64 neurons); lanes run across neurons, so the
-// weight row w[perm[k], j0..j0+63] is one coalesced 256-byte read, while the sorted value and the
-// row index of step k are the same for every lane and travel through the scalar path, eight steps
-// per fetch (segment rows are padded to a multiple of 16 entries).  The weights of the next eight
-// steps are requested while the current eight are consumed.  A lane that has closed its causal set
-// drops out of the loop (it is masked off and issues no further reads); the wavefront leaves when
-// its last lane has.
+// Kernels, by launch size (launch_scan_lds picks):
+//   scan_filter_kernel     large and mid-sized launches: weight slice in LDS, one or two neurons per
+//                          lane, and the tests of a step skipped wherever a margin test on a whole
+//                          chunk of eight inputs proves that none of them can close the set;
+//   scan_lds_kernel        small launches (a couple of wavefronts per SIMD): weight slice in LDS, every
+//                          step with its tests, written for latency;
+//   scan_lds_split_kernel  fewer work items than CUs: one item per workgroup, its wavefronts sharing
+//                          the item's tests;
+//   scan_kernel            segments so long that not even eight weight columns fit in LDS: weight
+//                          rows streamed from memory, one wavefront per (segment, 64 neurons).
+// In all of them lanes run across neurons, so a weight row is read coalesced (or conflict-free from
+// LDS), while the sorted value and the row index of a step are the same for all lanes of a segment
+// (segment rows are padded to a multiple of 16 entries so that they are fetched eight at a time
+// without bounds checks).
 #include <atomic>
 
 #include "snntc_common.h"
@@ -137,7 +144,7 @@ constexpr int LDS_SCAN_THREADS = 1024;
 constexpr int LDS_SCAN_BYTES = 160 * 1024;
 // The widest slice that fits is taken: the register budget allows one 16-wave workgroup per CU anyway,
 // and fewer slices re-read the sorted rows less often.
-constexpr int LDS_SCAN_TARGET = 160 * 1024;
+constexpr int LDS_SCAN_TARGET = 160 * 1024 - 64;          // 64 bytes behind the slice for a reduction
 
 struct Chunk {
     float x[CHUNK];
@@ -184,80 +191,20 @@ __device__ __forceinline__ void load_chunk(Chunk& c, const RowSource& src, int l
     c.p[4] = (int)pb.x; c.p[5] = (int)pb.y; c.p[6] = (int)pb.z; c.p[7] = (int)pb.w;
 }
 
-// Eight scan steps for the lanes in `run`, written out by hand: the closing test of a step simply
-// removes the lane from EXEC for the rest of the block, so a step is eight vector instructions and
-// three mask operations with no branch.  Per step (x = input time, w = its weight):
-//     close  = fired & (ya <= x*|wsum|)          -> closed |= close ; EXEC &= ~close
-//     wsum  += w ; ysum = fma(x, w, ysum) ; ya = wsum < 0 ? -ysum : ysum
-//     fired  = ya > x*|wsum|                      (bits of lanes outside EXEC read 0)
-// `fired` bits of lanes that do not run in this block are carried across it unchanged.
-#define SNNTC_SCAN_STEP(U)                                                   \
-    "v_mul_f32_e64 %[t], %[x" #U "], |%[wsum]|\n"                            \
-    "v_cmp_le_f32_e32 vcc, %[ya], %[t]\n"                                    \
-    "s_and_b64 vcc, vcc, %[fired]\n"                                         \
-    "s_or_b64 %[closed], %[closed], vcc\n"                                   \
-    "s_andn2_b64 exec, exec, vcc\n"                                          \
-    "v_add_f32_e32 %[wsum], %[wsum], %[w" #U "]\n"                           \
-    "v_fmac_f32_e32 %[ysum], %[x" #U "], %[w" #U "]\n"                       \
-    "v_cmp_gt_f32_e32 vcc, 0, %[wsum]\n"                                     \
-    "v_cndmask_b32_e64 %[ya], %[ysum], -%[ysum], vcc\n"                      \
-    "v_mul_f32_e64 %[t], %[x" #U "], |%[wsum]|\n"                            \
-    "v_cmp_gt_f32_e64 %[fired], %[ya], %[t]\n"
-
 #define SNNTC_SCAN_COUNT "v_add_u32_e32 %[kcnt], 1, %[kcnt]\n"
-
-#define SNNTC_SCAN_PROLOGUE                         \
-    "s_mov_b64 %[save], exec\n"                     \
-    "s_andn2_b64 %[keep], %[fired], %[run]\n"       \
-    "s_mov_b64 exec, %[run]\n"
-#define SNNTC_SCAN_EPILOGUE                         \
-    "s_or_b64 %[fired], %[fired], %[keep]\n"        \
-    "s_mov_b64 exec, %[save]\n"
-#define SNNTC_SCAN_STATE                                                                               \
-    [wsum] "+v"(wsum), [ysum] "+v"(ysum), [ya] "+v"(ya), [kcnt] "+v"(kcnt), [fired] "+s"(fired),       \
-        [closed] "+s"(closed), [save] "=&s"(saved_exec), [keep] "=&s"(keep), [t] "=&v"(t)
 #define SNNTC_SCAN_INPUTS(XC, X)                                                                       \
     [run] "s"(run), [x0] XC(X[0]), [x1] XC(X[1]), [x2] XC(X[2]), [x3] XC(X[3]), [x4] XC(X[4]),          \
         [x5] XC(X[5]), [x6] XC(X[6]), [x7] XC(X[7]), [w0] "v"(w[0]), [w1] "v"(w[1]), [w2] "v"(w[2]),    \
         [w3] "v"(w[3]), [w4] "v"(w[4]), [w5] "v"(w[5]), [w6] "v"(w[6]), [w7] "v"(w[7])
-#define SNNTC_SCAN_BODY_K                                                                              \
-    SNNTC_SCAN_PROLOGUE SNNTC_SCAN_STEP(0) SNNTC_SCAN_COUNT SNNTC_SCAN_STEP(1) SNNTC_SCAN_COUNT         \
-        SNNTC_SCAN_STEP(2) SNNTC_SCAN_COUNT SNNTC_SCAN_STEP(3) SNNTC_SCAN_COUNT SNNTC_SCAN_STEP(4)      \
-            SNNTC_SCAN_COUNT SNNTC_SCAN_STEP(5) SNNTC_SCAN_COUNT SNNTC_SCAN_STEP(6) SNNTC_SCAN_COUNT    \
-                SNNTC_SCAN_STEP(7) SNNTC_SCAN_COUNT SNNTC_SCAN_EPILOGUE
-#define SNNTC_SCAN_BODY                                                                                \
-    SNNTC_SCAN_PROLOGUE SNNTC_SCAN_STEP(0) SNNTC_SCAN_STEP(1) SNNTC_SCAN_STEP(2) SNNTC_SCAN_STEP(3)     \
-        SNNTC_SCAN_STEP(4) SNNTC_SCAN_STEP(5) SNNTC_SCAN_STEP(6) SNNTC_SCAN_STEP(7) SNNTC_SCAN_EPILOGUE
 
-// UNIFORM_X: the eight input times are the same for every lane (one segment per wavefront) and are
-// handed over in scalar registers.
-template <bool WANT_K, bool UNIFORM_X>
-__device__ __forceinline__ void scan_chunk(float& wsum, float& ysum, float& ya, int& kcnt, uint64_t& fired,
-                                           uint64_t& closed, uint64_t run, const float (&x)[CHUNK],
-                                           const float (&w)[CHUNK]) {
-    uint64_t saved_exec, keep;
-    float t;
-    if (UNIFORM_X) {
-        int xs[CHUNK];
-#pragma unroll
-        for (int u = 0; u < CHUNK; ++u) xs[u] = __builtin_amdgcn_readfirstlane(__float_as_int(x[u]));
-        if (WANT_K)
-            asm volatile(SNNTC_SCAN_BODY_K : SNNTC_SCAN_STATE : SNNTC_SCAN_INPUTS("s", xs) : "vcc", "scc");
-        else
-            asm volatile(SNNTC_SCAN_BODY : SNNTC_SCAN_STATE : SNNTC_SCAN_INPUTS("s", xs) : "vcc", "scc");
-    } else {
-        if (WANT_K)
-            asm volatile(SNNTC_SCAN_BODY_K : SNNTC_SCAN_STATE : SNNTC_SCAN_INPUTS("v", x) : "vcc", "scc");
-        else
-            asm volatile(SNNTC_SCAN_BODY : SNNTC_SCAN_STATE : SNNTC_SCAN_INPUTS("v", x) : "vcc", "scc");
-    }
-}
-
-// The same eight steps with every decision kept on the vector side: instead of a fired mask the
-// lane carries a gate value yg = fired ? ya : +inf, the closing test `yg > x*|wsum|` writes EXEC
-// directly and the new gate is a select.  One more vector instruction per step, but no
-// vector -> scalar -> EXEC round trips, so a step of a lone wavefront takes far fewer cycles: used
-// when a launch has too few wavefronts per SIMD to hide that latency.
+// Eight scan steps for the lanes in `run`, written out by hand, every decision on the vector side:
+// the lane carries a gate value yg = fired ? ya : +inf, the closing test `yg > x*|wsum|` writes
+// EXEC directly (a lane that closes drops out of the rest of the block) and the new gate is a
+// select.  Per step (x = input time, w = its weight), nine vector instructions and no branch:
+//     EXEC &= yg > x*|wsum|                       (a closing lane keeps its sums)
+//     wsum  += w ; ysum = fma(x, w, ysum) ; ya = wsum < 0 ? -ysum : ysum
+//     yg     = ya > x*|wsum| ? ya : +inf
+// No vector -> scalar -> EXEC round trips, so a step of a lone wavefront takes few cycles.
 #define SNNTC_VSCAN_STEP(U)                                                  \
     "v_mul_f32_e64 %[t], %[x" #U "], |%[wsum]|\n"                            \
     "v_cmpx_gt_f32_e32 vcc, %[yg], %[t]\n"                                   \
@@ -397,20 +344,21 @@ __device__ __forceinline__ void fill_weight_slice(float* __restrict__ wl, const 
     }
 }
 
-// LOW_LATENCY is the instantiation for launches with at most a couple of wavefronts per SIMD, where
-// nothing hides a stall: workgroups of at most four wavefronts (so that the work spreads over the
-// chip), seven chunks of (x, row) in flight instead of two, and the vector-only step block.
+// Launches with at most a couple of wavefronts per SIMD, where nothing hides a stall: workgroups of
+// at most four wavefronts (so that the work spreads over the chip), one neuron per lane, seven chunks
+// of (x, row) in flight through buffer loads, and the step-by-step block for every chunk (the
+// filtered kernel below pays a fixed price per work item that such small launches do not win back).
 constexpr int LOW_LATENCY_THREADS = 256;
 
-template <int COLS, bool WANT_K, bool LOW_LATENCY>
-__global__ void __launch_bounds__(LOW_LATENCY ? LOW_LATENCY_THREADS : LDS_SCAN_THREADS)
+template <int COLS, bool WANT_K>
+__global__ void __launch_bounds__(LOW_LATENCY_THREADS)
 scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
                 const int32_t* __restrict__ n_real, const float* __restrict__ w, float* __restrict__ y_out,
                 float* __restrict__ rcp_out, int32_t* __restrict__ k_out, int S, int I, int stride, int J,
                 int n_slices, int n_groups, NeuronParams np) {
     extern __shared__ __align__(16) float wl[];                          // [I + bias][COLS]
     constexpr int SEGS = kWave / COLS;                     // segments per wavefront
-    const int WAVES = blockDim.x / kWave;                  // 1..16, chosen by the launcher
+    const int WAVES = blockDim.x / kWave;                  // 1..4, chosen by the launcher
     // slice-major over XCD-contiguous ids: the workgroups of one XCD share a few weight slices
     const int block = xcd_contiguous(blockIdx.x, gridDim.x);
     const int slice = block / n_groups;
@@ -451,50 +399,35 @@ scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ pe
             ya = wsum < 0.0f ? -ysum : ysum;
             fired0 = ya > fabsf(wsum) * np.biasvolt;
         }
-        uint64_t fired = __ballot(fired0);
         uint64_t closed = 0;
         int kcnt = 0;
-        float yg = fired0 ? ya : INFINITY;                  // gate value of the vector-only step
+        float yg = fired0 ? ya : INFINITY;                  // gate value of the step block
 
         // NBUF chunks of (x, row) are held: c is consumed, c+1 feeds the LDS reads, up to c+NBUF-1
         // are being fetched.  The phase loop is unrolled so that buffer indices are compile-time.
-        constexpr int NBUF = LOW_LATENCY ? 8 : 3, AHEAD = NBUF - 1;
-        constexpr int PHASES = (NBUF % 2 == 0) ? NBUF : 2 * NBUF;
+        constexpr int NBUF = 8, AHEAD = NBUF - 1;
         Chunk xp[NBUF];
         float wv[2][CHUNK];
 #pragma unroll
-        for (int b = 0; b < AHEAD; ++b) {
-            const int kb = b * CHUNK <= last_chunk ? b * CHUNK : 0;
-            if (LOW_LATENCY) load_chunk(xp[b], rows_of_item, lane_bytes, kb);
-            else load_chunk_flat(xp[b], xs, pr, kb);
-        }
+        for (int b = 0; b < AHEAD; ++b) load_chunk(xp[b], rows_of_item, lane_bytes, b * CHUNK <= last_chunk ? b * CHUNK : 0);
 #pragma unroll
         for (int u = 0; u < CHUNK; ++u) wv[0][u] = wcol[xp[0].p[u] * COLS];
 
-        // LOW_LATENCY: the body is one straight block per PHASES chunks (no exit between phases: a
-        // phase whose lanes are all done runs with an empty EXEC), which lets the compiler keep
-        // all seven chunks in flight; the regular instantiation leaves as soon as nothing runs.
-        for (int k0 = 0;; k0 += PHASES * CHUNK) {
-            bool stop = false;
+        // The body is one straight block per NBUF chunks (no exit between phases: a phase whose lanes
+        // are all done runs with an empty EXEC), which lets the compiler keep all seven chunks in flight.
+        for (int k0 = 0;; k0 += NBUF * CHUNK) {
 #pragma unroll
-            for (int ph = 0; ph < PHASES; ++ph) {
-                if (LOW_LATENCY) __builtin_amdgcn_sched_barrier(0);   // keep each phase's loads and reads in it
+            for (int ph = 0; ph < NBUF; ++ph) {
+                __builtin_amdgcn_sched_barrier(0);          // keep each phase's loads and reads in it
                 const int k = k0 + ph * CHUNK;
                 const uint64_t run = __ballot(k < n_full) & ~closed;
-                if (!LOW_LATENCY && run == 0) { stop = true; break; }
                 const int kn = k + AHEAD * CHUNK;
-                const int kf = kn <= last_chunk ? kn : 0;
-                if (LOW_LATENCY) load_chunk(xp[(ph + AHEAD) % NBUF], rows_of_item, lane_bytes, kf);
-                else load_chunk_flat(xp[(ph + AHEAD) % NBUF], xs, pr, kf);
+                load_chunk(xp[(ph + AHEAD) % NBUF], rows_of_item, lane_bytes, kn <= last_chunk ? kn : 0);
 #pragma unroll
                 for (int u = 0; u < CHUNK; ++u) wv[(ph + 1) % 2][u] = wcol[xp[(ph + 1) % NBUF].p[u] * COLS];
-                if (LOW_LATENCY)
-                    scan_chunk_vector<WANT_K>(wsum, ysum, ya, yg, kcnt, closed, run, xp[ph % NBUF].x, wv[ph % 2]);
-                else
-                    scan_chunk<WANT_K, COLS == kWave>(wsum, ysum, ya, kcnt, fired, closed, run, xp[ph % NBUF].x,
-                                                      wv[ph % 2]);
+                scan_chunk_vector<WANT_K>(wsum, ysum, ya, yg, kcnt, closed, run, xp[ph % NBUF].x, wv[ph % 2]);
             }
-            if (stop || (__ballot(k0 + PHASES * CHUNK < n_full) & ~closed) == 0) break;
+            if ((__ballot(k0 + NBUF * CHUNK < n_full) & ~closed) == 0) break;
         }
 
         // per-lane epilogue: up to CHUNK-1 trailing inputs, then the output
@@ -502,7 +435,7 @@ scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ pe
             LaneState s;
             s.wsum = wsum; s.ysum = ysum; s.wa = fabsf(wsum); s.ya = ya;
             const bool was_closed = (closed >> lane) & 1;
-            s.fired = was_closed || (LOW_LATENCY ? yg < INFINITY : (bool)((fired >> lane) & 1));
+            s.fired = was_closed || yg < INFINITY;
             bool open = !was_closed;
             for (int k = n_full; k < n && open; ++k) {
                 open = scan_step(s, xs[k], wcol[pr[k] * COLS]);
@@ -749,14 +682,11 @@ scan_lds_split_kernel(const float* __restrict__ sorted, const int32_t* __restric
     }
 }
 
-// CH (2 or 4) neurons per lane.  Same workgroup layout as scan_lds_kernel, but a lane owns CH
-// adjacent columns of its segment: one row address and one 8- or 16-byte LDS read serve CH scans,
-// a wavefront covers 64*CH/COLS segments, and the (x, row) chunks are fetched once for all of
-// them.  Each scan keeps its own fired / closed masks and runs its own eight-step block under its
-// own EXEC.  This is the instantiation for launches with plenty of wavefronts per SIMD.
 template <int CH>
 __device__ __forceinline__ void read_columns(const float* p, float (&out)[CH]) {
-    if (CH == 2) {
+    if constexpr (CH == 1) {
+        out[0] = *p;
+    } else if constexpr (CH == 2) {
         const float2 v = *reinterpret_cast<const float2*>(p);
         out[0] = v.x; out[1] = v.y;
     } else {
@@ -764,20 +694,118 @@ __device__ __forceinline__ void read_columns(const float* p, float (&out)[CH]) {
         out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
     }
 }
+// The same through a pointer that is known to point into LDS.
+typedef float lds_float2 __attribute__((ext_vector_type(2)));
+template <int CH>
+__device__ __forceinline__ void read_columns(__attribute__((address_space(3))) const float* p, float (&out)[CH]) {
+    static_assert(CH == 1 || CH == 2, "one or two columns per lane");
+    if constexpr (CH == 1) {
+        out[0] = *p;
+    } else {
+        const lds_float2 v = *reinterpret_cast<__attribute__((address_space(3))) const lds_float2*>(p);
+        out[0] = v.x; out[1] = v.y;
+    }
+}
 
-constexpr int MULTI_SCAN_THREADS = 512;
+// ---------------------------------------------------------------------------------------------
+// Scan with a margin filter: the tests of a step are skipped wherever they provably cannot close.
+//
+// With D_k = ysum_k - x_k * wsum_k (the state after input k), consuming input k+1 leaves D
+// evaluated at x_{k+1} unchanged, and moving from x_k to x_{k+1} changes it by
+// -(x_{k+1} - x_k) * wsum_k.  D starts positive (theta * x_0 > 0), rises while wsum < 0 (the
+// neuron cannot have fired) and falls while wsum > 0: in exact arithmetic the causal set closes
+// at the first step where D reaches zero.  In fp32 the reference's own tests (products rounded
+// on their own, sign-corrected compares) can disagree with the sign of D only while |D| is
+// within a few ulp of the quantities compared.  So a chunk of eight inputs runs as
+//     wsum += w ; ysum = fma(x, w, ysum) ; t = fma(-x, wsum, ysum)          (3 instructions)
+// and the minimum of the eight t is compared once with
+//     thr = 4u * |ysum_end| + 36u * x_last * max|w|        (u = 2^-24)
+// If the minimum is above thr (and the chunk's first input is not negative) none of the
+// reference's tests before the chunk's eight inputs can close the set:
+//   * wsum_{k-1} > 0: closing before input k needs ysum_{k-1} <= x_k*wsum_{k-1}*(1+u); the sums
+//     after input k differ from those before by the input and two roundings, which puts D_k
+//     below u*(3.01*|ysum_k| + x_k*max|w|) / (1 - 2.01u);
+//   * wsum_{k-1} < 0: closing needs the neuron fired after input k-1, i.e. D_{k-1} < u*x*|wsum|
+//     <= u*(|ysum_{k-1}| + D_{k-1}) -- t of the step before (the last of the previous chunk for
+//     the first step; a neuron that fired on its bias alone never takes the fast path);
+//   * |ysum| anywhere in the chunk is at most 1.01*(|ysum_end| + 7*x_last*max|w|).
+// The running sums are then exactly those of the step-by-step scan, and the fired state is a
+// function of them.  A lane whose chunk fails the test keeps the sums it had before the chunk,
+// records the chunk and sits out; after the loop every lane evaluates its recorded chunk with
+// the reference's tests (the eight-step block above, fed per lane), which finds the close in
+// all but contrived cases, and otherwise walks on step by step.  NaN sums never pass a
+// reference test and never close; a NaN minimum or threshold fails the fast test.
+//
+// CH (1 or 2) adjacent neurons per lane: one row address and one 4- or 8-byte LDS read serve CH
+// scans, and a wavefront covers 64*CH/COLS segments.  Workgroups, slices and items are laid out as
+// in scan_lds_kernel, with up to 16 wavefronts per workgroup.
+// ---------------------------------------------------------------------------------------------
+constexpr float FILTER_REL = 0x1p-22f;                    // 4u
+constexpr float FILTER_W = 9.0f * 0x1p-22f;               // 36u, times max|w| of the slice
+
+// Eight inputs for one scan of every lane.  Lanes that are `open` and pass the test keep the new
+// sums; open lanes that fail keep the old ones, take the chunk's first index as kflag and leave
+// `open`.  Nothing here depends on EXEC or branches: lanes that are not open compute along and
+// discard, so the compiler is free to interleave these instructions with the LDS traffic of the
+// next chunk.
+__device__ __forceinline__ void filter_chunk(float& wsum, float& ysum, int& kflag, bool& open, int k, float thrx,
+                                             const float (&x)[CHUNK], const float (&w)[CHUNK]) {
+    float wb = wsum, yb = ysum, m = INFINITY;
+#pragma unroll
+    for (int u = 0; u < CHUNK; ++u) {
+        wb += w[u];
+        yb = __fmaf_rn(x[u], w[u], yb);
+        m = fminf(m, __fmaf_rn(-x[u], wb, yb));
+    }
+    const bool pass = m > __fmaf_rn(FILTER_REL, fabsf(yb), thrx);     // false for NaN on either side
+    const bool take = open && pass;
+    wsum = take ? wb : wsum;
+    ysum = take ? yb : ysum;
+    kflag = (open && !pass) ? k : kflag;
+    open = take;
+}
+
+// Largest |w| of the slice in LDS (n4 float4 entries), the same value in every thread.  `red` is
+// room for one float per wavefront.  NaN entries are skipped (a NaN sum never closes a set, with
+// or without the filter).
+__device__ __forceinline__ float slice_abs_max(const float* __restrict__ wl, int n4, float* __restrict__ red) {
+    float m = 0.0f;
+    for (int idx = threadIdx.x; idx < n4; idx += blockDim.x) {
+        const float4 v = reinterpret_cast<const float4*>(wl)[idx];
+        m = fmaxf(m, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+    }
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) m = fmaxf(m, __shfl_xor(m, d, kWave));
+    if (threadIdx.x % kWave == 0) red[threadIdx.x / kWave] = m;
+    __syncthreads();
+    const int waves = blockDim.x / kWave;
+    float r = red[0];
+    for (int v = 1; v < waves; ++v) r = fmaxf(r, red[v]);
+    return r;
+}
+
+constexpr int FILTER_RED_BYTES = 64;                       // one float per wavefront behind the slice
+
+// Value of `v` in lane 4*(lane/4) + q: a quad broadcast, which the hardware applies as an operand
+// modifier (DPP) of the move or of the VOP2 instruction that consumes it.
+template <int Q>
+__device__ __forceinline__ int quad_broadcast(int v) {
+    return __builtin_amdgcn_mov_dpp(v, Q * 0x55, 0xf, 0xf, true);
+}
+
+typedef __attribute__((address_space(3))) const float lds_cfloat;
 
 template <int COLS, int CH, bool WANT_K>
-__global__ void __launch_bounds__(CH == 2 ? LDS_SCAN_THREADS : MULTI_SCAN_THREADS)
-scan_lds_multi_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
-                      const int32_t* __restrict__ n_real, const float* __restrict__ w, float* __restrict__ y_out,
-                      float* __restrict__ rcp_out, int32_t* __restrict__ k_out, int S, int I, int stride, int J,
-                      int n_slices, int n_groups, NeuronParams np) {
-    extern __shared__ __align__(16) float wl[];                          // [I + bias][COLS]
+__global__ void __launch_bounds__(LDS_SCAN_THREADS)
+scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
+                   const int32_t* __restrict__ n_real, const float* __restrict__ w, float* __restrict__ y_out,
+                   float* __restrict__ rcp_out, int32_t* __restrict__ k_out, int S, int I, int stride, int J,
+                   int n_slices, int n_groups, NeuronParams np) {
+    extern __shared__ __align__(16) float wl[];                          // [I + bias][COLS], then `red`
     constexpr int LANES = COLS / CH;                       // lanes per segment
     constexpr int SEGS = kWave / LANES;                    // segments per wavefront
+    static_assert(LANES % 4 == 0, "the four lanes of a quad belong to one segment");
     const int WAVES = blockDim.x / kWave;
-    // slice-major over XCD-contiguous ids: the workgroups of one XCD share a few weight slices
     const int block = xcd_contiguous(blockIdx.x, gridDim.x);
     const int slice = block / n_groups;
     const int group = block - slice * n_groups;
@@ -785,6 +813,7 @@ scan_lds_multi_kernel(const float* __restrict__ sorted, const int32_t* __restric
     const int rows = I + np.bias;
     fill_weight_slice<COLS>(wl, w, rows, J, j0);
     __syncthreads();
+    const float thr_w = FILTER_W * slice_abs_max(wl, rows * COLS / 4, wl + rows * COLS);
 
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -793,88 +822,217 @@ scan_lds_multi_kernel(const float* __restrict__ sorted, const int32_t* __restric
     const float* __restrict__ wcol = wl + CH * cg;
     const int last_chunk = stride - CHUNK;
 
+    const int quad_lane = lane & 3;
+    const unsigned wbase = (unsigned)(uintptr_t)(lds_cfloat*)wcol;          // LDS byte address of the lane's columns
+    constexpr int NONE = 0x7fffffff;
+
     for (int item = group * WAVES + wave; item * SEGS < S; item += n_groups * WAVES) {
         const int seg_raw = item * SEGS + sub;
         const int seg = seg_raw < S ? seg_raw : S - 1;      // idle lanes shadow a valid segment
         const float* __restrict__ xs = sorted + (size_t)seg * stride;
         const int32_t* __restrict__ pr = perm + (size_t)seg * stride;
+        const int seg0 = __builtin_amdgcn_readfirstlane(item * SEGS);
+        const int n_segs = S - seg0 < SEGS ? S - seg0 : SEGS;
+        const RowSource rows_of_item = make_row_source(sorted + (size_t)seg0 * stride, perm + (size_t)seg0 * stride,
+                                                       n_segs * stride * (int)sizeof(float));
+        const int lane_bytes = ((seg - seg0) * stride + quad_lane) * (int)sizeof(float);
         const int n_seg = n_real[seg];
         const int n_full = n_seg & ~(CHUNK - 1);
 
-        float wsum[CH], ysum[CH], ya[CH];
-        uint64_t fired[CH], closed[CH];
-        int kcnt[CH];
-        bool live[CH];
+        // Per scan: the running sums, the number of inputs they hold (kcur), and where the scan stands:
+        //   armed    waits to run the fast loop from kcur (no reference test can close before kcur)
+        //   kflag    first index of a chunk that failed the fast test and has to be stepped through (or -1)
+        //   fin      closed; sums, fired state and count are final
+        float wsum[CH], ysum[CH];
+        int kcur[CH], kflag[CH];
+        bool live[CH], armed[CH], fin[CH], fired_cur[CH];   // fired_cur: the fired state that goes with the sums
         float wb[CH];
         if (np.bias) read_columns<CH>(wcol + I * COLS, wb);
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
             live[c] = seg_raw < S && j + c < J;
-            wsum[c] = -np.theta; ysum[c] = 0.0f; ya[c] = 0.0f; kcnt[c] = 0;
-            bool fired0 = false;
+            wsum[c] = -np.theta; ysum[c] = 0.0f;
+            fired_cur[c] = false;
             if (np.bias) {
                 wsum[c] += wb[c];
                 ysum[c] = np.biasvolt * wb[c];
-                ya[c] = wsum[c] < 0.0f ? -ysum[c] : ysum[c];
-                fired0 = ya[c] > fabsf(wsum[c]) * np.biasvolt;
+                const float ya0 = wsum[c] < 0.0f ? -ysum[c] : ysum[c];
+                fired_cur[c] = ya0 > fabsf(wsum[c]) * np.biasvolt;
             }
-            fired[c] = __ballot(fired0);
-            closed[c] = ~__ballot(live[c]);                 // dead lanes never run
+            kcur[c] = 0;
+            fin[c] = false;
+            // The fast loop takes scans whose fired state is what their sums imply between tests that
+            // pass with a margin: fired exactly when the weight sum is positive.  Any other start (a
+            // neuron that fired on its bias alone) is stepped through from the first input on.
+            const bool plain = fired_cur[c] == (wsum[c] > 0.0f) && !fired_cur[c];
+            armed[c] = live[c] && n_full > 0 && plain;
+            kflag[c] = (live[c] && n_full > 0 && !plain) ? 0 : -1;
         }
 
-        Chunk xp[3];
-        float wv[2][CH][CHUNK];                             // [buffer][scan][step]
-        load_chunk_flat(xp[0], xs, pr, 0);
-        load_chunk_flat(xp[1], xs, pr, CHUNK <= last_chunk ? CHUNK : 0);
+        // Passes: the fast loop for the armed scans that are furthest behind, then the recorded
+        // chunks step by step.  A scan that does not close in its recorded chunk is armed again.
+        // Practically every item takes one pass and a second look without work.
+        bool first_pass = true;
+        for (;;) {
+            int kmin = NONE;
 #pragma unroll
-        for (int u = 0; u < CHUNK; ++u) {
-            float wr[CH];
-            read_columns<CH>(wcol + xp[0].p[u] * COLS, wr);
+            for (int c = 0; c < CH; ++c) kmin = armed[c] ? min(kmin, kcur[c]) : kmin;
+            if (first_pass) {                               // every armed scan starts at input 0
+                kmin = __builtin_amdgcn_ballot_w64(kmin != NONE) != 0 ? 0 : NONE;
+            } else {
 #pragma unroll
-            for (int c = 0; c < CH; ++c) wv[0][c][u] = wr[c];
-        }
+                for (int d = kWave / 2; d > 0; d >>= 1) kmin = min(kmin, __shfl_xor(kmin, d, kWave));
+                kmin = __builtin_amdgcn_readfirstlane(kmin);
+            }
+            first_pass = false;
+            if (kmin != NONE) {
+                bool open[CH], ran[CH];
+#pragma unroll
+                for (int c = 0; c < CH; ++c) {
+                    open[c] = ran[c] = armed[c] && kcur[c] == kmin;
+                    armed[c] = armed[c] && !open[c];
+                    kcur[c] = open[c] ? n_full : kcur[c];   // unless the scan records a chunk below
+                }
+                // The (x, row) stream of a segment is the same for all its lanes.  If every lane fetched
+                // the eight entries of a chunk itself, a wavefront would move four kilobytes per chunk
+                // through the vector memory path, which then bounds the kernel.  Instead the four lanes
+                // of a quad fetch entries q and q + 4 of both arrays (q = lane % 4: four dwords per lane
+                // and chunk, through buffer loads that need no address arithmetic), and a value reaches
+                // the other lanes of the quad as a quad broadcast: free for the row offsets, which enter
+                // the LDS address through an add that takes the broadcast as an operand modifier, one
+                // move per input time (shared by the lane's CH scans).
+                // Per phase, with c the chunk being consumed: request the entries of chunk c+RING-1, read
+                // the weights of chunk c+1 from LDS, run chunk c.
+                constexpr int RING = 8;                     // chunks of entries held or on their way
+                float rxl[RING], rxh[RING];
+                int rpl[RING], rph[RING];
+                float wv[2][CH][CHUNK];                     // [buffer][scan][step]
+                auto request = [&](int slot, int k) {
+                    const int kb = (k <= last_chunk ? k : 0) * (int)sizeof(float);
+                    rxl[slot] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rows_of_item.xs, lane_bytes, kb, 0));
+                    rxh[slot] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rows_of_item.xs, lane_bytes + 16, kb, 0));
+                    rpl[slot] = (int)__builtin_amdgcn_raw_buffer_load_b32(rows_of_item.pr, lane_bytes, kb, 0);
+                    rph[slot] = (int)__builtin_amdgcn_raw_buffer_load_b32(rows_of_item.pr, lane_bytes + 16, kb, 0);
+                };
+                auto weights = [&](int slot, float (&wo)[CH][CHUNK]) {
+                    const int al = rpl[slot] * (COLS * 4), ah = rph[slot] * (COLS * 4);
+                    const int a[CHUNK] = {quad_broadcast<0>(al), quad_broadcast<1>(al), quad_broadcast<2>(al),
+                                          quad_broadcast<3>(al), quad_broadcast<0>(ah), quad_broadcast<1>(ah),
+                                          quad_broadcast<2>(ah), quad_broadcast<3>(ah)};
+#pragma unroll
+                    for (int u = 0; u < CHUNK; ++u) {
+                        float wr[CH];
+                        read_columns<CH>(reinterpret_cast<lds_cfloat*>((uintptr_t)(wbase + (unsigned)a[u])), wr);
+#pragma unroll
+                        for (int c = 0; c < CH; ++c) wo[c][u] = wr[c];
+                    }
+                };
+#pragma unroll
+                for (int b = 0; b < RING - 1; ++b) request(b, kmin + b * CHUNK);
+                weights(0, wv[0]);
 
-        for (int k0 = 0;; k0 += 6 * CHUNK) {
-            bool stop = false;
+                for (int k0 = kmin;; k0 += RING * CHUNK) {
+                    bool stop = false;
 #pragma unroll
-            for (int ph = 0; ph < 6; ++ph) {
-                const int k = k0 + ph * CHUNK;
-                const uint64_t in_range = __ballot(k < n_full);
-                uint64_t run[CH], any = 0;
+                    for (int ph = 0; ph < RING; ++ph) {
+                        const int k = k0 + ph * CHUNK;
+                        bool any = false;
 #pragma unroll
-                for (int c = 0; c < CH; ++c) { run[c] = in_range & ~closed[c]; any |= run[c]; }
-                if (any == 0) { stop = true; break; }
-                const int kn = k + 2 * CHUNK;
-                load_chunk_flat(xp[(ph + 2) % 3], xs, pr, kn <= last_chunk ? kn : 0);
+                        for (int c = 0; c < CH; ++c) {
+                            open[c] = open[c] && k < n_full;
+                            any |= open[c];
+                        }
+                        if (__builtin_amdgcn_ballot_w64(any) == 0) { stop = true; break; }
+                        request((ph + RING - 1) % RING, k + (RING - 1) * CHUNK);
+                        weights((ph + 1) % RING, wv[(ph + 1) % 2]);
+                        // The requests above stay ahead of the arithmetic below: what this phase consumes
+                        // was requested a phase or more ago, and what it requests has the whole phase to
+                        // arrive.
+                        __builtin_amdgcn_sched_barrier(0);
+                        const int xl = __float_as_int(rxl[ph % RING]), xh = __float_as_int(rxh[ph % RING]);
+                        const float x[CHUNK] = {
+                            __int_as_float(quad_broadcast<0>(xl)), __int_as_float(quad_broadcast<1>(xl)),
+                            __int_as_float(quad_broadcast<2>(xl)), __int_as_float(quad_broadcast<3>(xl)),
+                            __int_as_float(quad_broadcast<0>(xh)), __int_as_float(quad_broadcast<1>(xh)),
+                            __int_as_float(quad_broadcast<2>(xh)), __int_as_float(quad_broadcast<3>(xh))};
+                        // inputs below zero never take the fast path (the bounds assume x >= 0)
+                        const float thrx = x[0] >= 0.0f ? x[CHUNK - 1] * thr_w : INFINITY;
 #pragma unroll
-                for (int u = 0; u < CHUNK; ++u) {
-                    float wr[CH];
-                    read_columns<CH>(wcol + xp[(ph + 1) % 3].p[u] * COLS, wr);
-#pragma unroll
-                    for (int c = 0; c < CH; ++c) wv[(ph + 1) % 2][c][u] = wr[c];
+                        for (int c = 0; c < CH; ++c)
+                            filter_chunk(wsum[c], ysum[c], kflag[c], open[c], k, thrx, x, wv[ph % 2][c]);
+                    }
+                    if (stop) break;
                 }
 #pragma unroll
-                for (int c = 0; c < CH; ++c)
-                    if (run[c] != 0)
-                        scan_chunk<WANT_K, false>(wsum[c], ysum[c], ya[c], kcnt[c], fired[c], closed[c], run[c],
-                                                  xp[ph % 3].x, wv[ph % 2][c]);
+                for (int c = 0; c < CH; ++c) fired_cur[c] = ran[c] ? wsum[c] > 0.0f : fired_cur[c];
             }
-            if (stop) break;
+
+            // Recorded chunks, stepped through with the reference's tests: every lane fetches its own
+            // eight inputs (positions are multiples of eight inside the full chunks of the row).  A scan
+            // that closes is finished.  One that does not goes back to the fast loop if its fired state is
+            // the plain one; otherwise (fired on a negative weight sum, say) it keeps stepping here, chunk
+            // by chunk, with the entries of its next chunk requested while the current one is worked on.
+            bool need[CH], any_need = false, any_armed = false;
+            Chunk pc[CH];
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                need[c] = kflag[c] >= 0;
+                kcur[c] = need[c] ? kflag[c] : kcur[c];
+                kflag[c] = -1;
+                any_need |= need[c];
+                any_armed |= armed[c];
+            }
+            if (__builtin_amdgcn_ballot_w64(any_need) != 0) {
+#pragma unroll
+                for (int c = 0; c < CH; ++c) load_chunk_flat(pc[c], xs, pr, need[c] ? kcur[c] : 0);
+                do {
+                    any_need = false;
+#pragma unroll
+                    for (int c = 0; c < CH; ++c) {
+                        float pw[CHUNK], px[CHUNK];
+#pragma unroll
+                        for (int u = 0; u < CHUNK; ++u) {
+                            pw[u] = wcol[pc[c].p[u] * COLS + c];
+                            px[u] = pc[c].x[u];
+                        }
+                        const int knext = kcur[c] + CHUNK;
+                        load_chunk_flat(pc[c], xs, pr, (need[c] && knext + CHUNK <= n_full) ? knext : 0);
+                        float ya = wsum[c] < 0.0f ? -ysum[c] : ysum[c];
+                        float yg = fired_cur[c] ? ya : INFINITY;
+                        uint64_t exited = 0;
+                        int kc = kcur[c];
+                        const uint64_t run = __builtin_amdgcn_ballot_w64(need[c]);
+                        if (run != 0) scan_chunk_vector<true>(wsum[c], ysum[c], ya, yg, kc, exited, run, px, pw);
+                        const bool closed_here = (exited >> lane) & 1;
+                        kcur[c] = kc;                       // inputs consumed
+                        fin[c] = fin[c] || closed_here;
+                        fired_cur[c] = closed_here || yg < INFINITY;
+                        const bool more = need[c] && !closed_here && kc + CHUNK <= n_full;
+                        const bool plain = fired_cur[c] == (wsum[c] > 0.0f);
+                        armed[c] = armed[c] || (more && plain);
+                        any_armed |= more && plain;
+                        need[c] = more && !plain;
+                        any_need |= need[c];
+                    }
+                } while (__builtin_amdgcn_ballot_w64(any_need) != 0);
+            }
+            if (__builtin_amdgcn_ballot_w64(any_armed) == 0) break;
         }
 
-        // per-lane epilogue of each scan: up to CHUNK-1 trailing inputs, then the output
+        // Whatever is left of a row -- fewer than eight inputs behind the full chunks, as a rule -- step by
+        // step, then the output.
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
             if (!live[c]) continue;
             LaneState st;
-            st.wsum = wsum[c]; st.ysum = ysum[c]; st.wa = fabsf(wsum[c]); st.ya = ya[c];
-            const bool was_closed = (closed[c] >> lane) & 1;
-            st.fired = was_closed || ((fired[c] >> lane) & 1);
-            bool open = !was_closed;
-            int kc = kcnt[c];
-            for (int k = n_full; k < n_seg && open; ++k) {
-                open = scan_step(st, xs[k], wcol[pr[k] * COLS + c]);
-                if (WANT_K && open) ++kc;
+            st.wsum = wsum[c]; st.ysum = ysum[c]; st.wa = fabsf(wsum[c]);
+            st.ya = wsum[c] < 0.0f ? -ysum[c] : ysum[c];
+            int kc = kcur[c];
+            st.fired = fired_cur[c];
+            bool still = !fin[c];
+            for (int k = kc; k < n_seg && still; ++k) {
+                still = scan_step(st, xs[k], wcol[pr[k] * COLS + c]);
+                if (still) ++kc;
             }
             float y = np.max_time, r = 0.0f;
             if (st.fired) {
@@ -905,15 +1063,19 @@ unpad_rows_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ 
 }  // namespace
 
 namespace {
+// Neurons per lane of the instantiation for large launches (four need 151 registers: too few
+// wavefronts per SIMD, measured slower).
+constexpr int filter_ch(int cols) { return 2; }
+
 template <int COLS>
 int raise_scan_lds_limits() {
     const void* whole[] = {
-        reinterpret_cast<const void*>(scan_lds_kernel<COLS, true, true>),
-        reinterpret_cast<const void*>(scan_lds_kernel<COLS, false, true>),
-        reinterpret_cast<const void*>(scan_lds_kernel<COLS, true, false>),
-        reinterpret_cast<const void*>(scan_lds_kernel<COLS, false, false>),
-        reinterpret_cast<const void*>(scan_lds_multi_kernel<COLS, 2, true>),
-        reinterpret_cast<const void*>(scan_lds_multi_kernel<COLS, 2, false>)};
+        reinterpret_cast<const void*>(scan_lds_kernel<COLS, true>),
+        reinterpret_cast<const void*>(scan_lds_kernel<COLS, false>),
+        reinterpret_cast<const void*>(scan_filter_kernel<COLS, 1, true>),
+        reinterpret_cast<const void*>(scan_filter_kernel<COLS, 1, false>),
+        reinterpret_cast<const void*>(scan_filter_kernel<COLS, filter_ch(COLS), true>),
+        reinterpret_cast<const void*>(scan_filter_kernel<COLS, filter_ch(COLS), false>)};
     for (const void* k : whole)
         SNNTC_HIP_CHECK(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_SCAN_BYTES));
     const void* split[] = {reinterpret_cast<const void*>(scan_lds_split_kernel<COLS, true>),
@@ -959,7 +1121,7 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     const int n_slices = (int)((J + COLS - 1) / COLS);
     const int64_t items = (S + SEGS - 1) / SEGS;
     // workgroups the chip holds at once (two per CU when two weight slices fit in its LDS)
-    const int wgs_per_cu = lds_bytes * 2 <= (size_t)LDS_SCAN_BYTES ? 2 : 1;
+    const int wgs_per_cu = (lds_bytes + FILTER_RED_BYTES) * 2 <= (size_t)LDS_SCAN_BYTES ? 2 : 1;
     const int64_t capacity = (int64_t)cus * wgs_per_cu;
     // A launch whose work items all find a wavefront of their own in workgroups of four (one
     // wavefront per SIMD of a CU, and four times the threads of a single wavefront for copying the
@@ -975,11 +1137,14 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     // With at least four wavefronts of multi-neuron lanes for every SIMD, CH neurons per lane (CH times
     // the segments per wavefront) is the cheaper instruction stream; in between, one neuron per
     // lane in 16-wave workgroups balances better.
-    constexpr int CH = 2;          // four per lane need 151 registers: too few wavefronts per SIMD, measured slower
+    constexpr int CH = filter_ch(COLS);
     const int64_t multi_items = (S + CH * SEGS - 1) / (CH * SEGS);
     const bool multi = !low_latency && multi_items * n_slices >= (int64_t)cus * 4 * 4;
     const int64_t work_items = multi ? multi_items : items;
-    if (multi) WAVES = (CH == 4 ? MULTI_SCAN_THREADS : LDS_SCAN_THREADS) / kWave;
+    if (multi) {
+        const int64_t per_wg = (multi_items * n_slices + capacity - 1) / capacity;
+        WAVES = (int)(per_wg >= 16 ? 16 : (per_wg + 3) / 4 * 4);
+    }
     // Fewer items than CUs: a whole workgroup per item, its wavefronts sharing the item's tests.
     const size_t split_lds = split_lds_bytes(lds_bytes, SEGS, (int)stride);
     const bool split = low_latency && items * n_slices <= (int64_t)cus && I >= 2 * CHUNK * SPLIT_WAVES &&
@@ -990,16 +1155,15 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     const int64_t max_groups = (work_items + WAVES - 1) / WAVES;
     if (n_groups > max_groups) n_groups = max_groups;
     if (n_groups < 1) n_groups = 1;
-    auto kern_k = split ? scan_lds_split_kernel<COLS, true>
-                  : low_latency ? scan_lds_kernel<COLS, true, true>
-                  : multi ? scan_lds_multi_kernel<COLS, CH, true> : scan_lds_kernel<COLS, true, false>;
-    auto kern = split ? scan_lds_split_kernel<COLS, false>
-                : low_latency ? scan_lds_kernel<COLS, false, true>
-                : multi ? scan_lds_multi_kernel<COLS, CH, false> : scan_lds_kernel<COLS, false, false>;
-    dim3 grid((unsigned)(n_slices * n_groups)), block((unsigned)(split ? LOW_LATENCY_THREADS : WAVES * kWave));
+    const bool filt = !(split || low_latency);
+    auto kern_k = filt ? (multi ? scan_filter_kernel<COLS, CH, true> : scan_filter_kernel<COLS, 1, true>)
+                  : split ? scan_lds_split_kernel<COLS, true> : scan_lds_kernel<COLS, true>;
+    auto kern = filt ? (multi ? scan_filter_kernel<COLS, CH, false> : scan_filter_kernel<COLS, 1, false>)
+                : split ? scan_lds_split_kernel<COLS, false> : scan_lds_kernel<COLS, false>;
+    dim3 grid((unsigned)(n_slices * n_groups)), block((unsigned)((split && !filt) ? LOW_LATENCY_THREADS : WAVES * kWave));
     {
         KernelTimerScope timer_("scan", stream);
-        const size_t dyn_lds = split ? split_lds : lds_bytes;
+        const size_t dyn_lds = filt ? lds_bytes + FILTER_RED_BYTES : split ? split_lds : lds_bytes;
         if (causal_k)
             hipLaunchKernelGGL(kern_k, grid, block, dyn_lds, stream, sorted, perm, n_real, w, y, rcp, causal_k,
                                (int)S, (int)I, (int)stride, (int)J, n_slices, (int)n_groups, np);

@@ -62,8 +62,8 @@ DENSE_CASES = [
     (17, 32, 512, 1000, True, "baseline"),     # ImageNet-shaped net, classifier
     # inputs so long that not even 8 weight columns fit in LDS: the scan streams the weight rows
     # (I + bias > 5120), and the last size that still uses the LDS-resident slice
-    (18, 3, 5119, 24, True, "baseline"),       # 5120 rows x 8 columns = exactly 160 KB of LDS
-    (19, 3, 5120, 24, False, "baseline"),      # same slice size without a bias row
+    (18, 3, 5117, 24, True, "baseline"),       # 5118 rows x 8 columns: the largest slice that is kept in LDS
+    (19, 3, 5120, 24, False, "baseline"),      # 160 KB exactly: no room left beside the slice, streaming scan
     (20, 3, 5120, 70, True, "baseline"),       # first size past it: streaming scan, two column blocks
     (21, 2, 8192, 33, True, "reftest"),        # the longest supported segment
     (22, 5, 6000, 7, False, "reftest"),        # streaming scan with a narrow layer (the narrow backward pass)
@@ -98,6 +98,62 @@ def test_dense_forward_backward(seed, B, I, J, bias, dist):
     sdx, sdw, _ = capi.fc_backward_dev(g, x, w, p, ref_out)
     check_grad(sdx, rdx, adx * 8, "oracle fp32 dX")
     check_grad(sdw, rdw, adw * 8, "oracle fp32 dW")
+
+
+def _adversarial_dense(kind, seed, B, I, J):
+    """Inputs that take the scan off its common path: weights of both signs (neurons that fire on a
+    negative weight sum, that never fire, whose weight sum crosses zero many times), exact ties between
+    an output and an input, inputs below zero, all-zero weights, a bias that fires alone."""
+    rng = np.random.default_rng(seed)
+    if kind == "randn":                      # the reference scripts' law
+        x = np.exp(np.abs(rng.standard_normal((B, I))))
+        w = rng.standard_normal((I + 1, J))
+    elif kind == "ties":                     # few distinct times, weights on a coarse grid: y == x happens
+        x = 1.0 + rng.integers(0, 8, (B, I)) / 4.0
+        w = rng.integers(-2, 6, (I + 1, J)) / 16.0
+    elif kind == "negative":                 # times below zero
+        x = rng.standard_normal((B, I)) * 2.0
+        w = 0.3 * rng.standard_normal((I + 1, J)) + 0.1
+    elif kind == "sparse":                   # mostly zero weights, some columns all zero
+        x = np.exp(rng.random((B, I)))
+        w = rng.standard_normal((I + 1, J)) * (rng.random((I + 1, J)) < 0.1)
+        w[:, ::7] = 0.0
+    elif kind == "bias_fires":               # bias weight above the threshold: fired before the first input
+        x = np.exp(1.0 + rng.random((B, I)))
+        w = 4.0 / I + np.sqrt(1.0 / I) * rng.standard_normal((I + 1, J))
+        w[I, ::2] = 1.5 + rng.random(J)[::2]
+    elif kind == "late":                     # small weights: sets close near the end of the row or not at all
+        x = np.exp(rng.random((B, I)))
+        w = (1.05 / I) * (1.0 + 0.2 * rng.standard_normal((I + 1, J)))
+    else:
+        raise ValueError(kind)
+    return x.astype(np.float32), w.astype(np.float32)
+
+
+@pytest.mark.parametrize("kind,seed,B,I,J", [
+    # one neuron per lane, one segment per wavefront (64-column slices), and two segments (32-column slices)
+    ("randn", 0, 4096, 64, 64), ("ties", 1, 4096, 64, 64), ("negative", 2, 4096, 72, 64),
+    ("sparse", 3, 3000, 203, 130), ("bias_fires", 4, 3000, 131, 70), ("late", 5, 2500, 330, 96),
+    ("randn", 6, 1500, 700, 100), ("ties", 7, 2000, 1000, 40),
+    # two neurons per lane (launches with many work items)
+    ("randn", 8, 20000, 40, 64), ("ties", 9, 20000, 48, 33), ("negative", 10, 18000, 27, 64),
+    ("bias_fires", 11, 20000, 35, 20), ("late", 12, 9000, 100, 128), ("sparse", 13, 17000, 19, 8),
+])
+def test_filtered_scan_off_the_common_path(kind, seed, B, I, J):
+    """Launches large enough for the scan that skips provably idle tests, on inputs chosen so that its
+    rare branches run: chunks stepped through without closing, scans that return to the fast loop or
+    stay on the step-by-step path, rows with tails, neurons that fired before the first input."""
+    import snntc_amd as snn
+    x, w = _adversarial_dense(kind, seed, B, I, J)
+    p = capi.fc_params(1.0)
+    ref_out, ref_k, _, _ = capi.fc_forward_dev(x, w, p, want_aux=True)
+    out, _, _, ck = snn.snnfc(t(x), t(w), p, return_aux=True)
+    out2 = snn.snnfc(t(x), t(w), p)
+    torch.cuda.synchronize()
+    out, ck, out2 = out.cpu().numpy(), ck.cpu().numpy(), out2.cpu().numpy()
+    assert np.array_equal(ck, ref_k), f"causal-set sizes differ at {np.argwhere(ck != ref_k)[:5]}"
+    assert np.array_equal(out.view(np.uint32), ref_out.view(np.uint32)), "y / 1/S not bit-exact"
+    assert np.array_equal(out2.view(np.uint32), out.view(np.uint32)), "plain and _ex entry points differ"
 
 
 @pytest.mark.parametrize("B,I,J", [(300, 70, 10), (64, 100, 48)])
