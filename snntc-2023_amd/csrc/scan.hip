@@ -743,12 +743,12 @@ __device__ __forceinline__ void read_columns(__attribute__((address_space(3))) c
 constexpr float FILTER_REL = 0x1p-22f;                    // 4u
 constexpr float FILTER_W = 9.0f * 0x1p-22f;               // 36u, times max|w| of the slice
 
-// Eight inputs for one scan of every lane.  Lanes that are `open` and pass the test keep the new
+// Eight inputs for one scan of every lane.  Lanes in the mask `open` that pass the test keep the new
 // sums; open lanes that fail keep the old ones, take the chunk's first index as kflag and leave
-// `open`.  Nothing here depends on EXEC or branches: lanes that are not open compute along and
-// discard, so the compiler is free to interleave these instructions with the LDS traffic of the
-// next chunk.
-__device__ __forceinline__ void filter_chunk(float& wsum, float& ysum, int& kflag, bool& open, int k, float thrx,
+// `open`.  The arithmetic does not depend on EXEC or branches (lanes that are not open compute along
+// and discard), so the compiler is free to interleave it with the LDS traffic of the next chunk; the
+// decision works on lane masks in scalar registers: one compare, three mask operations, three selects.
+__device__ __forceinline__ void filter_chunk(float& wsum, float& ysum, int& kflag, uint64_t& open, int k, float thrx,
                                              const float (&x)[CHUNK], const float (&w)[CHUNK]) {
     float wb = wsum, yb = ysum, m = INFINITY;
 #pragma unroll
@@ -757,12 +757,17 @@ __device__ __forceinline__ void filter_chunk(float& wsum, float& ysum, int& kfla
         yb = __fmaf_rn(x[u], w[u], yb);
         m = fminf(m, __fmaf_rn(-x[u], wb, yb));
     }
-    const bool pass = m > __fmaf_rn(FILTER_REL, fabsf(yb), thrx);     // false for NaN on either side
-    const bool take = open && pass;
-    wsum = take ? wb : wsum;
-    ysum = take ? yb : ysum;
-    kflag = (open && !pass) ? k : kflag;
-    open = take;
+    const float thr = __fmaf_rn(FILTER_REL, fabsf(yb), thrx);
+    uint64_t stop;
+    asm("v_cmp_gt_f32_e32 vcc, %[m], %[thr]\n"                       // pass: false for NaN on either side
+        "s_andn2_b64 %[stop], %[open], vcc\n"
+        "s_and_b64 %[open], %[open], vcc\n"
+        "v_cndmask_b32_e64 %[ws], %[ws], %[wb], %[open]\n"
+        "v_cndmask_b32_e64 %[ys], %[ys], %[yb], %[open]\n"
+        "v_cndmask_b32_e64 %[kf], %[kf], %[vk], %[stop]\n"
+        : [ws] "+v"(wsum), [ys] "+v"(ysum), [kf] "+v"(kflag), [open] "+s"(open), [stop] "=&s"(stop)
+        : [m] "v"(m), [thr] "v"(thr), [wb] "v"(wb), [yb] "v"(yb), [vk] "v"(k)
+        : "vcc", "scc");
 }
 
 // Largest |w| of the slice in LDS (n4 float4 entries), the same value in every thread.  `red` is
@@ -791,6 +796,23 @@ constexpr int FILTER_RED_BYTES = 64;                       // one float per wave
 template <int Q>
 __device__ __forceinline__ int quad_broadcast(int v) {
     return __builtin_amdgcn_mov_dpp(v, Q * 0x55, 0xf, 0xf, true);
+}
+
+// a[q] = base + (value of `row` in lane q of the quad << SHIFT), q = 0..3: the LDS addresses of four
+// weight rows from the row indices the quad's lanes hold.  One shift, then four adds that take the
+// broadcast as an operand modifier (the two idle cycles between them are what a DPP read of a
+// register written by the instruction before it needs).
+template <int SHIFT>
+__device__ __forceinline__ void quad_row_addresses(int row, unsigned base, unsigned (&a)[4]) {
+    int t;
+    asm("v_lshlrev_b32_e32 %[t], %[sh], %[row]\n"
+        "s_nop 1\n"
+        "v_add_u32_dpp %[a0], %[t], %[base] quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_u32_dpp %[a1], %[t], %[base] quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_u32_dpp %[a2], %[t], %[base] quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_u32_dpp %[a3], %[t], %[base] quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        : [t] "=&v"(t), [a0] "=&v"(a[0]), [a1] "=&v"(a[1]), [a2] "=&v"(a[2]), [a3] "=&v"(a[3])
+        : [row] "v"(row), [base] "v"(base), [sh] "n"(SHIFT));
 }
 
 typedef __attribute__((address_space(3))) const float lds_cfloat;
@@ -825,6 +847,8 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
     const int quad_lane = lane & 3;
     const unsigned wbase = (unsigned)(uintptr_t)(lds_cfloat*)wcol;          // LDS byte address of the lane's columns
     constexpr int NONE = 0x7fffffff;
+    constexpr int ROW_SHIFT = COLS == 64 ? 8 : COLS == 32 ? 7 : COLS == 16 ? 6 : 5;      // a weight row is COLS * 4 bytes
+    static_assert(COLS == 64 || COLS == 32 || COLS == 16 || COLS == 8, "slice width");
 
     for (int item = group * WAVES + wave; item * SEGS < S; item += n_groups * WAVES) {
         const int seg_raw = item * SEGS + sub;
@@ -838,6 +862,7 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
         const int lane_bytes = ((seg - seg0) * stride + quad_lane) * (int)sizeof(float);
         const int n_seg = n_real[seg];
         const int n_full = n_seg & ~(CHUNK - 1);
+        const float first_x = xs[0];
 
         // Per scan: the running sums, the number of inputs they hold (kcur), and where the scan stands:
         //   armed    waits to run the fast loop from kcur (no reference test can close before kcur)
@@ -862,9 +887,11 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
             kcur[c] = 0;
             fin[c] = false;
             // The fast loop takes scans whose fired state is what their sums imply between tests that
-            // pass with a margin: fired exactly when the weight sum is positive.  Any other start (a
-            // neuron that fired on its bias alone) is stepped through from the first input on.
-            const bool plain = fired_cur[c] == (wsum[c] > 0.0f) && !fired_cur[c];
+            // pass with a margin: fired exactly when the weight sum is positive, and whose remaining
+            // inputs are not negative (its bounds assume x >= 0; rows are ascending).  Any other start (a
+            // neuron that fired on its bias alone, a row that begins below zero) is stepped through
+            // from the first input on.
+            const bool plain = fired_cur[c] == (wsum[c] > 0.0f) && !fired_cur[c] && first_x >= 0.0f;
             armed[c] = live[c] && n_full > 0 && plain;
             kflag[c] = (live[c] && n_full > 0 && !plain) ? 0 : -1;
         }
@@ -886,12 +913,14 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
             }
             first_pass = false;
             if (kmin != NONE) {
-                bool open[CH], ran[CH];
+                uint64_t open[CH];                          // lanes whose scan runs in this loop
+                bool ran[CH];
 #pragma unroll
                 for (int c = 0; c < CH; ++c) {
-                    open[c] = ran[c] = armed[c] && kcur[c] == kmin;
-                    armed[c] = armed[c] && !open[c];
-                    kcur[c] = open[c] ? n_full : kcur[c];   // unless the scan records a chunk below
+                    ran[c] = armed[c] && kcur[c] == kmin;
+                    open[c] = __builtin_amdgcn_ballot_w64(ran[c]);
+                    armed[c] = armed[c] && !ran[c];
+                    kcur[c] = ran[c] ? n_full : kcur[c];    // unless the scan records a chunk below
                 }
                 // The (x, row) stream of a segment is the same for all its lanes.  If every lane fetched
                 // the eight entries of a chunk itself, a wavefront would move four kilobytes per chunk
@@ -915,14 +944,13 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
                     rph[slot] = (int)__builtin_amdgcn_raw_buffer_load_b32(rows_of_item.pr, lane_bytes + 16, kb, 0);
                 };
                 auto weights = [&](int slot, float (&wo)[CH][CHUNK]) {
-                    const int al = rpl[slot] * (COLS * 4), ah = rph[slot] * (COLS * 4);
-                    const int a[CHUNK] = {quad_broadcast<0>(al), quad_broadcast<1>(al), quad_broadcast<2>(al),
-                                          quad_broadcast<3>(al), quad_broadcast<0>(ah), quad_broadcast<1>(ah),
-                                          quad_broadcast<2>(ah), quad_broadcast<3>(ah)};
+                    unsigned al[4], ah[4];
+                    quad_row_addresses<ROW_SHIFT>(rpl[slot], wbase, al);
+                    quad_row_addresses<ROW_SHIFT>(rph[slot], wbase, ah);
 #pragma unroll
                     for (int u = 0; u < CHUNK; ++u) {
                         float wr[CH];
-                        read_columns<CH>(reinterpret_cast<lds_cfloat*>((uintptr_t)(wbase + (unsigned)a[u])), wr);
+                        read_columns<CH>(reinterpret_cast<lds_cfloat*>((uintptr_t)(u < 4 ? al[u] : ah[u - 4])), wr);
 #pragma unroll
                         for (int c = 0; c < CH; ++c) wo[c][u] = wr[c];
                     }
@@ -936,13 +964,14 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
 #pragma unroll
                     for (int ph = 0; ph < RING; ++ph) {
                         const int k = k0 + ph * CHUNK;
-                        bool any = false;
+                        const uint64_t inside = __builtin_amdgcn_ballot_w64(k < n_full);
+                        uint64_t any = 0;
 #pragma unroll
                         for (int c = 0; c < CH; ++c) {
-                            open[c] = open[c] && k < n_full;
+                            open[c] &= inside;
                             any |= open[c];
                         }
-                        if (__builtin_amdgcn_ballot_w64(any) == 0) { stop = true; break; }
+                        if (any == 0) { stop = true; break; }
                         request((ph + RING - 1) % RING, k + (RING - 1) * CHUNK);
                         weights((ph + 1) % RING, wv[(ph + 1) % 2]);
                         // The requests above stay ahead of the arithmetic below: what this phase consumes
@@ -955,8 +984,7 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
                             __int_as_float(quad_broadcast<2>(xl)), __int_as_float(quad_broadcast<3>(xl)),
                             __int_as_float(quad_broadcast<0>(xh)), __int_as_float(quad_broadcast<1>(xh)),
                             __int_as_float(quad_broadcast<2>(xh)), __int_as_float(quad_broadcast<3>(xh))};
-                        // inputs below zero never take the fast path (the bounds assume x >= 0)
-                        const float thrx = x[0] >= 0.0f ? x[CHUNK - 1] * thr_w : INFINITY;
+                        const float thrx = x[CHUNK - 1] * thr_w;
 #pragma unroll
                         for (int c = 0; c < CH; ++c)
                             filter_chunk(wsum[c], ysum[c], kflag[c], open[c], k, thrx, x, wv[ph % 2][c]);
@@ -1008,7 +1036,7 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
                         fin[c] = fin[c] || closed_here;
                         fired_cur[c] = closed_here || yg < INFINITY;
                         const bool more = need[c] && !closed_here && kc + CHUNK <= n_full;
-                        const bool plain = fired_cur[c] == (wsum[c] > 0.0f);
+                        const bool plain = fired_cur[c] == (wsum[c] > 0.0f) && px[CHUNK - 1] >= 0.0f;
                         armed[c] = armed[c] || (more && plain);
                         any_armed |= more && plain;
                         need[c] = more && !plain;
