@@ -285,7 +285,7 @@ def account(torch, snn, layers, extras=None):
                             add("crop_time", 0.0, 4.0 * (inp.numel() + x_op.numel()))
                 _, sz, _, ck = snn.snncv(x_op, W, layer.Params, return_aux=True)
                 max_t, bias = float(layer.Params[0]), int(layer.Params[11] > 1e-8)
-                merged = layer.C >= 32 and layer.C % 4 == 0 and layer.Kh * layer.Kw >= 2
+                merged = layer.C >= 32 and layer.C % 4 == 0 and layer.Kw >= 2
         S, I = sz.shape
         J = ck.shape[1]
         n_real = (sz <= np.float32(max_t) - np.float32(0.1)).sum(dim=1, keepdim=True)

@@ -7,10 +7,13 @@
 //   1. column lists: the Kh pixels of one image column under the window merge into a list of
 //      Kh*C elements; rank = own position + (elements of the other pixels that precede it),
 //      each count one binary search.  A column list serves every patch of the tile that covers it.
-//   2. patch: the Kw column lists merge the same way into the P = Kh*Kw*C sorted entries.
+//   2. patch: the Kw column lists are merged one after the other (list 0 with 1, the result with 2,
+//      ...) by a wavefront; every lane takes a run of consecutive outputs, finds where its run starts
+//      in the two inputs with one binary search (merge path) and then merges sequentially.
 // "Precedes" is the stable order of the flat patch index (kh, kw, c): smaller value first, equal
-// values by (kh, kw, c).  Column lists carry 64-bit keys  orderable(value) << 32 | kh << 16 | c,
-// so one unsigned compare against a threshold decides precedence including ties.
+// values by (kh, kw, c).  Column lists carry 64-bit keys  orderable(value) << 32 | kh << 24 | c with
+// an empty field for kw at bit 16, which a patch fills in as it reads a column; all keys of a patch
+// are then distinct and one unsigned compare decides precedence including ties.
 // The result is identical to the bitonic path (and to a stable argsort); it replaces the same
 // reference code (snntc/snncv_kernels.cu.cc:112-166).
 #include <atomic>
@@ -60,63 +63,73 @@ __device__ __forceinline__ void count_before_f32(const float* list, int n, const
     }
 }
 
-// cnt[i] += (entries of key list A that are < thrA[i]) + (entries of key list B that are < thrB[i]);
-// both lists ascending with n entries.  2*EB chains run side by side.
-template <int EB>
-__device__ __forceinline__ void count_below_u64_pair(const u64* listA, const u64* listB, int n,
-                                                     const u64 (&thrA)[EB], const u64 (&thrB)[EB], int (&cnt)[EB]) {
-    int ba[EB], bb[EB];
+// Merges the ascending key lists A[0..nA) and B[0..nB) (all keys distinct once `orB` is or-ed into
+// the keys of B; both lists are followed by an all-ones sentinel) into out[0..nA+nB), with one
+// wavefront, and ends `out` with a sentinel of its own.  A lane produces RUNS runs of E consecutive
+// outputs each (independent chains of LDS reads that overlap): a binary search along the diagonal
+// i + j = first output finds how many of a run's outputs come from A, then one output per step.  `out` must not overlap the inputs (the lanes of a wavefront read and write side by side).
+template <int RUNS>
+__device__ __forceinline__ void wave_merge(const u64* A, int nA, const u64* B, int nB, u64 orB, u64* out, int lane) {
+    const int n = nA + nB;
+    const int E = (n + kWave * RUNS - 1) / (kWave * RUNS);
+    int d0[RUNS], d1[RUNS], lo[RUNS], hi[RUNS];
 #pragma unroll
-    for (int i = 0; i < EB; ++i) { ba[i] = 0; bb[i] = 0; }
-    int len = n;
-    while (len > 1) {
-        const int half = len >> 1;
-        u64 va[EB], vb[EB];
+    for (int r = 0; r < RUNS; ++r) {
+        d0[r] = min((lane * RUNS + r) * E, n);
+        d1[r] = min(d0[r] + E, n);
+        lo[r] = max(0, d0[r] - nB);
+        hi[r] = min(d0[r], nA);
+    }
+    const int iters = 32 - __builtin_clz(min(nA, nB) | 1);            // wave-uniform bound on the search length
+    for (int it = 0; it < iters; ++it) {
+        u64 a[RUNS], b[RUNS];
+        int mid[RUNS];
 #pragma unroll
-        for (int i = 0; i < EB; ++i) { va[i] = listA[ba[i] + half - 1]; vb[i] = listB[bb[i] + half - 1]; }
-#pragma unroll
-        for (int i = 0; i < EB; ++i) {
-            ba[i] += va[i] < thrA[i] ? half : 0;
-            bb[i] += vb[i] < thrB[i] ? half : 0;
+        for (int r = 0; r < RUNS; ++r) {
+            mid[r] = (lo[r] + hi[r]) >> 1;
+            const bool open = lo[r] < hi[r];
+            a[r] = A[open ? mid[r] : 0];
+            b[r] = B[open ? d0[r] - mid[r] - 1 : 0];
         }
-        len -= half;
+#pragma unroll
+        for (int r = 0; r < RUNS; ++r) {
+            const bool open = lo[r] < hi[r];
+            const bool a_first = a[r] < (b[r] | orB);                  // A[i] goes before B[j-1]: i is too small
+            lo[r] = (open && a_first) ? mid[r] + 1 : lo[r];
+            hi[r] = (open && !a_first) ? mid[r] : hi[r];
+        }
     }
+    int i[RUNS], j[RUNS];
 #pragma unroll
-    for (int i = 0; i < EB; ++i)
-        cnt[i] += ba[i] + (listA[ba[i]] < thrA[i] ? 1 : 0) + bb[i] + (listB[bb[i]] < thrB[i] ? 1 : 0);
-}
-
-template <int EB>
-__device__ __forceinline__ void count_below_u64(const u64* list, int n, const u64 (&thr)[EB], int (&cnt)[EB]) {
-    int base[EB];
+    for (int r = 0; r < RUNS; ++r) { i[r] = lo[r]; j[r] = d0[r] - lo[r]; }
+    for (int u = 0; u < E; ++u) {
+        u64 a[RUNS], b[RUNS];
 #pragma unroll
-    for (int i = 0; i < EB; ++i) base[i] = 0;
-    int len = n;
-    while (len > 1) {
-        const int half = len >> 1;
-        u64 v[EB];
+        for (int r = 0; r < RUNS; ++r) { a[r] = A[i[r]]; b[r] = B[j[r]] | orB; }   // sentinels stand in for an exhausted list
 #pragma unroll
-        for (int i = 0; i < EB; ++i) v[i] = list[base[i] + half - 1];
-#pragma unroll
-        for (int i = 0; i < EB; ++i) base[i] += v[i] < thr[i] ? half : 0;
-        len -= half;
+        for (int r = 0; r < RUNS; ++r) {
+            const bool live = d0[r] + u < d1[r];
+            const bool take_a = a[r] < b[r];
+            if (live) out[d0[r] + u] = take_a ? a[r] : b[r];
+            i[r] += (live && take_a) ? 1 : 0;
+            j[r] += (live && !take_a) ? 1 : 0;
+        }
     }
-#pragma unroll
-    for (int i = 0; i < EB; ++i) cnt[i] += base[i] + (list[base[i]] < thr[i] ? 1 : 0);
+    if (lane == 0) out[n] = ~0ull;
 }
 
 constexpr int MERGE_THREADS = 256;
+constexpr int MERGE_RUNS = 1;                             // runs of outputs a lane merges side by side
 constexpr int MERGE_WAVES = MERGE_THREADS / kWave;
 
 // One workgroup = TW consecutive patches of one output row.
 //   pix_z / pix_c : every pixel's channels sorted ascending and their channel ids, rows of Cs entries
 //   sorted / perm : [S, stride] outputs (entries past P padded with +inf / 0), n_real[S]
-template <int EB>   // own-column elements a lane ranks per pass
 __global__ void __launch_bounds__(MERGE_THREADS)
 merge_patches_kernel(const float* __restrict__ pix_z, const int32_t* __restrict__ pix_c, int Cs,
                      float* __restrict__ sorted, int32_t* __restrict__ perm, int32_t* __restrict__ n_real,
                      int H, int W, int C, int Kh, int Kw, int Sh, int Sw, int Nh, int Nw, int TW, int tiles_w,
-                     int stride, float max_cmp) {
+                     int stride, float max_cmp, int c4_shift, unsigned tile_cols_magic) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     const int tile_cols = (TW - 1) * Sw + Kw;
     const int KhC = Kh * C;
@@ -124,8 +137,11 @@ merge_patches_kernel(const float* __restrict__ pix_z, const int32_t* __restrict_
     // LDS carve-up (8-byte pieces first)
     // The pixel lists are dead once the column lists exist; the per-wave output staging reuses
     // their space.
-    u64* col_keys = reinterpret_cast<u64*>(lds_raw);                                   // [tile_cols][KhC]
-    u64* out_keys = col_keys + (size_t)tile_cols * KhC;                                // [MERGE_WAVES][P]
+    // lists end with a sentinel; a wavefront owns a buffer for the finished patch and one for the
+    // list before it (the merges of a patch alternate between the two)
+    const int col_stride = KhC + 1, out_stride = P + 1 + (Kw > 2 ? P - KhC + 1 : 0);
+    u64* col_keys = reinterpret_cast<u64*>(lds_raw);                                   // [tile_cols][KhC + 1]
+    u64* out_keys = col_keys + (size_t)tile_cols * col_stride;                         // [MERGE_WAVES][out_stride]
     float* px_z = reinterpret_cast<float*>(out_keys);                                  // [Kh][tile_cols][C]
     uint16_t* px_c = reinterpret_cast<uint16_t*>(px_z + (size_t)Kh * tile_cols * C);   // [Kh][tile_cols][C]
 
@@ -135,148 +151,125 @@ merge_patches_kernel(const float* __restrict__ pix_z, const int32_t* __restrict_
     const int nw0 = tile * TW;
     const int w_first = nw0 * Sw;
 
+    // Both passes below walk the pixel lists in groups of four channels: group g is channels
+    // 4*(g % C4) .. +3 of pixel row g / C4 (row = kh * tile_cols + col).  The divisions by runtime
+    // values are a shift (C4 a power of two, the usual case) and a multiply-high.
+    const int C4 = C / 4;
+    const int n_groups = Kh * tile_cols * C4;
+    auto split = [&](int g, int& row, int& c, int& kh, int& col) {
+        row = c4_shift >= 0 ? g >> c4_shift : g / C4;
+        c = (g - row * C4) * 4;
+        kh = (int)__umulhi((unsigned)row, tile_cols_magic);
+        col = row - kh * tile_cols;
+    };
+
     // ---- stage the sorted pixels under the tile ------------------------------------------------
-    const int n_px = Kh * tile_cols * C;
-    // loads are issued in batches: one at a time would cost a memory latency per element
-    constexpr int STAGE = 8;
-    for (int base = threadIdx.x; base < n_px; base += STAGE * MERGE_THREADS) {
-        float zv[STAGE];
-        int cv[STAGE];
+    // loads are issued in batches: one at a time would cost a memory latency per group
+    constexpr int STAGE = 4;
+    for (int base = threadIdx.x; base < n_groups; base += STAGE * MERGE_THREADS) {
+        float4 zv[STAGE];
+        int4 cv[STAGE];
 #pragma unroll
         for (int u = 0; u < STAGE; ++u) {
-            const int idx = base + u * MERGE_THREADS;
-            const int c = idx % C;
-            const int pc = idx / C;
-            const int col = pc % tile_cols, kh = pc / tile_cols;
+            const int g = base + u * MERGE_THREADS;
+            int row, c, kh, col;
+            split(g, row, c, kh, col);
             const int wp = w_first + col;
-            zv[u] = INFINITY;
-            cv[u] = c;
-            if (idx < n_px && wp < W) {
-                const size_t g = ((size_t)(a * H + nh * Sh + kh) * W + wp) * Cs + c;
-                zv[u] = pix_z[g];
-                cv[u] = pix_c[g];
+            zv[u] = make_float4(INFINITY, INFINITY, INFINITY, INFINITY);
+            cv[u] = make_int4(c, c + 1, c + 2, c + 3);
+            if (g < n_groups && wp < W) {
+                const size_t src = ((size_t)(a * H + nh * Sh + kh) * W + wp) * Cs + c;
+                zv[u] = *reinterpret_cast<const float4*>(pix_z + src);
+                cv[u] = *reinterpret_cast<const int4*>(pix_c + src);
             }
         }
 #pragma unroll
         for (int u = 0; u < STAGE; ++u) {
-            const int idx = base + u * MERGE_THREADS;
-            if (idx < n_px) { px_z[idx] = zv[u]; px_c[idx] = (uint16_t)cv[u]; }
+            const int g = base + u * MERGE_THREADS;
+            if (g < n_groups) {
+                reinterpret_cast<float4*>(px_z)[g] = zv[u];
+                reinterpret_cast<uint2*>(px_c)[g] = make_uint2((uint32_t)cv[u].x | ((uint32_t)cv[u].y << 16),
+                                                               (uint32_t)cv[u].z | ((uint32_t)cv[u].w << 16));
+            }
         }
     }
     __syncthreads();
 
     // ---- column lists: merge the Kh pixels of every column -----------------------------------------
-    // A thread takes NB elements of the same (kh, col) pixel list at a time (idx, idx+1, ...).
-    for (int idx0 = threadIdx.x * NB; idx0 < n_px; idx0 += MERGE_THREADS * NB) {
-        // C is a multiple of NB, so the NB elements share their pixel
-        const int l0 = idx0 % C;
-        const int pc = idx0 / C;
-        const int col = pc % tile_cols, kh = pc / tile_cols;
-        float z[NB];
+    // A thread ranks the NB = 4 elements of a group side by side.
+    for (int g = threadIdx.x; g < n_groups; g += MERGE_THREADS) {
+        int row, l0, kh, col;
+        split(g, row, l0, kh, col);
+        const float4 zq = reinterpret_cast<const float4*>(px_z)[g];
+        const uint2 cq = reinterpret_cast<const uint2*>(px_c)[g];
+        const float z[NB] = {zq.x, zq.y, zq.z, zq.w};
+        const uint32_t ch[NB] = {cq.x & 0xffffu, cq.x >> 16, cq.y & 0xffffu, cq.y >> 16};
         int rank[NB];
 #pragma unroll
-        for (int i = 0; i < NB; ++i) { z[i] = px_z[idx0 + i]; rank[i] = l0 + i; }
+        for (int i = 0; i < NB; ++i) rank[i] = l0 + i;
         for (int k2 = 0; k2 < kh; ++k2)          // pixels above: equal values come first there
             count_before_f32<false>(px_z + (size_t)(k2 * tile_cols + col) * C, C, z, rank);
         for (int k2 = kh + 1; k2 < Kh; ++k2)     // pixels below: only strictly smaller values precede
             count_before_f32<true>(px_z + (size_t)(k2 * tile_cols + col) * C, C, z, rank);
 #pragma unroll
         for (int i = 0; i < NB; ++i)
-            col_keys[(size_t)col * KhC + rank[i]] =
-                ((u64)order_key(z[i]) << 32) | ((u64)kh << 16) | px_c[idx0 + i];
+            col_keys[(size_t)col * col_stride + rank[i]] = ((u64)order_key(z[i]) << 32) | ((u64)kh << 24) | ch[i];
     }
+    __syncthreads();                                          // the pixel lists are dead from here on
+    for (int col = threadIdx.x; col < tile_cols; col += MERGE_THREADS) col_keys[(size_t)col * col_stride + KhC] = ~0ull;
     __syncthreads();
 
     // ---- patches: merge the Kw columns of every patch ----------------------------------------------
+    // From here on a wavefront works alone: the column lists are read-only and its two buffers are
+    // its own, so no workgroup barrier is needed between its merges and its output.
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
-    u64* my_out = out_keys + (size_t)wave * P;
-    const int rounds = (TW + MERGE_WAVES - 1) / MERGE_WAVES;
-    for (int rd = 0; rd < rounds; ++rd) {
-        const int j = rd * MERGE_WAVES + wave;
-        const bool valid = j < TW && nw0 + j < Nw;
-        if (valid) {
-            for (int kw = 0; kw < Kw; ++kw) {
-                const u64* mine = col_keys + (size_t)(j * Sw + kw) * KhC;
-                // EB elements of the own column per pass (lane, lane+64, ...); a tail element repeats
-                // the last one and is not written.  The other columns are taken two at a time.
-                for (int e0 = lane; e0 < KhC; e0 += kWave * EB) {
-                    u64 key[EB], thr_incl[EB], thr_strict[EB];
-                    int rank[EB];
-#pragma unroll
-                    for (int i = 0; i < EB; ++i) {
-                        const int e = min(e0 + i * kWave, KhC - 1);
-                        key[i] = mine[e];
-                        const u64 hi = key[i] & 0xffffffff00000000ull;
-                        const u64 kh = (key[i] >> 16) & 0xffffull;
-                        // entries of a column to the left precede on (value, kh) <= mine, to the right on <
-                        thr_incl[i] = hi | ((kh + 1) << 16);
-                        thr_strict[i] = hi | (kh << 16);
-                        rank[i] = e;
-                    }
-                    const u64* cols = col_keys + (size_t)(j * Sw) * KhC;
-                    int k2 = 0;
-                    for (; k2 + 1 < kw; k2 += 2)             // two columns to the left
-                        count_below_u64_pair<EB>(cols + (size_t)k2 * KhC, cols + (size_t)(k2 + 1) * KhC, KhC,
-                                                 thr_incl, thr_incl, rank);
-                    int k3 = kw + 1;
-                    if (k2 < kw && k3 < Kw) {                // one left, one right
-                        count_below_u64_pair<EB>(cols + (size_t)k2 * KhC, cols + (size_t)k3 * KhC, KhC, thr_incl,
-                                                 thr_strict, rank);
-                        ++k2; ++k3;
-                    }
-                    if (k2 < kw) count_below_u64<EB>(cols + (size_t)k2 * KhC, KhC, thr_incl, rank);
-                    for (; k3 + 1 < Kw; k3 += 2)             // two columns to the right
-                        count_below_u64_pair<EB>(cols + (size_t)k3 * KhC, cols + (size_t)(k3 + 1) * KhC, KhC,
-                                                 thr_strict, thr_strict, rank);
-                    if (k3 < Kw) count_below_u64<EB>(cols + (size_t)k3 * KhC, KhC, thr_strict, rank);
-#pragma unroll
-                    for (int i = 0; i < EB; ++i) {
-                        if (e0 + i * kWave < KhC) {
-                            const uint32_t kh = (uint32_t)(key[i] >> 16) & 0xffffu, c = (uint32_t)key[i] & 0xffffu;
-                            my_out[rank[i]] = (key[i] & 0xffffffff00000000ull) | (u64)((kh * Kw + kw) * C + c);
-                        }
-                    }
-                }
-            }
+    u64* my_out = out_keys + (size_t)wave * out_stride;
+    for (int j = wave; j < TW && nw0 + j < Nw; j += MERGE_WAVES) {
+        // column 0 with 1, the result with 2, ...: the merge that takes in column kw writes the
+        // patch buffer when Kw - 1 - kw is even and the other buffer otherwise, so that the last
+        // one lands in the patch buffer
+        const u64* cols = col_keys + (size_t)(j * Sw) * col_stride;
+        u64* other = my_out + P + 1;
+        const u64* acc = cols;
+        for (int kw = 1; kw < Kw; ++kw) {
+            u64* dst = ((Kw - 1 - kw) & 1) ? other : my_out;
+            wave_merge<MERGE_RUNS>(acc, kw * KhC, cols + (size_t)kw * col_stride, KhC, (u64)kw << 16, dst, lane);
+            acc = dst;
         }
-        __syncthreads();
-        if (valid) {
-            const size_t s = (size_t)(a * Nh + nh) * Nw + nw0 + j;
-            float* so = sorted + s * stride;
-            int32_t* po = perm + s * stride;
-            int below = 0;
-            for (int e = lane; e < stride; e += kWave) {
-                float z = INFINITY;
-                int32_t id = 0;
-                if (e < P) {
-                    const u64 key = my_out[e];
-                    z = order_key_to_float((uint32_t)(key >> 32));
-                    id = (int32_t)(uint32_t)key;
-                    below += z <= max_cmp ? 1 : 0;
-                }
-                so[e] = z;
-                po[e] = id;
+        const size_t s = (size_t)(a * Nh + nh) * Nw + nw0 + j;
+        float* so = sorted + s * stride;
+        int32_t* po = perm + s * stride;
+        int below = 0;                                        // wave-uniform count of entries <= max_cmp
+        for (int e = lane; e < stride; e += kWave) {
+            float z = INFINITY;
+            int32_t id = 0;
+            if (e < P) {
+                const u64 key = my_out[e];
+                z = order_key_to_float((uint32_t)(key >> 32));
+                const uint32_t low = (uint32_t)key;                    // kh | kw | c
+                id = (int32_t)(((low >> 24) * Kw + ((low >> 16) & 0xffu)) * C + (low & 0xffffu));
             }
-#pragma unroll
-            for (int d = 1; d < kWave; d <<= 1) below += __shfl_xor(below, d, kWave);
-            if (lane == 0) n_real[s] = below;
+            below += __builtin_popcountll(__builtin_amdgcn_ballot_w64(e < P && z <= max_cmp));
+            so[e] = z;
+            po[e] = id;
         }
-        __syncthreads();
+        if (lane == 0) n_real[s] = below;
     }
 }
 
 size_t merge_lds_bytes(int C, int Kh, int Kw, int Sw, int TW) {
     const size_t tile_cols = (size_t)(TW - 1) * Sw + Kw;
     const size_t KhC = (size_t)Kh * C, P = KhC * Kw;
-    const size_t staging = (size_t)MERGE_WAVES * P * 8, pixels = (size_t)Kh * tile_cols * C * (4 + 2);
-    return tile_cols * KhC * 8 + (staging > pixels ? staging : pixels);
+    const size_t staging = (size_t)MERGE_WAVES * (P + 1 + (Kw > 2 ? P - KhC + 1 : 0)) * 8;
+    const size_t pixels = (size_t)Kh * tile_cols * C * (4 + 2);
+    return tile_cols * (KhC + 1) * 8 + (staging > pixels ? staging : pixels);
 }
 
 // Patches per tile: as many as fit in 52 KB of LDS (so three workgroups share a CU), at
 // most 16, never more than the row holds.  Layers with so many channels that not even two
 // patches fit in 52 KB take what fits in MERGE_LDS_CAP (one workgroup per CU).
-constexpr size_t MERGE_LDS_CAP = 128 * 1024;
+constexpr size_t MERGE_LDS_CAP = 160 * 1024;
 int merge_tile_width(const ConvGeom& g) {
     const int tw_max = g.Nw < 16 ? (int)g.Nw : 16;
     int tw = tw_max;
@@ -293,7 +286,7 @@ int merge_tile_width(const ConvGeom& g) {
 // The merge path needs channel ids and kh in 16 bits, a useful amount of sharing and an LDS
 // footprint within reach; everything else goes through the bitonic network.
 bool merge_sort_supported(const ConvGeom& g) {
-    if (g.C < 32 || g.C % NB != 0 || g.C > 4096 || g.Kh * g.Kw < 2 || g.Kh > 255) return false;
+    if (g.C < 32 || g.C % NB != 0 || g.C > 4096 || g.Kw < 2 || g.Kh > 255 || g.Kw > 255) return false;
     const int tw = merge_tile_width(g);
     return merge_lds_bytes((int)g.C, (int)g.Kh, (int)g.Kw, (int)g.Sw, tw) <= MERGE_LDS_CAP && tw >= 2;
 }
@@ -304,12 +297,8 @@ int merge_prepare_device(int dev) {
     static std::atomic<bool> done[kMaxDevices];
     if (dev < 0 || dev >= kMaxDevices) return fail(SNNTC_ERR_UNSUPPORTED, "patch merge: device index %d not supported", dev);
     if (done[dev].load(std::memory_order_acquire)) return SNNTC_OK;
-    const void* kernels[] = {reinterpret_cast<const void*>(merge_patches_kernel<1>),
-                             reinterpret_cast<const void*>(merge_patches_kernel<2>),
-                             reinterpret_cast<const void*>(merge_patches_kernel<3>),
-                             reinterpret_cast<const void*>(merge_patches_kernel<4>)};
-    for (const void* k : kernels)
-        SNNTC_HIP_CHECK(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)MERGE_LDS_CAP));
+    SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(merge_patches_kernel),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)MERGE_LDS_CAP));
     done[dev].store(true, std::memory_order_release);
     return SNNTC_OK;
 }
@@ -322,20 +311,21 @@ int launch_merge_patches(const float* pix_z, const int32_t* pix_c, int64_t Cs, f
     const int tiles_w = (int)((g.Nw + tw - 1) / tw);
     const int64_t blocks = g.B * g.Nh * tiles_w;
     if (blocks > 0x7fffffffLL) return fail(SNNTC_ERR_TOO_LARGE, "patch merge: grid too large");
-    // elements of one column per lane: Kh*C / 64, at most four ranked side by side
-    const int64_t per_lane = (g.Kh * g.C + kWave - 1) / kWave;
-    const int eb = per_lane >= 4 ? 4 : (int)per_lane;
-    auto kern = eb == 1 ? merge_patches_kernel<1> : eb == 2 ? merge_patches_kernel<2>
-              : eb == 3 ? merge_patches_kernel<3> : merge_patches_kernel<4>;
+    // C / 4 as a shift where it is a power of two; row / tile_cols as a multiply-high (exact for rows < 2^16)
+    const int c4 = (int)g.C / 4;
+    int c4_shift = -1;
+    if ((c4 & (c4 - 1)) == 0) { c4_shift = 0; while ((1 << c4_shift) < c4) ++c4_shift; }
+    const unsigned tile_cols = (unsigned)((tw - 1) * g.Sw + g.Kw);
+    const unsigned magic = (unsigned)((0x100000000ull + tile_cols - 1) / tile_cols);
     int dev = 0;
     SNNTC_HIP_CHECK(hipGetDevice(&dev));
     const int prep = merge_prepare_device(dev);
     if (prep) return prep;
     {
         KernelTimerScope timer_("merge_patches", stream);
-        hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(MERGE_THREADS), lds, stream, pix_z, pix_c, (int)Cs,
+        hipLaunchKernelGGL(merge_patches_kernel, dim3((unsigned)blocks), dim3(MERGE_THREADS), lds, stream, pix_z, pix_c, (int)Cs,
                            sorted, perm, n_real, (int)g.H, (int)g.W, (int)g.C, (int)g.Kh, (int)g.Kw, (int)g.Sh,
-                           (int)g.Sw, (int)g.Nh, (int)g.Nw, tw, tiles_w, (int)stride, max_cmp);
+                           (int)g.Sw, (int)g.Nh, (int)g.Nw, tw, tiles_w, (int)stride, max_cmp, c4_shift, magic);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
