@@ -67,7 +67,8 @@ class Workload:
 
     def layers(self):
         """[(layer module, its input tensor, whether the step asks for the input gradient, whether the
-        tensor is already the padded one the conv op takes)], in forward order, for the accounting."""
+        tensor is already the padded one the conv op takes -- or "fed" when the layer before has written
+        the padded tensor)], in forward order, for the accounting."""
         raise NotImplementedError
 
     extras = {}          # algorithmic bytes of the step's glue kernels (loss, SGD), by kernel name
@@ -132,7 +133,7 @@ class NetworkStep(Workload):
         self.z = torch.from_numpy(np.exp(1.0 - x)).to(dev)
         labels = rng.integers(0, classes, batch)
         self.onehot = torch.from_numpy(np.eye(classes, dtype=np.float32)[labels]).to(dev)
-        self.net = networks.build(spec, rng=rng).to(dev)
+        self.net = networks.build(spec, rng=rng, chain=True).to(dev)     # no padding pass between chained layers
         self.params = self.net.weights()
         self._networks = networks
         n_w = float(sum(p.numel() for p in self.params))
@@ -150,7 +151,13 @@ class NetworkStep(Workload):
         acts = []
         with self.torch.no_grad():
             self.net(self.z, keep=acts)
-        return [(l, a, i > 0, False) for i, (l, a) in enumerate(zip(self.net, acts))]
+        out, mods = [], list(self.net)
+        for i, (l, a) in enumerate(zip(mods, acts)):
+            # a conv layer fed by the conv / pooling layer before it finds its input in its padded buffer
+            fed = (i > 0 and isinstance(l, self.snn.SNN_conv) and l.padding == 'SAME'
+                   and isinstance(mods[i - 1], (self.snn.SNN_conv, self.snn.SNN_maxpool2d)))
+            out.append((l, a, i > 0, "fed" if fed else False))
+        return out
 
 
 def _make(key):
@@ -250,7 +257,7 @@ def account(torch, snn, layers, extras=None):
       grad_weight   : bytes 4*(2*S*J + in + (I+b)*J)               flops 3*pairs
       prep_upstream : bytes 4*(3*S*J + 2*S*J + 2*I*J)              flops S*J   (carries the weight copy dX reads)
       fc_backward_narrow (J <= 16, the three above in one launch): bytes 4*(3*S*J + 2*in + 2*(I+b)*J), flops 5*pairs + S*J
-      pad_time / crop_time : bytes 4*(in + out) ;  min_pool / min_pool_grad : bytes 4*(in + 2*out)
+      pad_time : bytes 4*(in + out) ;  min_pool / min_pool_grad : bytes 4*(in + 2*out)
     `in` is the op's input tensor (B*I dense, B*H*W*C padded image for conv)."""
     acc = {}
 
@@ -277,12 +284,10 @@ def account(torch, snn, layers, extras=None):
                 merged = False
             else:
                 x_op = inp
-                if not padded:                       # a network layer: the layer pads (SAME) or crops (VALID) first
-                    x_op = layer.prepare_input(inp).contiguous()
-                    if x_op.numel() > inp.numel():
+                if padded is not True:               # a network layer: the layer pads (SAME) or crops (VALID) first;
+                    x_op = layer.prepare_input(inp).contiguous()        # "fed": the layer before wrote the padded tensor
+                    if x_op.numel() > inp.numel() and padded != "fed":
                         add("pad_time", 0.0, 4.0 * (inp.numel() + x_op.numel()))
-                        if want_dx:
-                            add("crop_time", 0.0, 4.0 * (inp.numel() + x_op.numel()))
                 _, sz, _, ck = snn.snncv(x_op, W, layer.Params, return_aux=True)
                 max_t, bias = float(layer.Params[0]), int(layer.Params[11] > 1e-8)
                 merged = layer.C >= 32 and layer.C % 4 == 0 and layer.Kw >= 2

@@ -168,6 +168,18 @@ SNNTC_API int snntc_cv_forward_ex(const float* xpad, const float* w, const float
                         int64_t B, int64_t H, int64_t W, int64_t C, int64_t Kc, int64_t w_rows,
                         void* workspace, size_t workspace_bytes, void* stream);
 
+/* snntc_cv_forward that also leaves the spike times where the next layer reads them: next_xpad is the
+ * next SNN_conv's padded input, [B, next_h, next_w, Kc], and the time of output pixel (nh, nw) is
+ * written to its pixel (nh + next_top, nw + next_left) as well as to `out`.  The border of next_xpad
+ * (the layer's MAX_SPIKE_TIME padding, SNN_TC_Modules.py:147-161) is the caller's: it is constant, so it
+ * is filled once when the buffer is made, not per call.  This replaces the tf.pad between two conv
+ * layers of the reference's models (snntc/snntc-cifar10.py:73-106 stacks SNN_conv layers directly).
+ * Errors: as snntc_cv_forward; an output that does not fit the destination at that offset -> BAD_ARGUMENT. */
+SNNTC_API int snntc_cv_forward_chained(const float* xpad, const float* w, const float* params_host, float* out,
+                             float* next_xpad, int64_t next_h, int64_t next_w, int64_t next_top, int64_t next_left,
+                             int64_t B, int64_t H, int64_t W, int64_t C, int64_t Kc, int64_t w_rows,
+                             void* workspace, size_t workspace_bytes, void* stream);
+
 /* grad[grad_rows,Nh,Nw,Kc] (rows [0,B) read), oldout[2B,Nh,Nw,Kc].
  * dxpad[B,H,W,C] (gradient w.r.t. the padded input), dw[w_rows,Kc], dparams[12]; any may be NULL
  * (not computed).
@@ -176,6 +188,17 @@ SNNTC_API int snntc_cv_backward(const float* grad, const float* xpad, const floa
                       const float* oldout, float* dxpad, float* dw, float* dparams,
                       int64_t B, int64_t H, int64_t W, int64_t C, int64_t Kc, int64_t w_rows,
                       int64_t grad_rows, void* workspace, size_t workspace_bytes, void* stream);
+
+/* snntc_cv_backward that stores only a window of the padded input's gradient:
+ *   dx[B, dx_h, dx_w, C] = dxpad[:, dx_top : dx_top + dx_h, dx_left : dx_left + dx_w, :].
+ * With the window of the un-padded image this is the gradient the layer before expects, i.e. the
+ * backward of the tf.pad in SNN_conv.__call__ (SNN_TC_Modules.py:147-161) folded into the op.
+ * Errors: as snntc_cv_backward; a window that does not lie inside the padded image -> BAD_ARGUMENT. */
+SNNTC_API int snntc_cv_backward_cropped(const float* grad, const float* xpad, const float* w, const float* params_host,
+                              const float* oldout, float* dx, int64_t dx_h, int64_t dx_w, int64_t dx_top,
+                              int64_t dx_left, float* dw, float* dparams, int64_t B, int64_t H, int64_t W, int64_t C,
+                              int64_t Kc, int64_t w_rows, int64_t grad_rows, void* workspace, size_t workspace_bytes,
+                              void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Loss of the example networks, loss_func (SNN_TC_Modules.py:286-288): categorical cross-entropy of
@@ -205,6 +228,13 @@ SNNTC_API int snntc_softmax_time_loss(const float* times, const float* label, fl
 SNNTC_API int snntc_min_pool_forward(const float* x, float* y, int32_t* arg, int64_t B, int64_t H, int64_t W,
                            int64_t C, int64_t Kh, int64_t Kw, int64_t Sh, int64_t Sw, int64_t pad_top,
                            int64_t pad_left, int64_t Nh, int64_t Nw, float pad_value, void* stream);
+/* snntc_min_pool_forward that also leaves the pooled times inside the padded input of the SNN_conv that
+ * follows (next_xpad[B, next_h, next_w, C], pixel offset (next_top, next_left), border filled by the
+ * caller): see snntc_cv_forward_chained. */
+SNNTC_API int snntc_min_pool_forward_chained(const float* x, float* y, int32_t* arg, float* next_xpad, int64_t next_h,
+                                   int64_t next_w, int64_t next_top, int64_t next_left, int64_t B, int64_t H, int64_t W,
+                                   int64_t C, int64_t Kh, int64_t Kw, int64_t Sh, int64_t Sw, int64_t pad_top,
+                                   int64_t pad_left, int64_t Nh, int64_t Nw, float pad_value, void* stream);
 SNNTC_API int snntc_min_pool_backward(const float* grad_y, const int32_t* arg, float* dx, int64_t B, int64_t H,
                             int64_t W, int64_t C, int64_t Kh, int64_t Kw, int64_t Sh, int64_t Sw,
                             int64_t pad_top, int64_t pad_left, int64_t Nh, int64_t Nw, void* stream);

@@ -152,12 +152,12 @@ FcFwdWs fc_fwd_ws(void* ws, int64_t S, int64_t I, int64_t n_pix = 0, int64_t pix
 // sort -> (optional copy of the side outputs) -> scan, shared by the dense and the conv op
 int forward_chain(const SegmentSource& src, const FcFwdWs& ws, const float* w, float* out, float* sorted_z,
                   int32_t* perm, int32_t* causal_k, int64_t S, int64_t I, int64_t J, const NeuronParams& np,
-                  hipStream_t st) {
+                  const TimeCopy& copy, hipStream_t st) {
     int rc = launch_sort(src, S, ws.sorted, ws.perm, ws.n_real, (int)ws.stride, np.max_cmp, st);
     if (rc) return rc;
     rc = launch_unpad_rows(ws.sorted, ws.perm, sorted_z, perm, S, I, ws.stride, st);
     if (rc) return rc;
-    return launch_scan(ws.sorted, ws.perm, ws.n_real, w, out, out + S * J, causal_k, S, I, ws.stride, J, np, st);
+    return launch_scan(ws.sorted, ws.perm, ws.n_real, w, out, out + S * J, causal_k, S, I, ws.stride, J, np, copy, st);
 }
 
 // Backward scratch.  `rows` is the weight row count including a possible bias row; the partial-sum
@@ -202,7 +202,7 @@ int fc_forward_impl(const float* x, const float* w, const float* params, float* 
     const NeuronParams np = neuron_params(params[0], params[2], params[5]);
     SegmentSource src{};
     src.base = x; src.conv = 0; src.I = (int)I;
-    return forward_chain(src, ws, w, out, sorted_z, perm, causal_k, B, I, J, np, st);
+    return forward_chain(src, ws, w, out, sorted_z, perm, causal_k, B, I, J, np, TimeCopy{}, st);
 }
 
 // ---- conv --------------------------------------------------------------------------------------
@@ -250,12 +250,25 @@ SegmentSource conv_source(const float* xpad, const ConvGeom& g) {
     return src;
 }
 
+// next_xpad (may be NULL): a second copy of the spike times, placed as pixel (nh + next_top, nw + next_left)
+// of an image tensor [B, next_h, next_w, Kc]
 int cv_forward_impl(const float* xpad, const float* w, const float* params, float* out, float* sorted_z,
-                    int32_t* perm, int32_t* causal_k, int64_t B, int64_t H, int64_t W, int64_t C, int64_t Kc,
+                    int32_t* perm, int32_t* causal_k, float* next_xpad, int64_t next_h, int64_t next_w,
+                    int64_t next_top, int64_t next_left, int64_t B, int64_t H, int64_t W, int64_t C, int64_t Kc,
                     int64_t w_rows, void* workspace, size_t workspace_bytes, void* stream) {
     ConvGeom g;
     int rc = cv_geom(B, H, W, C, Kc, w_rows, params, true, "snntc_cv_forward", &g);
     if (rc) return rc;
+    TimeCopy copy{};
+    if (next_xpad) {
+        if (next_top < 0 || next_left < 0 || next_h < next_top + g.Nh || next_w < next_left + g.Nw)
+            return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_cv_forward_chained: the %lld x %lld output does not fit the "
+                        "%lld x %lld destination at offset (%lld, %lld)", (long long)g.Nh, (long long)g.Nw,
+                        (long long)next_h, (long long)next_w, (long long)next_top, (long long)next_left);
+        if (B * next_h * next_w * Kc > kInt32Max)
+            return fail(SNNTC_ERR_TOO_LARGE, "snntc_cv_forward_chained: Too many elements in the destination tensor");
+        copy = TimeCopy{next_xpad, (int)g.Nh, (int)g.Nw, (int)next_h, (int)next_w, (int)next_top, (int)next_left};
+    }
     if (g.S == 0 || Kc == 0) return SNNTC_OK;
     if (!xpad || !w || !out) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_cv_forward: NULL tensor pointer");
     const bool merge = merge_sort_supported(g);
@@ -265,7 +278,7 @@ int cv_forward_impl(const float* xpad, const float* w, const float* params, floa
     hipStream_t st = static_cast<hipStream_t>(stream);
     const NeuronParams np = neuron_params(params[0], params[4], params[11]);
     if (!merge)
-        return forward_chain(conv_source(xpad, g), ws, w, out, sorted_z, perm, causal_k, g.S, g.P, Kc, np, st);
+        return forward_chain(conv_source(xpad, g), ws, w, out, sorted_z, perm, causal_k, g.S, g.P, Kc, np, copy, st);
     // sort every pixel's channels once, then assemble the patches by rank merging
     SegmentSource pixels{};
     pixels.base = xpad; pixels.conv = 0; pixels.I = (int)C;
@@ -277,7 +290,7 @@ int cv_forward_impl(const float* xpad, const float* w, const float* params, floa
     rc = launch_unpad_rows(ws.sorted, ws.perm, sorted_z, perm, g.S, g.P, ws.stride, st);
     if (rc) return rc;
     return launch_scan(ws.sorted, ws.perm, ws.n_real, w, out, out + g.S * Kc, causal_k, g.S, g.P, ws.stride, Kc, np,
-                       st);
+                       copy, st);
 }
 
 
@@ -369,7 +382,28 @@ int snntc_min_pool_forward(const float* x, float* y, int32_t* arg, int64_t B, in
     if (rc) return rc;
     if (B * Nh * Nw * C == 0) return SNNTC_OK;
     if (!y || (!x && B * H * W * C > 0)) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_min_pool_forward: NULL tensor pointer");
-    return launch_min_pool_forward(x, y, arg, g, pad_value, static_cast<hipStream_t>(stream));
+    return launch_min_pool_forward(x, y, arg, g, pad_value, TimeCopy{}, static_cast<hipStream_t>(stream));
+}
+
+int snntc_min_pool_forward_chained(const float* x, float* y, int32_t* arg, float* next_xpad, int64_t next_h,
+                                   int64_t next_w, int64_t next_top, int64_t next_left, int64_t B, int64_t H, int64_t W,
+                                   int64_t C, int64_t Kh, int64_t Kw, int64_t Sh, int64_t Sw, int64_t pad_top,
+                                   int64_t pad_left, int64_t Nh, int64_t Nw, float pad_value, void* stream) {
+    PoolGeom g;
+    int rc = pool_geom(B, H, W, C, Kh, Kw, Sh, Sw, pad_top, pad_left, Nh, Nw, "snntc_min_pool_forward_chained", &g);
+    if (rc) return rc;
+    if (!next_xpad) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_min_pool_forward_chained: next_xpad is NULL");
+    if (next_top < 0 || next_left < 0 || next_h < next_top + Nh || next_w < next_left + Nw)
+        return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_min_pool_forward_chained: the %lld x %lld output does not fit the "
+                    "%lld x %lld destination at offset (%lld, %lld)", (long long)Nh, (long long)Nw, (long long)next_h,
+                    (long long)next_w, (long long)next_top, (long long)next_left);
+    if (B * next_h * next_w * C > kInt32Max)
+        return fail(SNNTC_ERR_TOO_LARGE, "snntc_min_pool_forward_chained: Too many elements in the destination tensor");
+    if (B * Nh * Nw * C == 0) return SNNTC_OK;
+    if (!y || (!x && B * H * W * C > 0))
+        return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_min_pool_forward_chained: NULL tensor pointer");
+    const TimeCopy copy{next_xpad, (int)Nh, (int)Nw, (int)next_h, (int)next_w, (int)next_top, (int)next_left};
+    return launch_min_pool_forward(x, y, arg, g, pad_value, copy, static_cast<hipStream_t>(stream));
 }
 
 int snntc_min_pool_backward(const float* grad_y, const int32_t* arg, float* dx, int64_t B, int64_t H, int64_t W,
@@ -600,22 +634,32 @@ int snntc_cv_backward_workspace_bytes(int64_t B, int64_t H, int64_t W, int64_t C
 int snntc_cv_forward(const float* xpad, const float* w, const float* params_host, float* out, int64_t B,
                      int64_t H, int64_t W, int64_t C, int64_t Kc, int64_t w_rows, void* workspace,
                      size_t workspace_bytes, void* stream) {
-    return cv_forward_impl(xpad, w, params_host, out, nullptr, nullptr, nullptr, B, H, W, C, Kc, w_rows,
-                           workspace, workspace_bytes, stream);
+    return cv_forward_impl(xpad, w, params_host, out, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, B, H, W, C, Kc,
+                           w_rows, workspace, workspace_bytes, stream);
+}
+
+int snntc_cv_forward_chained(const float* xpad, const float* w, const float* params_host, float* out,
+                             float* next_xpad, int64_t next_h, int64_t next_w, int64_t next_top, int64_t next_left,
+                             int64_t B, int64_t H, int64_t W, int64_t C, int64_t Kc, int64_t w_rows,
+                             void* workspace, size_t workspace_bytes, void* stream) {
+    if (!next_xpad) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_cv_forward_chained: next_xpad is NULL");
+    return cv_forward_impl(xpad, w, params_host, out, nullptr, nullptr, nullptr, next_xpad, next_h, next_w, next_top,
+                           next_left, B, H, W, C, Kc, w_rows, workspace, workspace_bytes, stream);
 }
 
 int snntc_cv_forward_ex(const float* xpad, const float* w, const float* params_host, float* out,
                         float* sorted_z, int32_t* perm, int32_t* causal_k, int64_t B, int64_t H, int64_t W,
                         int64_t C, int64_t Kc, int64_t w_rows, void* workspace, size_t workspace_bytes,
                         void* stream) {
-    return cv_forward_impl(xpad, w, params_host, out, sorted_z, perm, causal_k, B, H, W, C, Kc, w_rows,
-                           workspace, workspace_bytes, stream);
+    return cv_forward_impl(xpad, w, params_host, out, sorted_z, perm, causal_k, nullptr, 0, 0, 0, 0, B, H, W, C, Kc,
+                           w_rows, workspace, workspace_bytes, stream);
 }
 
-int snntc_cv_backward(const float* grad, const float* xpad, const float* w, const float* params_host,
-                      const float* oldout, float* dxpad, float* dw, float* dparams, int64_t B, int64_t H,
-                      int64_t W, int64_t C, int64_t Kc, int64_t w_rows, int64_t grad_rows, void* workspace,
-                      size_t workspace_bytes, void* stream) {
+// dx[B, crop.h, crop.w, C]: the window of the padded input's gradient that starts at (crop.top, crop.left)
+static int cv_backward_impl(const float* grad, const float* xpad, const float* w, const float* params_host,
+                            const float* oldout, float* dxpad, CropGeom crop, float* dw, float* dparams, int64_t B,
+                            int64_t H, int64_t W, int64_t C, int64_t Kc, int64_t w_rows, int64_t grad_rows,
+                            void* workspace, size_t workspace_bytes, void* stream) {
     ConvGeom g;
     int rc = cv_geom(B, H, W, C, Kc, w_rows, params_host, true, "snntc_cv_backward", &g);
     if (rc) return rc;
@@ -626,7 +670,7 @@ int snntc_cv_backward(const float* grad, const float* xpad, const float* w, cons
     if (!dxpad && !dw) return dparams ? launch_fill_zero(dparams, 12, st) : SNNTC_OK;   // a NULL gradient output is simply not computed
     if (g.S == 0 || Kc == 0) {
         if (dparams) { rc = launch_fill_zero(dparams, 12, st); if (rc) return rc; }
-        if (dxpad) { rc = launch_fill_zero(dxpad, B * H * W * C, st); if (rc) return rc; }
+        if (dxpad) { rc = launch_fill_zero(dxpad, B * crop.h * crop.w * C, st); if (rc) return rc; }
         return dw ? launch_fill_zero(dw, w_rows * Kc, st) : SNNTC_OK;
     }
     if (!grad || !xpad || !w || !oldout) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_cv_backward: NULL tensor pointer");
@@ -643,9 +687,9 @@ int snntc_cv_backward(const float* grad, const float* xpad, const float* w, cons
     if (rc) return rc;
     if (dxpad) {
         if (chan_dx) {
-            rc = launch_cv_grad_input_chan(xpad, ws.wt, ws.upm, ws.ym, dxpad, g, np, st);
+            rc = launch_cv_grad_input_chan(xpad, ws.wt, ws.upm, ws.ym, dxpad, crop, g, np, st);
         } else {
-            rc = launch_cv_grad_input(conv_source(xpad, g), ws.wt, ws.upm, ws.ym, ws.dxp, dxpad, g, g.P, st);
+            rc = launch_cv_grad_input(conv_source(xpad, g), ws.wt, ws.upm, ws.ym, ws.dxp, dxpad, crop, g, g.P, st);
         }
         if (rc) return rc;
     }
@@ -662,6 +706,28 @@ int snntc_cv_backward(const float* grad, const float* xpad, const float* w, cons
     }
     if (rc) return rc;
     return launch_reduce_partials(ws.partial, dw, w_rows * Kc, nsplit, st);
+}
+
+int snntc_cv_backward(const float* grad, const float* xpad, const float* w, const float* params_host,
+                      const float* oldout, float* dxpad, float* dw, float* dparams, int64_t B, int64_t H,
+                      int64_t W, int64_t C, int64_t Kc, int64_t w_rows, int64_t grad_rows, void* workspace,
+                      size_t workspace_bytes, void* stream) {
+    return cv_backward_impl(grad, xpad, w, params_host, oldout, dxpad, CropGeom{(int)H, (int)W, 0, 0}, dw, dparams, B,
+                            H, W, C, Kc, w_rows, grad_rows, workspace, workspace_bytes, stream);
+}
+
+int snntc_cv_backward_cropped(const float* grad, const float* xpad, const float* w, const float* params_host,
+                              const float* oldout, float* dx, int64_t dx_h, int64_t dx_w, int64_t dx_top,
+                              int64_t dx_left, float* dw, float* dparams, int64_t B, int64_t H, int64_t W, int64_t C,
+                              int64_t Kc, int64_t w_rows, int64_t grad_rows, void* workspace, size_t workspace_bytes,
+                              void* stream) {
+    if (dx_h < 0 || dx_w < 0 || dx_top < 0 || dx_left < 0 || dx_top + dx_h > H || dx_left + dx_w > W)
+        return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_cv_backward_cropped: the %lld x %lld window at (%lld, %lld) does not "
+                    "lie inside the %lld x %lld padded image", (long long)dx_h, (long long)dx_w, (long long)dx_top,
+                    (long long)dx_left, (long long)H, (long long)W);
+    return cv_backward_impl(grad, xpad, w, params_host, oldout, dx,
+                            CropGeom{(int)dx_h, (int)dx_w, (int)dx_top, (int)dx_left}, dw, dparams, B, H, W, C, Kc,
+                            w_rows, grad_rows, workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

@@ -65,8 +65,9 @@ template <int KCB, int HALVES>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KCB == 64 && HALVES == 2 ? 3 : 4)))
 cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restrict__ wq,
                           const float* __restrict__ upm, const float* __restrict__ ym,
-                          float* __restrict__ dxpad, int H, int W, int C, int Kc, int Kh, int Kw, int Sh, int Sw,
-                          int Nh, int Nw, int tiles_w, int c_blocks, int64_t n_items, float max_cmp, int ksplit) {
+                          float* __restrict__ dx, CropGeom crop, int H, int W, int C, int Kc, int Kh, int Kw, int Sh,
+                          int Sw, int Nh, int Nw, int tiles_w, int c_blocks, int64_t n_items, float max_cmp,
+                          int ksplit) {
     extern __shared__ __align__(16) float staged[];                    // per wavefront: [2][n_slots + 1][KCB]
     __shared__ float partial[3][DX_TILE][kWave];         // ksplit = 4: sums of wavefronts 1..3
     constexpr int SPAN = DX_TILE * HALVES;               // pixels of one wavefront
@@ -209,11 +210,15 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
         for (int t = 0; t < DX_TILE; ++t)
             acc[t] = ((acc[t] + partial[0][t][lane]) + partial[1][t][lane]) + partial[2][t][lane];
     }
-    if (lane_ok) {
-        float* __restrict__ orow = dxpad + ((size_t)(a * H + h) * W) * C + c;
+    // only the pixels inside the caller's window of the padded image are stored
+    const int oh = h - crop.top;
+    if (lane_ok && oh >= 0 && oh < crop.h) {
+        float* __restrict__ orow = dx + ((size_t)(a * crop.h + oh) * crop.w) * C + c;
 #pragma unroll
-        for (int t = 0; t < DX_TILE; ++t)
-            if (p0 + t < W) orow[(size_t)(p0 + t) * C] = acc[t];
+        for (int t = 0; t < DX_TILE; ++t) {
+            const int ow = p0 + t - crop.left;
+            if (p0 + t < W && ow >= 0 && ow < crop.w) orow[(size_t)ow * C] = acc[t];
+        }
     }
 }
 
@@ -431,7 +436,8 @@ bool cv_grad_input_chan_supported(const ConvGeom& g) {
 
 // wq: the weights regrouped by launch_backward_prologue (mode 2)
 int launch_cv_grad_input_chan(const float* xpad, const float* wq, const float* upm, const float* ym,
-                              float* dxpad, const ConvGeom& g, const NeuronParams& np, hipStream_t stream) {
+                              float* dx, const CropGeom& crop, const ConvGeom& g, const NeuronParams& np,
+                              hipStream_t stream) {
     const int halves = g.C <= 32 ? 2 : 1;
     const int span = DX_TILE * halves;
     const int tiles_w = (int)((g.W + span - 1) / span);
@@ -446,8 +452,8 @@ int launch_cv_grad_input_chan(const float* xpad, const float* wq, const float* u
     if (blocks > 0x7fffffffLL) return fail(SNNTC_ERR_TOO_LARGE, "conv backward: grid too large");
     dim3 grid((unsigned)blocks), block(256);
     const size_t lds = (size_t)4 * 2 * (span + g.Kw) * kcb * sizeof(float);
-    void (*kern)(const float*, const float*, const float*, const float*, float*, int, int, int, int, int, int, int,
-                 int, int, int, int, int, int64_t, float, int);
+    void (*kern)(const float*, const float*, const float*, const float*, float*, CropGeom, int, int, int, int, int, int,
+                 int, int, int, int, int, int, int64_t, float, int);
     if (halves == 2)
         kern = kcb == 64 ? cv_grad_input_chan_kernel<64, 2> : kcb == 32 ? cv_grad_input_chan_kernel<32, 2>
                                                                          : cv_grad_input_chan_kernel<16, 2>;
@@ -456,7 +462,7 @@ int launch_cv_grad_input_chan(const float* xpad, const float* wq, const float* u
                                                                          : cv_grad_input_chan_kernel<16, 1>;
     {
         KernelTimerScope timer_("cv_grad_input", stream);
-        hipLaunchKernelGGL(kern, grid, block, lds, stream, xpad, wq, upm, ym, dxpad, (int)g.H, (int)g.W, (int)g.C,
+        hipLaunchKernelGGL(kern, grid, block, lds, stream, xpad, wq, upm, ym, dx, crop, (int)g.H, (int)g.W, (int)g.C,
                            (int)g.Kc, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.Nh, (int)g.Nw, tiles_w,
                            c_blocks, n_items, np.max_cmp, ksplit);
     }

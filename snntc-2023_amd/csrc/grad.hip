@@ -532,8 +532,8 @@ reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ ou
 // (kh, kw) order.  Gather form: no atomics, fixed summation order.
 // ---------------------------------------------------------------------------------------------
 __global__ void __launch_bounds__(256)
-cv_col2im_kernel(const float* __restrict__ dxp, float* __restrict__ dxpad, int64_t n, int H, int W, int C, int Kh,
-                 int Kw, int Sh, int Sw, int Nh, int Nw) {
+cv_col2im_kernel(const float* __restrict__ dxp, float* __restrict__ dx, CropGeom crop, int64_t n, int H, int W, int C,
+                 int Kh, int Kw, int Sh, int Sw, int Nh, int Nw) {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= n) return;
     const int c = (int)(t % C);
@@ -542,6 +542,8 @@ cv_col2im_kernel(const float* __restrict__ dxp, float* __restrict__ dxpad, int64
     const int64_t rowi = pix / W;
     const int h = (int)(rowi % H);
     const int a = (int)(rowi / H);
+    const int oh = h - crop.top, ow = wx - crop.left;         // only the caller's window is stored
+    if (oh < 0 || oh >= crop.h || ow < 0 || ow >= crop.w) return;
     const int P = Kh * Kw * C;
     float acc = 0.0f;
     for (int kh = 0; kh < Kh; ++kh) {
@@ -554,7 +556,7 @@ cv_col2im_kernel(const float* __restrict__ dxp, float* __restrict__ dxpad, int64
             acc += dxp[s * P + (kh * Kw + kw) * C + c];
         }
     }
-    dxpad[t] = acc;
+    dx[(((size_t)a * crop.h + oh) * crop.w + ow) * C + c] = acc;
 }
 
 int blocks_for(int64_t n, int block) { return (int)((n + block - 1) / block); }
@@ -701,10 +703,10 @@ int launch_fc_backward_narrow(const float* x, const float* w, const float* grad,
 
 // dxp: scratch of S * P floats (gradient per patch element)
 int launch_cv_grad_input(const SegmentSource& src, const float* wt, const float* upm, const float* ym, float* dxp,
-                         float* dxpad, const ConvGeom& g, int64_t wt_stride, hipStream_t stream) {
+                         float* dx, const CropGeom& crop, const ConvGeom& g, int64_t wt_stride, hipStream_t stream) {
     const int64_t n = g.B * g.H * g.W * g.C;
     if (n <= 0) return SNNTC_OK;
-    if (g.Kc <= 0 || g.S <= 0) return launch_fill_zero(dxpad, n, stream);
+    if (g.Kc <= 0 || g.S <= 0) return launch_fill_zero(dx, g.B * crop.h * crop.w * g.C, stream);
     dim3 grid((unsigned)((g.S + DX_RB - 1) / DX_RB), (unsigned)((g.P + kWave - 1) / kWave));
     if (grid.y > 65535u) return fail(SNNTC_ERR_TOO_LARGE, "conv backward: patch length %lld too large", (long long)g.P);
     { KernelTimerScope timer_("cv_grad_input", stream);
@@ -713,7 +715,7 @@ int launch_cv_grad_input(const SegmentSource& src, const float* wt, const float*
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     { KernelTimerScope timer_("cv_col2im", stream);
-    hipLaunchKernelGGL(cv_col2im_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream, dxp, dxpad, n, (int)g.H,
+    hipLaunchKernelGGL(cv_col2im_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream, dxp, dx, crop, n, (int)g.H,
                        (int)g.W, (int)g.C, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.Nh, (int)g.Nw);
     }
     SNNTC_HIP_CHECK(hipGetLastError());

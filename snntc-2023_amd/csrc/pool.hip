@@ -37,7 +37,7 @@ template <int VEC>
 __global__ void __launch_bounds__(256)
 min_pool_forward_kernel(const float* __restrict__ x, float* __restrict__ y, int32_t* __restrict__ arg, int H, int W,
                         int C, int Kh, int Kw, int Sh, int Sw, int pad_top, int pad_left, int Nh, int Nw,
-                        float pad_value, FastDiv by_c) {
+                        float pad_value, FastDiv by_c, TimeCopy copy) {
     const unsigned e = (blockIdx.y * 256u + threadIdx.x) * VEC;
     if (e >= (unsigned)(Nw * C)) return;
     const unsigned nw = fast_div(e, by_c), c = e - nw * (unsigned)C;
@@ -77,6 +77,11 @@ min_pool_forward_kernel(const float* __restrict__ x, float* __restrict__ y, int3
     } else {
         y[t] = best[0];
         if (arg) arg[t] = where[0];
+    }
+    if (copy.dst) {                                      // the same times inside the next layer's padded input
+        float* q = copy.dst + (((size_t)b * copy.h + nh + copy.top) * copy.w + nw + copy.left) * C + c;
+        if (VEC == 4) *reinterpret_cast<float4*>(q) = make_float4(best[0], best[1], best[2], best[3]);
+        else *q = best[0];
     }
 }
 
@@ -215,10 +220,10 @@ int launch_crop_time(const float* dxpad, float* dx, const PadGeom& g, hipStream_
 static bool aligned16(const void* p) { return (uintptr_t)p % 16 == 0; }
 
 int launch_min_pool_forward(const float* x, float* y, int32_t* arg, const PoolGeom& g, float pad_value,
-                            hipStream_t stream) {
+                            const TimeCopy& copy, hipStream_t stream) {
     const int64_t rows = g.B * g.Nh, per_row = g.Nw * g.C;
     if (rows <= 0 || per_row <= 0) return SNNTC_OK;
-    const bool vec = g.C % 4 == 0 && aligned16(x) && aligned16(y) && aligned16(arg);
+    const bool vec = g.C % 4 == 0 && aligned16(x) && aligned16(y) && aligned16(arg) && aligned16(copy.dst);
     const int64_t threads = vec ? per_row / 4 : per_row;
     dim3 grid((unsigned)rows, (unsigned)((threads + 255) / 256));
     if (grid.y > 65535u) return fail(SNNTC_ERR_TOO_LARGE, "pooling: output row of %lld elements too long", (long long)per_row);
@@ -227,7 +232,7 @@ int launch_min_pool_forward(const float* x, float* y, int32_t* arg, const PoolGe
         auto kern = vec ? min_pool_forward_kernel<4> : min_pool_forward_kernel<1>;
         hipLaunchKernelGGL(kern, grid, dim3(256), 0, stream, x, y, arg, (int)g.H, (int)g.W, (int)g.C, (int)g.Kh,
                            (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.pad_top, (int)g.pad_left, (int)g.Nh, (int)g.Nw,
-                           pad_value, make_fast_div(g.C, per_row));
+                           pad_value, make_fast_div(g.C, per_row), copy);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;

@@ -52,7 +52,7 @@ __global__ void __launch_bounds__(256)
 scan_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
             const int32_t* __restrict__ n_real, const float* __restrict__ w, float* __restrict__ y_out,
             float* __restrict__ rcp_out, int32_t* __restrict__ k_out, int64_t n_items, int I, int stride,
-            int J, int j_blocks, NeuronParams np) {
+            int J, int j_blocks, NeuronParams np, TimeCopy copy) {
     // work item = (segment, 64-neuron block); one per wavefront
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int64_t item = (int64_t)blockIdx.x * (blockDim.x / kWave) + wave;
@@ -125,6 +125,7 @@ scan_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
         const size_t o = (size_t)seg * J + j;
         y_out[o] = y;
         rcp_out[o] = r;
+        if (copy.dst) copy.dst[time_copy_pixel(copy, seg) * J + j] = y;
         if (WANT_K) k_out[o] = (s.fired && r != 0.0f) ? kcnt : -1;
     }
 }
@@ -355,7 +356,7 @@ __global__ void __launch_bounds__(LOW_LATENCY_THREADS)
 scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
                 const int32_t* __restrict__ n_real, const float* __restrict__ w, float* __restrict__ y_out,
                 float* __restrict__ rcp_out, int32_t* __restrict__ k_out, int S, int I, int stride, int J,
-                int n_slices, int n_groups, NeuronParams np) {
+                int n_slices, int n_groups, NeuronParams np, TimeCopy copy) {
     extern __shared__ __align__(16) float wl[];                          // [I + bias][COLS]
     constexpr int SEGS = kWave / COLS;                     // segments per wavefront
     const int WAVES = blockDim.x / kWave;                  // 1..4, chosen by the launcher
@@ -450,6 +451,7 @@ scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ pe
             const size_t o = (size_t)seg * J + j;
             y_out[o] = y;
             rcp_out[o] = r;
+            if (copy.dst) copy.dst[time_copy_pixel(copy, seg) * J + j] = y;
             if (WANT_K) k_out[o] = (s.fired && r != 0.0f) ? kcnt : -1;
         }
     }
@@ -481,7 +483,7 @@ __global__ void __launch_bounds__(LOW_LATENCY_THREADS)
 scan_lds_split_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
                       const int32_t* __restrict__ n_real, const float* __restrict__ w, float* __restrict__ y_out,
                       float* __restrict__ rcp_out, int32_t* __restrict__ k_out, int S, int I, int stride, int J,
-                      int n_slices, int n_groups, NeuronParams np) {
+                      int n_slices, int n_groups, NeuronParams np, TimeCopy copy) {
     extern __shared__ __align__(16) float wl[];                          // [I + bias][COLS], rows, sums
     __shared__ int k_found[SPLIT_WAVES][kWave];
     __shared__ float w_found[SPLIT_WAVES][kWave], y_found[SPLIT_WAVES][kWave];
@@ -676,6 +678,7 @@ scan_lds_split_kernel(const float* __restrict__ sorted, const int32_t* __restric
             const size_t o = (size_t)seg * J + j;
             y_out[o] = y;
             rcp_out[o] = r;
+            if (copy.dst) copy.dst[time_copy_pixel(copy, seg) * J + j] = y;
             if (WANT_K) k_out[o] = (fired && r != 0.0f) ? (kb != NONE ? kb : consumed) : -1;
         }
         __syncthreads();                                    // LDS is reused by the next item
@@ -822,7 +825,7 @@ __global__ void __launch_bounds__(LDS_SCAN_THREADS)
 scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
                    const int32_t* __restrict__ n_real, const float* __restrict__ w, float* __restrict__ y_out,
                    float* __restrict__ rcp_out, int32_t* __restrict__ k_out, int S, int I, int stride, int J,
-                   int n_slices, int n_groups, NeuronParams np) {
+                   int n_slices, int n_groups, NeuronParams np, TimeCopy copy) {
     extern __shared__ __align__(16) float wl[];                          // [I + bias][COLS], then `red`
     constexpr int LANES = COLS / CH;                       // lanes per segment
     constexpr int SEGS = kWave / LANES;                    // segments per wavefront
@@ -1071,6 +1074,7 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
             const size_t o = (size_t)seg * J + j + c;
             y_out[o] = y;
             rcp_out[o] = r;
+            if (copy.dst) copy.dst[time_copy_pixel(copy, seg) * J + j + c] = y;
             if (WANT_K) k_out[o] = (st.fired && r != 0.0f) ? kc : -1;
         }
     }
@@ -1140,7 +1144,7 @@ int scan_prepare_device(int dev, int* cu_count_out) {
 template <int COLS>
 int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_real, const float* w, float* y,
                     float* rcp, int32_t* causal_k, int64_t S, int64_t I, int64_t stride, int64_t J,
-                    const NeuronParams& np, size_t lds_bytes, hipStream_t stream) {
+                    const NeuronParams& np, const TimeCopy& copy, size_t lds_bytes, hipStream_t stream) {
     int dev = 0, cus = 0;
     SNNTC_HIP_CHECK(hipGetDevice(&dev));
     const int prep = scan_prepare_device(dev, &cus);
@@ -1194,10 +1198,10 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
         const size_t dyn_lds = filt ? lds_bytes + FILTER_RED_BYTES : split ? split_lds : lds_bytes;
         if (causal_k)
             hipLaunchKernelGGL(kern_k, grid, block, dyn_lds, stream, sorted, perm, n_real, w, y, rcp, causal_k,
-                               (int)S, (int)I, (int)stride, (int)J, n_slices, (int)n_groups, np);
+                               (int)S, (int)I, (int)stride, (int)J, n_slices, (int)n_groups, np, copy);
         else
             hipLaunchKernelGGL(kern, grid, block, dyn_lds, stream, sorted, perm, n_real, w, y, rcp, causal_k,
-                               (int)S, (int)I, (int)stride, (int)J, n_slices, (int)n_groups, np);
+                               (int)S, (int)I, (int)stride, (int)J, n_slices, (int)n_groups, np, copy);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
@@ -1205,7 +1209,7 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
 
 int launch_scan(const float* sorted, const int32_t* perm, const int32_t* n_real, const float* w, float* y,
                 float* rcp, int32_t* causal_k, int64_t S, int64_t I, int64_t stride, int64_t J,
-                const NeuronParams& np, hipStream_t stream) {
+                const NeuronParams& np, const TimeCopy& copy, hipStream_t stream) {
     if (S <= 0 || J <= 0) return SNNTC_OK;
     // widest column slice (8..64) whose I+bias rows fit in LDS; none fits -> stream W from memory
     const size_t rows = (size_t)I + np.bias;
@@ -1214,10 +1218,10 @@ int launch_scan(const float* sorted, const int32_t* perm, const int32_t* n_real,
     const size_t lds_bytes = rows * cols * sizeof(float);
     if (lds_bytes <= (size_t)LDS_SCAN_BYTES) {
         switch (cols) {
-            case 64: return launch_scan_lds<64>(sorted, perm, n_real, w, y, rcp, causal_k, S, I, stride, J, np, lds_bytes, stream);
-            case 32: return launch_scan_lds<32>(sorted, perm, n_real, w, y, rcp, causal_k, S, I, stride, J, np, lds_bytes, stream);
-            case 16: return launch_scan_lds<16>(sorted, perm, n_real, w, y, rcp, causal_k, S, I, stride, J, np, lds_bytes, stream);
-            default: return launch_scan_lds<8>(sorted, perm, n_real, w, y, rcp, causal_k, S, I, stride, J, np, lds_bytes, stream);
+            case 64: return launch_scan_lds<64>(sorted, perm, n_real, w, y, rcp, causal_k, S, I, stride, J, np, copy, lds_bytes, stream);
+            case 32: return launch_scan_lds<32>(sorted, perm, n_real, w, y, rcp, causal_k, S, I, stride, J, np, copy, lds_bytes, stream);
+            case 16: return launch_scan_lds<16>(sorted, perm, n_real, w, y, rcp, causal_k, S, I, stride, J, np, copy, lds_bytes, stream);
+            default: return launch_scan_lds<8>(sorted, perm, n_real, w, y, rcp, causal_k, S, I, stride, J, np, copy, lds_bytes, stream);
         }
     }
     const int j_blocks = (int)((J + kWave - 1) / kWave);
@@ -1230,10 +1234,10 @@ int launch_scan(const float* sorted, const int32_t* perm, const int32_t* n_real,
         KernelTimerScope timer_("scan_stream", stream);
         if (causal_k)
             hipLaunchKernelGGL(scan_kernel<true>, grid, block, 0, stream, sorted, perm, n_real, w, y, rcp,
-                               causal_k, n_items, (int)I, (int)stride, (int)J, j_blocks, np);
+                               causal_k, n_items, (int)I, (int)stride, (int)J, j_blocks, np, copy);
         else
             hipLaunchKernelGGL(scan_kernel<false>, grid, block, 0, stream, sorted, perm, n_real, w, y, rcp,
-                               causal_k, n_items, (int)I, (int)stride, (int)J, j_blocks, np);
+                               causal_k, n_items, (int)I, (int)stride, (int)J, j_blocks, np, copy);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;

@@ -93,6 +93,26 @@ struct ConvGeom {
     int64_t B, H, W, C, Kc, Kh, Kw, Sh, Sw, Nh, Nw, P, S;
 };
 
+// Optional second destination of the spike times a scan writes: an NHWC image tensor [*, h, w, J]
+// in which segment s = (a * Nh + nh) * Nw + nw is pixel (nh + top, nw + left) of image a -- the
+// padded input of the next layer, whose border the caller has filled.  dst == NULL: none.
+struct TimeCopy {
+    float* dst;
+    int Nh, Nw, h, w, top, left;
+};
+__device__ __forceinline__ size_t time_copy_pixel(const TimeCopy& tc, int seg) {
+    const int per_image = tc.Nh * tc.Nw;
+    const int a = seg / per_image, r = seg - a * per_image;
+    const int nh = r / tc.Nw, nw = r - nh * tc.Nw;
+    return ((size_t)a * tc.h + nh + tc.top) * tc.w + nw + tc.left;
+}
+
+// The window of the padded input's gradient that conv dX stores:
+// dx[B, h, w, C] = dxpad[:, top : top + h, left : left + w, :] (the whole of it: {H, W, 0, 0}).
+struct CropGeom {
+    int h, w, top, left;
+};
+
 // ---- launchers (each enqueues on `stream` and returns a status) --------------------------------
 
 // Row stride of the sorted / perm scratch arrays: segments are padded to a multiple of 16 entries
@@ -118,7 +138,7 @@ int launch_unpad_rows(const float* sorted, const int32_t* perm, float* sorted_ou
 // y[S,J], rcp[S,J], optional causal_k[S,J].
 int launch_scan(const float* sorted, const int32_t* perm, const int32_t* n_real, const float* w, float* y,
                 float* rcp, int32_t* causal_k, int64_t S, int64_t I, int64_t stride, int64_t J,
-                const NeuronParams& np, hipStream_t stream);
+                const NeuronParams& np, const TimeCopy& copy, hipStream_t stream);
 
 // One-time set-up on device `dev`, which must be the current device: the dynamic-LDS limits of every
 // scan / merge instantiation (and the CU count the scan sizes its launches with).  The launchers call
@@ -160,7 +180,8 @@ int launch_fc_backward_narrow(const float* x, const float* w, const float* grad,
 bool cv_grad_input_chan_supported(const ConvGeom& g);
 // launch_cv_grad_input_chan reads the weights from the copy regrouped by launch_backward_prologue (mode 2).
 int launch_cv_grad_input_chan(const float* xpad, const float* wq, const float* upm, const float* ym,
-                              float* dxpad, const ConvGeom& g, const NeuronParams& np, hipStream_t stream);
+                              float* dx, const CropGeom& crop, const ConvGeom& g, const NeuronParams& np,
+                              hipStream_t stream);
 bool cv_grad_weight_wide_supported(const ConvGeom& g);
 int cv_grad_weight_wide_blocks(const ConvGeom& g);
 int launch_cv_grad_weight_wide(const float* xpad, const float* upm, const float* ym, float* dst, int nsplit,
@@ -168,7 +189,7 @@ int launch_cv_grad_weight_wide(const float* xpad, const float* upm, const float*
 
 // Conv dX for layers launch_cv_grad_input_chan does not take; dxp is scratch of S * P floats.
 int launch_cv_grad_input(const SegmentSource& src, const float* wt, const float* upm, const float* ym, float* dxp,
-                         float* dxpad, const ConvGeom& g, int64_t wt_stride, hipStream_t stream);
+                         float* dx, const CropGeom& crop, const ConvGeom& g, int64_t wt_stride, hipStream_t stream);
 
 int launch_fill_zero(float* p, int64_t n, hipStream_t stream);
 
@@ -179,7 +200,7 @@ struct PoolGeom {
     int64_t B, H, W, C, Kh, Kw, Sh, Sw, pad_top, pad_left, Nh, Nw;
 };
 int launch_min_pool_forward(const float* x, float* y, int32_t* arg, const PoolGeom& g, float pad_value,
-                            hipStream_t stream);
+                            const TimeCopy& copy, hipStream_t stream);
 int launch_min_pool_backward(const float* gy, const int32_t* arg, float* dx, const PoolGeom& g, hipStream_t stream);
 
 // SAME padding of a conv layer's input with a constant (pool.hip): xpad[B,Hp,Wp,C] holds x[B,H,W,C]

@@ -6,7 +6,7 @@ Public names follow the reference module ``SNN_TC_Modules``: the op handles ``sn
 """
 from . import _lib
 from ._lib import SnntcError, SnntcLibraryError
-from .ops import SnnCv, SnnCvTimes, SnnFc, SnnFcTimes, SnnMinPool, SnnPadTime, SoftmaxTimeLoss, min_pool, min_pool_grad, pad_time, pad_time_grad, sgd_update, softmax_time_loss, snncv, snncv_grad, snncv_output_dims, snnfc, snnfc_grad, snnfc_static, init
+from .ops import SnnCv, SnnCvSame, SnnCvTimes, SnnFc, SnnFcTimes, SnnMinPool, SnnPadTime, SoftmaxTimeLoss, min_pool, min_pool_grad, pad_time, pad_time_grad, sgd_update, softmax_time_loss, snncv, snncv_grad, snncv_output_dims, snnfc, snnfc_grad, snnfc_static, init
 from . import train
 from . import networks
 from .layers import (SNN_LRN, SNN_avgpool2d, SNN_conv, SNN_dense, SNN_flatten, SNN_globalminpool2d, SNN_maxpool2d,

@@ -26,7 +26,8 @@ EXPORTS = (
     "snntc_fc_forward_workspace_bytes", "snntc_fc_backward_workspace_bytes",
     "snntc_fc_forward", "snntc_fc_forward_ex", "snntc_fc_backward",
     "snntc_cv_output_dims", "snntc_cv_forward_workspace_bytes", "snntc_cv_backward_workspace_bytes",
-    "snntc_cv_forward", "snntc_cv_forward_ex", "snntc_cv_backward",
+    "snntc_cv_forward", "snntc_cv_forward_ex", "snntc_cv_forward_chained", "snntc_cv_backward",
+    "snntc_cv_backward_cropped", "snntc_min_pool_forward_chained",
     "snntc_softmax_time_loss", "snntc_sgd_update",
     "snntc_min_pool_forward", "snntc_min_pool_backward",
     "snntc_pad_time_forward", "snntc_pad_time_backward",
@@ -93,6 +94,10 @@ def load():
     lib.snntc_cv_forward_ex.argtypes = [vp, vp, fparams, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, sz, vp]
     lib.snntc_cv_backward.argtypes = [vp, vp, vp, fparams, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64,
                                       vp, sz, vp]
+    lib.snntc_cv_forward_chained.argtypes = [vp, vp, fparams, vp, vp] + [i64] * 10 + [vp, sz, vp]
+    lib.snntc_cv_backward_cropped.argtypes = [vp, vp, vp, fparams, vp, vp, i64, i64, i64, i64, vp, vp] + [i64] * 7 + [
+        vp, sz, vp]
+    lib.snntc_min_pool_forward_chained.argtypes = [vp, vp, vp, vp] + [i64] * 16 + [c.c_float, vp]
     lib.snntc_softmax_time_loss.argtypes = [vp, vp, vp, vp, i64, i64, vp]
     lib.snntc_sgd_update.argtypes = [c.POINTER(vp), c.POINTER(vp), c.POINTER(i64), i64, c.c_float, vp]
     lib.snntc_min_pool_forward.argtypes = [vp, vp, vp] + [i64] * 12 + [c.c_float, vp]

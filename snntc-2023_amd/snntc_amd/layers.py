@@ -12,7 +12,7 @@ import numpy as np
 import torch
 import torch.nn.functional as F
 
-from .ops import SnnCvTimes, SnnFcTimes, SnnMinPool, SnnPadTime, SoftmaxTimeLoss
+from .ops import SnnCvSame, SnnCvTimes, SnnFcTimes, SnnMinPool, SnnPadTime, SoftmaxTimeLoss
 
 # Mirrors the reference's module-level switch (SNN_TC_Modules.py:11): when True the layers keep
 # the largest batch and element count they have seen in ``maxD`` (every tensor must stay below
@@ -131,6 +131,7 @@ class SNN_conv(torch.nn.Module, _CostsMixin):
         if tuple(weight.shape) != (self.in_size, self.Kc):
             raise ValueError(f"weight shape {tuple(weight.shape)} != {(self.in_size, self.Kc)}")
         self.weight = torch.nn.Parameter(torch.from_numpy(weight))
+        self._padded = {}                  # padded input buffers by (B, H, W, device), see padded_input_buffer
 
     def prepare_input(self, input):
         """The padded (SAME) or cropped (VALID) tensor handed to the op."""
@@ -141,8 +142,51 @@ class SNN_conv(torch.nn.Module, _CostsMixin):
         nw = int((W - self.Kw) / self.Sw + 1.0)
         return input[:, 0:(nh - 1) * self.Sh + self.Kh, 0:(nw - 1) * self.Sw + self.Kw, :]
 
-    def forward(self, input):
+    def same_pads(self, H, W):
+        """(top, bottom, left, right) of the SAME padding of an H x W image."""
+        top, bottom = _same_pad(H, self.Kh, self.Sh)
+        left, right = _same_pad(W, self.Kw, self.Sw)
+        if min(top, bottom, left, right) < 0:
+            raise ValueError("negative SAME padding: kernel smaller than stride is not supported")
+        return top, bottom, left, right
+
+    def padded_input_buffer(self, B, H, W, device):
+        """The layer's own padded input for B images of H x W (SAME mode): a tensor [B,Hp,Wp,C] that lives as
+        long as the layer, its border filled with MAX_SPIKE_TIME once, and (top, left), where the image
+        goes.  The layer before writes its output straight into the interior (`feed`), so no padding pass
+        runs between the two; the content belongs to the latest forward pass."""
+        top, bottom, left, right = self.same_pads(H, W)
+        key = (B, H, W, str(device))
+        buf = self._padded.get(key)
+        if buf is None:
+            buf = torch.full((B, top + H + bottom, left + W + right, self.C), float(self.Params[0]),
+                             dtype=torch.float32, device=device)
+            self._padded[key] = buf
+        return buf, (top, left)
+
+    def output_hw(self, H, W):
+        if self.padding == 'SAME':
+            return -(-H // self.Sh), -(-W // self.Sw)
+        return int((H - self.Kh) / self.Sh + 1.0), int((W - self.Kw) / self.Sw + 1.0)
+
+    def forward(self, input, prefilled=False, feed=None):
+        """prefilled: the layer before has written `input` into this layer's padded_input_buffer.
+        feed: the SNN_conv that follows; its padded input buffer receives this layer's output as well."""
         B = input.shape[0]
+        on_device = input.is_cuda and input.dtype == torch.float32 and input.dim() == 4
+        if self.padding == 'SAME' and on_device:
+            H, W = input.shape[1], input.shape[2]
+            xpad = self.padded_input_buffer(B, H, W, input.device)[0] if prefilled else None
+            next_xpad, next_offset = None, (0, 0)
+            if feed is not None:
+                nh, nw = self.output_hw(H, W)
+                next_xpad, next_offset = feed.padded_input_buffer(B, nh, nw, input.device)
+            if Check_Dim:
+                self.maxD[0] = max(self.maxD[0], int(B))
+            return SnnCvSame.apply(input.contiguous(), self.weight, self.Params, self.same_pads(H, W), xpad, next_xpad,
+                                   next_offset)
+        if prefilled or feed is not None:
+            raise ValueError("chaining needs SAME padding and float32 device tensors")
         X = self.prepare_input(input)
         if Check_Dim:
             self.maxD[0] = max(self.maxD[0], int(B))
@@ -188,7 +232,10 @@ class _Pool2d(torch.nn.Module):
 class SNN_maxpool2d(_Pool2d):
     """Earliest-spike pooling: pad with 1e5, then -maxpool(-x), VALID (SNN_TC_Modules.py:215-246)."""
 
-    def forward(self, input):
+    def forward(self, input, feed=None):
+        """feed: the SNN_conv that follows; its padded input buffer receives the pooled times as well."""
+        if feed is not None and not (input.is_cuda and input.dtype == torch.float32 and input.dim() == 4):
+            raise ValueError("chaining needs float32 device tensors")
         if input.is_cuda and input.dtype == torch.float32 and input.dim() == 4:
             # one kernel each way: the padding is implicit and the minimum is taken directly
             H, W = input.shape[1], input.shape[2]
@@ -200,8 +247,11 @@ class SNN_maxpool2d(_Pool2d):
                     raise ValueError("negative SAME padding: kernel smaller than stride is not supported")
             nh = (H + top + bottom - self.Kh) // self.Sh + 1
             nw = (W + left + right - self.Kw) // self.Sw + 1
+            next_xpad, next_offset = None, (0, 0)
+            if feed is not None:
+                next_xpad, next_offset = feed.padded_input_buffer(input.shape[0], nh, nw, input.device)
             return SnnMinPool.apply(input.contiguous(), (self.Kh, self.Kw), (self.Sh, self.Sw), (top, left), (nh, nw),
-                                    float(self.padvalue))
+                                    float(self.padvalue), next_xpad, next_offset)
         x = self._padded_nchw(input)                         # host tensors: the reference's formula itself
         y = -F.max_pool2d(-x, (self.Kh, self.Kw), (self.Sh, self.Sw))
         return y.permute(0, 2, 3, 1)

@@ -63,22 +63,46 @@ def draw_weights(spec, rng):
 
 
 class SnnSequential(torch.nn.Sequential):
-    """The layers of a spec in order.  forward(x, keep=list) appends every layer's input to `keep`."""
+    """The layers of a spec in order.  forward(x, keep=list) appends every layer's input to `keep`.
+
+    chain=True removes the padding pass between a conv or pooling layer and the SAME-padded conv layer
+    that follows it: the first writes its spike times into the second's padded input buffer as well (a
+    buffer the second layer keeps, its border filled once), and the second reads from there.  Results
+    are the same bit for bit.  The buffers hold the latest forward pass only: run backward before the
+    next forward, as a training loop does."""
+
+    def __init__(self, *mods, chain=False):
+        super().__init__(*mods)
+        self.chain = chain
 
     def forward(self, x, keep=None):
-        for layer in self:
+        layers = list(self)
+        prefilled = False
+        for i, layer in enumerate(layers):
             if keep is not None:
                 keep.append(x)
-            x = layer(x)
+            nxt = layers[i + 1] if i + 1 < len(layers) else None
+            feed = None
+            if (self.chain and x.is_cuda and isinstance(nxt, L.SNN_conv) and nxt.padding == 'SAME'
+                    and isinstance(layer, (L.SNN_conv, L.SNN_maxpool2d))
+                    and not (isinstance(layer, L.SNN_conv) and layer.padding != 'SAME')):
+                feed = nxt
+            if isinstance(layer, L.SNN_conv) and (prefilled or feed is not None):
+                x = layer(x, prefilled=prefilled, feed=feed)
+            elif isinstance(layer, L.SNN_maxpool2d) and feed is not None:
+                x = layer(x, feed=feed)
+            else:
+                x = layer(x)
+            prefilled = feed is not None
         return x
 
     def weights(self):
         return [l.weight for l in self if hasattr(l, "weight")]
 
 
-def build(spec, weights=None, rng=None):
+def build(spec, weights=None, rng=None, chain=False):
     """SnnSequential for `spec`.  `weights`: one numpy array per weighted layer; drawn from
-    baseline_weight with `rng` when omitted."""
+    baseline_weight with `rng` when omitted.  chain: see SnnSequential."""
     if weights is None:
         weights = draw_weights(spec, rng if rng is not None else np.random.default_rng(0))
     weights = list(weights)
@@ -100,7 +124,7 @@ def build(spec, weights=None, rng=None):
             raise ValueError(f"unknown layer kind {kind!r}")
     if weights:
         raise ValueError("more weight arrays than weighted layers")
-    return SnnSequential(*mods)
+    return SnnSequential(*mods, chain=chain)
 
 
 def forward_backward(net, z, onehot):

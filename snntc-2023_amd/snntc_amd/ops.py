@@ -165,9 +165,11 @@ def snncv_output_dims(H, W, Params):
     return nh.value, nw.value
 
 
-def snncv(X, W, Params, return_aux=False):
+def snncv(X, W, Params, return_aux=False, next_xpad=None, next_offset=(0, 0)):
     """Conv forward on the already padded / cropped NHWC input X[B,H,W,C]; W[Kh*Kw*C+bias,Kc]
-    -> Y[2B,Nh,Nw,Kc].  With return_aux=True also returns per-patch (sorted_z, perm, causal_k)."""
+    -> Y[2B,Nh,Nw,Kc].  With return_aux=True also returns per-patch (sorted_z, perm, causal_k).
+    next_xpad[B,h,w,Kc], if given, also receives the spike times, output pixel (nh, nw) at its pixel
+    (nh + next_offset[0], nw + next_offset[1]): the padded input of the conv layer that follows."""
     lib = _lib.load()
     X = _dev_f32(X, "X", 4)
     W = _dev_f32(W, "W", 2)
@@ -188,13 +190,24 @@ def snncv(X, W, Params, return_aux=False):
             _lib.check(lib.snntc_cv_forward_ex(_ptr(X), _ptr(W), pp, _ptr(out), _ptr(sz), _ptr(perm), _ptr(ck),
                                                B, H, Wd, C, Kc, w_rows, _ptr(ws), ws.numel(), _stream(X.device)))
             return out, sz, perm, ck
+        if next_xpad is not None:
+            nx = _dev_f32(next_xpad, "next_xpad", 4)
+            if nx.shape[0] != B or nx.shape[3] != Kc:
+                raise ValueError(f"next_xpad {tuple(nx.shape)} does not match batch {B} / channels {Kc}")
+            _lib.check(lib.snntc_cv_forward_chained(_ptr(X), _ptr(W), pp, _ptr(out), _ptr(nx), nx.shape[1], nx.shape[2],
+                                                    next_offset[0], next_offset[1], B, H, Wd, C, Kc, w_rows, _ptr(ws),
+                                                    ws.numel(), _stream(X.device)))
+            return out
         _lib.check(lib.snntc_cv_forward(_ptr(X), _ptr(W), pp, _ptr(out), B, H, Wd, C, Kc, w_rows, _ptr(ws),
                                         ws.numel(), _stream(X.device)))
     return out
 
 
-def snncv_grad(grad, X, W, Params, Y, want_dparams=True, want_dx=True, want_dw=True, first_half_grad=False):
-    """Conv backward -> (dXpad like X, dW like W, dParams[12] of zeros, or None if not wanted)."""
+def snncv_grad(grad, X, W, Params, Y, want_dparams=True, want_dx=True, want_dw=True, first_half_grad=False,
+               crop=None):
+    """Conv backward -> (dXpad like X, dW like W, dParams[12] of zeros, or None if not wanted).
+    crop = (h, w, top, left): dX is only that window of the padded input's gradient, [B,h,w,C] (the
+    gradient with respect to the image before its SAME padding)."""
     lib = _lib.load()
     grad = _dev_f32(grad, "grad", 4)
     X = _dev_f32(X, "X", 4)
@@ -210,13 +223,19 @@ def snncv_grad(grad, X, W, Params, Y, want_dparams=True, want_dx=True, want_dw=T
         need = ctypes.c_size_t()
         _lib.check(lib.snntc_cv_backward_workspace_bytes(B, H, Wd, C, Kc, pp, ctypes.byref(need)))
         ws = _workspace(X.device, need.value)
-        dX = torch.empty_like(X) if want_dx else None
         dW = torch.empty_like(W) if want_dw else None
         dP = torch.empty(12, dtype=torch.float32, device=X.device) if want_dparams else None
+        grad_rows = 2 * B if (first_half_grad and grad.shape[0] == B) else grad.shape[0]
+        if crop is not None:
+            ch, cw, ctop, cleft = crop
+            dX = torch.empty((B, ch, cw, C), dtype=torch.float32, device=X.device) if want_dx else None
+            _lib.check(lib.snntc_cv_backward_cropped(_ptr(grad), _ptr(X), _ptr(W), pp, _ptr(Y), _ptr(dX), ch, cw, ctop,
+                                                     cleft, _ptr(dW), _ptr(dP), B, H, Wd, C, Kc, w_rows, grad_rows,
+                                                     _ptr(ws), ws.numel(), _stream(X.device)))
+            return dX, dW, dP
+        dX = torch.empty_like(X) if want_dx else None
         _lib.check(lib.snntc_cv_backward(_ptr(grad), _ptr(X), _ptr(W), pp, _ptr(Y), _ptr(dX), _ptr(dW), _ptr(dP),
-                                         B, H, Wd, C, Kc, w_rows,
-                                         2 * B if (first_half_grad and grad.shape[0] == B) else grad.shape[0],
-                                         _ptr(ws), ws.numel(), _stream(X.device)))
+                                         B, H, Wd, C, Kc, w_rows, grad_rows, _ptr(ws), ws.numel(), _stream(X.device)))
     return dX, dW, dP
 
 
@@ -297,6 +316,39 @@ class SnnCvTimes(torch.autograd.Function):
         return dX, dW, None
 
 
+class SnnCvSame(torch.autograd.Function):
+    """SNN_conv with SAME padding as one differentiable step on the un-padded image x[B,H,W,C]: pad with
+    MAX_SPIKE_TIME, snncv, and in the backward pass the gradient with respect to x itself (the op stores
+    only that window of the padded gradient, so no separate crop runs).
+      xpad      None: the padded tensor is made here (one pass).  Otherwise the layer's padded input
+                buffer, already holding x in its interior (written there by the layer before, see
+                next_xpad) and MAX_SPIKE_TIME on its border.
+      next_xpad None, or the padded input buffer of the conv layer that follows: the spike times are
+                written there as well, at pixel offset next_offset."""
+
+    @staticmethod
+    def forward(ctx, x, W, Params, pads, xpad, next_xpad, next_offset):
+        top, bottom, left, right = pads
+        B, H, Wd, C = x.shape
+        if xpad is None:
+            xpad = pad_time(x, top, bottom, left, right, float(Params[0])) if (top or bottom or left or right) else x
+        elif tuple(xpad.shape) != (B, top + H + bottom, left + Wd + right, C):
+            raise ValueError(f"padded buffer {tuple(xpad.shape)} does not match input {tuple(x.shape)} and pads {pads}")
+        Y = snncv(xpad, W, Params, next_xpad=next_xpad, next_offset=next_offset)
+        ctx.save_for_backward(xpad, W, Y)
+        ctx.params = np.array(Params, dtype=np.float32, copy=True)
+        ctx.crop = (H, Wd, top, left)
+        return Y[:B]
+
+    @staticmethod
+    def backward(ctx, grad):
+        X, W, Y = ctx.saved_tensors
+        dX, dW, _ = snncv_grad(grad.contiguous(), X, W, ctx.params, Y, want_dparams=False,
+                               want_dx=ctx.needs_input_grad[0], want_dw=ctx.needs_input_grad[1],
+                               first_half_grad=True, crop=ctx.crop)
+        return dX, dW, None, None, None, None, None
+
+
 def softmax_time_loss(times, label, want_loss=True, want_grad=True):
     """Per-sample cross-entropy of label[B,J] against softmax(-times[B,J]) and the gradient of its batch
     mean with respect to times, in one kernel (loss_func, SNN_TC_Modules.py:286-288).
@@ -361,16 +413,27 @@ class SoftmaxTimeLoss(torch.autograd.Function):
         return grad * upstream, None
 
 
-def min_pool(x, kernel, stride, pad, out_hw, pad_value=1e5, want_arg=True):
+def min_pool(x, kernel, stride, pad, out_hw, pad_value=1e5, want_arg=True, next_xpad=None, next_offset=(0, 0)):
     """Earliest-spike pooling of NHWC spike times x[B,H,W,C] -> (y[B,Nh,Nw,C], arg or None).
     kernel = (Kh, Kw), stride = (Sh, Sw), pad = (top, left), out_hw = (Nh, Nw); pixels outside the
-    image count as pad_value.  arg records, per output, the window position that attained the minimum."""
+    image count as pad_value.  arg records, per output, the window position that attained the minimum.
+    next_xpad[B,h,w,C], if given, also receives y at pixel offset next_offset (the padded input of the
+    conv layer that follows)."""
     lib = _lib.load()
     x = _dev_f32(x, "x", 4)
     B, H, W, C = x.shape
     with torch.cuda.device(x.device):
         y = torch.empty((B, out_hw[0], out_hw[1], C), dtype=torch.float32, device=x.device)
         arg = torch.empty(y.shape, dtype=torch.int32, device=x.device) if want_arg else None
+        if next_xpad is not None:
+            nx = _dev_f32(next_xpad, "next_xpad", 4)
+            if nx.shape[0] != B or nx.shape[3] != C:
+                raise ValueError(f"next_xpad {tuple(nx.shape)} does not match batch {B} / channels {C}")
+            _lib.check(lib.snntc_min_pool_forward_chained(_ptr(x), _ptr(y), _ptr(arg), _ptr(nx), nx.shape[1], nx.shape[2],
+                                                          next_offset[0], next_offset[1], B, H, W, C, kernel[0],
+                                                          kernel[1], stride[0], stride[1], pad[0], pad[1], out_hw[0],
+                                                          out_hw[1], float(pad_value), _stream(x.device)))
+            return y, arg
         _lib.check(lib.snntc_min_pool_forward(_ptr(x), _ptr(y), _ptr(arg), B, H, W, C, kernel[0], kernel[1], stride[0],
                                               stride[1], pad[0], pad[1], out_hw[0], out_hw[1], float(pad_value),
                                               _stream(x.device)))
@@ -398,8 +461,9 @@ class SnnMinPool(torch.autograd.Function):
     position that attained it."""
 
     @staticmethod
-    def forward(ctx, x, kernel, stride, pad, out_hw, pad_value):
-        y, arg = min_pool(x, kernel, stride, pad, out_hw, pad_value, want_arg=x.requires_grad)
+    def forward(ctx, x, kernel, stride, pad, out_hw, pad_value, next_xpad=None, next_offset=(0, 0)):
+        y, arg = min_pool(x, kernel, stride, pad, out_hw, pad_value, want_arg=x.requires_grad, next_xpad=next_xpad,
+                          next_offset=next_offset)
         ctx.geom = (tuple(x.shape), tuple(kernel), tuple(stride), tuple(pad))
         if arg is not None:
             ctx.save_for_backward(arg)
@@ -409,10 +473,10 @@ class SnnMinPool(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_y):
         if not ctx.has_arg:
-            return (None,) * 6
+            return (None,) * 8
         (arg,) = ctx.saved_tensors
         in_shape, kernel, stride, pad = ctx.geom
-        return (min_pool_grad(grad_y.contiguous(), arg, in_shape, kernel, stride, pad),) + (None,) * 5
+        return (min_pool_grad(grad_y.contiguous(), arg, in_shape, kernel, stride, pad),) + (None,) * 7
 
 
 def pad_time(x, top, bottom, left, right, value):

@@ -152,3 +152,26 @@ def test_sgd_update_argument_errors(lib):
     assert lib.snntc_sgd_update(one, null_in, n, 2, 0.1, None) == 3
     assert lib.snntc_sgd_update(None, None, None, 0, 0.1, None) == 0            # no tensors: nothing to do
     assert lib.snntc_sgd_update(null_in, null_in, (i64 * 2)(0, 0), 2, 0.1, None) == 0   # empty tensors are skipped
+
+
+def test_chained_entry_points_check_their_windows(lib):
+    from snntc_amd import _lib
+    p = np.array([1e5, 0, 0, 1e-10, 1, 0, 3, 3, 1, 1, 1, 1.0], np.float32)      # 3x3, stride 1, SAME, bias
+    # 6x6 padded input -> 4x4 output; a 5x5 destination at offset (1, 1) holds it, (2, 2) does not
+    args = (2, 6, 6, 8, 16, 73, FAKE, 1 << 30, None)
+    assert lib.snntc_cv_forward_chained(FAKE, FAKE, _fp(p), FAKE, None, 5, 5, 1, 1, *args) == _lib.ERR_BAD_ARGUMENT
+    assert lib.snntc_cv_forward_chained(FAKE, FAKE, _fp(p), FAKE, FAKE, 5, 5, 2, 2, *args) == _lib.ERR_BAD_ARGUMENT
+    assert b"does not fit" in lib.snntc_last_error()
+    assert lib.snntc_cv_forward_chained(FAKE, FAKE, _fp(p), FAKE, FAKE, 5, 5, -1, 0, *args) == _lib.ERR_BAD_ARGUMENT
+    # the gradient window has to lie inside the 6x6 padded image
+    bargs = (FAKE, FAKE, 2, 6, 6, 8, 16, 73, 4, FAKE, 1 << 30, None)
+    assert lib.snntc_cv_backward_cropped(FAKE, FAKE, FAKE, _fp(p), FAKE, FAKE, 4, 4, 3, 1, *bargs) == _lib.ERR_BAD_ARGUMENT
+    assert b"does not lie inside" in lib.snntc_last_error()
+    assert lib.snntc_cv_backward_cropped(FAKE, FAKE, FAKE, _fp(p), FAKE, FAKE, 4, 7, 0, 0, *bargs) == _lib.ERR_BAD_ARGUMENT
+    # a window that fits passes on to the op's own checks (here: grad rows must be 2 * batch)
+    bad_rows = (FAKE, FAKE, 2, 6, 6, 8, 16, 73, 3, FAKE, 1 << 30, None)
+    assert lib.snntc_cv_backward_cropped(FAKE, FAKE, FAKE, _fp(p), FAKE, FAKE, 4, 4, 1, 1, *bad_rows) == _lib.ERR_DIM_MISMATCH
+    # pooling: 4x4 image, 2x2/2 windows -> 2x2 output, which a 3x3 destination holds at (1, 1) only
+    pool = (2, 4, 4, 8, 2, 2, 2, 2, 0, 0, 2, 2, ctypes.c_float(1e5), None)
+    assert lib.snntc_min_pool_forward_chained(FAKE, FAKE, None, None, 3, 3, 1, 1, *pool) == _lib.ERR_BAD_ARGUMENT
+    assert lib.snntc_min_pool_forward_chained(FAKE, FAKE, None, FAKE, 3, 3, 2, 1, *pool) == _lib.ERR_BAD_ARGUMENT
