@@ -29,7 +29,7 @@
  * finite differences of a float64 forward.  Tie order inside the reference's GPU sort is
  * implementation-defined in the reference itself and therefore "parity unpinned".
  *
- * Build: see oracle/Makefile (gcc -O2 -ffp-contract=off -mfma).
+ * Build: see oracle/Makefile (gcc -O3 -ffp-contract=off -mfma).
  */
 #include <math.h>
 #include <stdint.h>
