@@ -135,9 +135,9 @@ def git_commit():
     return r.stdout.strip() or "unknown"
 
 
-def summarise(workloads, raw, out):
+def summarise(workloads, raw, out, commit=None):
     os.makedirs(out, exist_ok=True)
-    table = {"commit": git_commit(),
+    table = {"commit": commit or git_commit(),
              "note": "rocprofv3 --pmc readings per launch, averaged over the launches of a kernel in one step of the "
                      "workload (scan instantiations that also write causal-set sizes excluded: they belong to the "
                      "accounting forward): hbm_bytes_per_launch = FETCH_SIZE * f + WRITE_SIZE * g KiB with the "
@@ -237,10 +237,11 @@ def main():
     ap.add_argument("--raw", default=os.path.join(ROOT, "gpurun_out", "profiles_raw"))
     ap.add_argument("--out", default=os.path.join(ROOT, "profiles"))
     ap.add_argument("--keep-raw", action="store_true", help="keep the rocprofv3 databases after summarising")
+    ap.add_argument("--commit", default=None, help="commit the measured tree is at (default: git rev-parse HEAD here)")
     args = ap.parse_args()
     if args.action == "collect":
         collect(args.workloads, args.raw)
-    summarise(args.workloads, args.raw, args.out)
+    summarise(args.workloads, args.raw, args.out, args.commit)
     if args.action == "collect" and not args.keep_raw:
         for w in args.workloads:
             for tag in ("trace", "FETCH_SIZE", "WRITE_SIZE", "valu"):
