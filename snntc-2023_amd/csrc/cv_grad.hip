@@ -66,23 +66,31 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KCB ==
 cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restrict__ wq,
                           const float* __restrict__ upm, const float* __restrict__ ym,
                           float* __restrict__ dx, CropGeom crop, int H, int W, int C, int Kc, int Kh, int Kw, int Sh,
-                          int Sw, int Nh, int Nw, int tiles_w, int c_blocks, int64_t n_items, float max_cmp,
-                          int ksplit) {
-    extern __shared__ __align__(16) float staged[];                    // per wavefront: [2][n_slots + 1][KCB]
-    __shared__ float partial[3][DX_TILE][kWave];         // ksplit = 4: sums of wavefronts 1..3
+                          int Sw, int Nh, int Nw, int tiles_w, int c_blocks, int64_t n_items, int64_t lead_items,
+                          int lead_blocks, float max_cmp, int ksplit) {
+    extern __shared__ __align__(16) float staged[];      // per wavefront: [2][n_slots + 1][KCB]; ksplit = 4: then `partial`
     constexpr int SPAN = DX_TILE * HALVES;               // pixels of one wavefront
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    // ksplit = 1: a tile per wavefront.  ksplit = 4 (layers with few tiles and many output channels):
-    // a tile per workgroup, its wavefronts take a quarter of the output channels each and their
-    // sums are added in wavefront order.
-    const int64_t item = ksplit == 1 ? (int64_t)blockIdx.x * (blockDim.x / kWave) + wave : (int64_t)blockIdx.x;
-    const int ks = ksplit == 1 ? 0 : wave;
-    if (item >= n_items) return;
+    // ksplit = 1: a tile per single-wavefront workgroup.  ksplit = 4 (layers with few tiles and many
+    // output channels): a tile per workgroup of four, its wavefronts take a quarter of the output
+    // channels each and their sums are added in wavefront order.
+    // Items are (image, row, tile, channel block).  When the last tile of a row is a partial one, those
+    // tiles form a second run of workgroups behind all others (`lead_blocks` workgroups, a multiple of
+    // the XCD count, hold the `lead_items` others), so that the launch ends on its shortest items and
+    // the CUs drain together.  Both runs are numbered XCD-contiguously: an XCD works on the same
+    // rows in both, and on neighbouring tiles, which share their staged rows, one after another.
+    const bool lead = (int)blockIdx.x < lead_blocks;
+    const int64_t item = lead ? xcd_contiguous(blockIdx.x, lead_blocks)
+                              : xcd_contiguous(blockIdx.x - lead_blocks, gridDim.x - lead_blocks);
+    const int ks = wave;                                 // 0 without the split
+    if (item >= (lead ? lead_items : n_items - lead_items)) return;
     const int lane = threadIdx.x % kWave;
     const int half = HALVES == 2 ? lane / 32 : 0;
+    const int tiles_lead = lead_items < n_items ? tiles_w - 1 : tiles_w;
     const int cb = (int)(item % c_blocks);
     int64_t rest = item / c_blocks;
-    const int tw = (int)(rest % tiles_w); rest /= tiles_w;
+    int tw = tiles_w - 1;
+    if (lead) { tw = (int)(rest % tiles_lead); rest /= tiles_lead; }
     const int h = (int)(rest % H);
     const int a = (int)(rest / H);
     const int w0 = tw * SPAN;                            // first pixel of the wavefront
@@ -207,15 +215,18 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
         }
     }
     if (ksplit > 1) {                                     // block-uniform: all four wavefronts hold the same tile
+        // sums of wavefronts 1..3, [3][DX_TILE][64], behind the staging areas
+        float* __restrict__ partial = staged + (size_t)(blockDim.x / kWave) * 2 * (n_slots + 1) * KCB;
         if (ks > 0) {
 #pragma unroll
-            for (int t = 0; t < DX_TILE; ++t) partial[ks - 1][t][lane] = acc[t];
+            for (int t = 0; t < DX_TILE; ++t) partial[((ks - 1) * DX_TILE + t) * kWave + lane] = acc[t];
         }
         __syncthreads();
         if (ks > 0) return;
 #pragma unroll
         for (int t = 0; t < DX_TILE; ++t)
-            acc[t] = ((acc[t] + partial[0][t][lane]) + partial[1][t][lane]) + partial[2][t][lane];
+            acc[t] = ((acc[t] + partial[t * kWave + lane]) + partial[(DX_TILE + t) * kWave + lane]) +
+                     partial[(2 * DX_TILE + t) * kWave + lane];
     }
     // only the pixels inside the caller's window of the padded image are stored
     if (lane_ok) {
@@ -454,12 +465,23 @@ int launch_cv_grad_input_chan(const float* xpad, const float* wq, const float* u
     // wavefronts of a workgroup.  Decided by the layer's geometry alone, never by the batch: the
     // order of the additions, and with it the last bits of dX, must not depend on the batch size.
     const int ksplit = (halves == 1 && g.H * tiles_w * c_blocks <= 160 && g.Kc % (4 * kcb) == 0) ? 4 : 1;
-    const int64_t blocks = ksplit == 4 ? n_items : (n_items + 3) / 4;
+    // One item per workgroup.  Without the split a workgroup is a single wavefront: the
+    // wavefronts do not cooperate, their running times differ (border tiles, rows outside the window),
+    // and a CU takes a new workgroup only when a whole one has left, so in larger workgroups the slots
+    // of the early finishers would idle.
+    const int wg_waves = ksplit == 4 ? 4 : 1;
+    // a last tile with at most half its pixels inside the row goes to the end of the launch
+    const bool partial_last = tiles_w > 1 && (g.W - (int64_t)(tiles_w - 1) * span) * 2 <= span;
+    const int64_t lead_items = partial_last ? g.B * g.H * (tiles_w - 1) * c_blocks : n_items;
+    int64_t lead_blocks = lead_items;
+    if (partial_last) lead_blocks = (lead_blocks + kXcds - 1) / kXcds * kXcds;
+    const int64_t blocks = lead_blocks + (n_items - lead_items);
     if (blocks > 0x7fffffffLL) return fail(SNNTC_ERR_TOO_LARGE, "conv backward: grid too large");
-    dim3 grid((unsigned)blocks), block(256);
-    const size_t lds = (size_t)4 * 2 * (span + g.Kw) * kcb * sizeof(float);
+    dim3 grid((unsigned)blocks), block(wg_waves * kWave);
+    const size_t lds = (size_t)wg_waves * 2 * (span + g.Kw) * kcb * sizeof(float) +
+                       (ksplit == 4 ? (size_t)3 * DX_TILE * kWave * sizeof(float) : 0);
     void (*kern)(const float*, const float*, const float*, const float*, float*, CropGeom, int, int, int, int, int, int,
-                 int, int, int, int, int, int, int64_t, float, int);
+                 int, int, int, int, int, int, int64_t, int64_t, int, float, int);
     if (halves == 2)
         kern = kcb == 64 ? cv_grad_input_chan_kernel<64, 2> : kcb == 32 ? cv_grad_input_chan_kernel<32, 2>
                                                                          : cv_grad_input_chan_kernel<16, 2>;
@@ -470,7 +492,7 @@ int launch_cv_grad_input_chan(const float* xpad, const float* wq, const float* u
         KernelTimerScope timer_("cv_grad_input", stream);
         hipLaunchKernelGGL(kern, grid, block, lds, stream, xpad, wq, upm, ym, dx, crop, (int)g.H, (int)g.W, (int)g.C,
                            (int)g.Kc, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.Nh, (int)g.Nw, tiles_w,
-                           c_blocks, n_items, np.max_cmp, ksplit);
+                           c_blocks, n_items, lead_items, (int)lead_blocks, np.max_cmp, ksplit);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;

@@ -964,6 +964,7 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
 
                 for (int k0 = kmin;; k0 += RING * CHUNK) {
                     bool stop = false;
+                    rotate_wave_priority(k0 / (RING * CHUNK) + (wave >> 2));
 #pragma unroll
                     for (int ph = 0; ph < RING; ++ph) {
                         const int k = k0 + ph * CHUNK;

@@ -39,6 +39,23 @@ __device__ __forceinline__ int xcd_contiguous(int block, int total) {
     return xcd * per + (xcd < extra ? xcd : extra) + local;
 }
 
+// The instruction arbiter of a SIMD prefers its oldest wavefront.  Wavefronts that start together
+// on long loops of equal length therefore do not advance together: the oldest runs at the pace of a
+// lone wavefront, the youngest crawls, and once the older ones are gone the SIMD is left with one
+// or two wavefronts that cannot fill it.  rotate_wave_priority(turn) gives the wavefronts of a SIMD
+// the top priority in turns: called with a wave-uniform counter that advances at the same pace in
+// all of them (a loop iteration count) plus a number that differs between the wavefronts of a SIMD
+// (wavefronts of a workgroup go to the four SIMDs round-robin, so index / 4 does), it keeps their
+// progress level, and they finish together.  s_setprio takes its level as an immediate.
+__device__ __forceinline__ void rotate_wave_priority(int turn) {
+    switch (turn & 3) {
+        case 0: __builtin_amdgcn_s_setprio(0); break;
+        case 1: __builtin_amdgcn_s_setprio(1); break;
+        case 2: __builtin_amdgcn_s_setprio(2); break;
+        default: __builtin_amdgcn_s_setprio(3); break;
+    }
+}
+
 // Opt-in per-kernel timing (snntc_profile_*): while enabled, every launcher brackets its kernel
 // with a pair of HIP events on the launch stream.  Disabled (the default) it costs one branch.
 struct KernelTimerScope {
