@@ -145,7 +145,10 @@ constexpr int LDS_SCAN_THREADS = 1024;
 constexpr int LDS_SCAN_BYTES = 160 * 1024;
 // The widest slice that fits is taken: the register budget allows one 16-wave workgroup per CU anyway,
 // and fewer slices re-read the sorted rows less often.
-constexpr int LDS_SCAN_TARGET = 160 * 1024 - 64;          // 64 bytes behind the slice for a reduction
+// Behind the slice: 64 bytes for a reduction and room for the chunk buffers of at least four
+// wavefronts (scan_filter_kernel: 64 bytes per segment of a wavefront, at most 8 segments).
+constexpr int FILTER_XBUF_SEG_BYTES = 2 * CHUNK * (int)sizeof(float);
+constexpr int LDS_SCAN_TARGET = 160 * 1024 - 64 - 4 * 8 * FILTER_XBUF_SEG_BYTES;
 
 struct Chunk {
     float x[CHUNK];
@@ -820,6 +823,16 @@ __device__ __forceinline__ void quad_row_addresses(int row, unsigned base, unsig
 
 typedef __attribute__((address_space(3))) const float lds_cfloat;
 
+// Segments a wavefront of the filter kernel works on, and whether their input times go through
+// LDS: they do unless every quad has a segment of its own (then the quad broadcast is all there is
+// to share, and the buffers of 16 segments per wavefront would not fit beside the slice).
+constexpr int filter_segments(int cols, int ch) { return kWave / (cols / ch); }
+constexpr bool filter_stages_times(int cols, int ch) { return filter_segments(cols, ch) <= 8; }
+// dynamic LDS of a workgroup of `waves` wavefronts behind its slice
+constexpr size_t filter_extra_lds(int cols, int ch, int waves) {
+    return FILTER_RED_BYTES + (filter_stages_times(cols, ch) ? (size_t)waves * filter_segments(cols, ch) * FILTER_XBUF_SEG_BYTES : 0);
+}
+
 template <int COLS, int CH, bool WANT_K>
 __global__ void __launch_bounds__(LDS_SCAN_THREADS)
 scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
@@ -830,6 +843,8 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
     constexpr int LANES = COLS / CH;                       // lanes per segment
     constexpr int SEGS = kWave / LANES;                    // segments per wavefront
     static_assert(LANES % 4 == 0, "the four lanes of a quad belong to one segment");
+    // Input times reach the lanes through LDS where several quads share a segment (see the fast loop)
+    constexpr bool XLDS = filter_stages_times(COLS, CH);
     const int WAVES = blockDim.x / kWave;
     const int block = xcd_contiguous(blockIdx.x, gridDim.x);
     const int slice = block / n_groups;
@@ -849,6 +864,10 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
 
     const int quad_lane = lane & 3;
     const unsigned wbase = (unsigned)(uintptr_t)(lds_cfloat*)wcol;          // LDS byte address of the lane's columns
+    // [wave][buffer][segment of the wavefront][CHUNK] input times, behind the slice and `red`
+    float* __restrict__ xbuf = wl + rows * COLS + FILTER_RED_BYTES / (int)sizeof(float) +
+                               (size_t)wave * 2 * SEGS * CHUNK + sub * CHUNK;
+    const bool x_writer = cg < 4;                          // the first quad of every segment
     constexpr int NONE = 0x7fffffff;
     constexpr int ROW_SHIFT = COLS == 64 ? 8 : COLS == 32 ? 7 : COLS == 16 ? 6 : 5;      // a weight row is COLS * 4 bytes
     static_assert(COLS == 64 || COLS == 32 || COLS == 16 || COLS == 8, "slice width");
@@ -958,9 +977,30 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
                         for (int c = 0; c < CH; ++c) wo[c][u] = wr[c];
                     }
                 };
+                // Input times: with DPP alone every lane needs a move per time and chunk.  Where a
+                // segment spans several quads, its first quad instead leaves the eight times of the
+                // next chunk in a small LDS buffer of the wavefront (two chunks deep) and every lane
+                // reads them back as two 16-byte broadcasts, a phase ahead like the weights.  LDS
+                // serves the requests of a wavefront in order, so the reads find what was written.
+                float xq[2][CHUNK];
+                auto stage_times = [&](int slot, int buf) {
+                    if constexpr (XLDS) {
+                        float* __restrict__ xb = xbuf + buf * SEGS * CHUNK;
+                        if (x_writer) {
+                            xb[quad_lane] = rxl[slot];
+                            xb[quad_lane + 4] = rxh[slot];
+                        }
+                        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                        __builtin_amdgcn_wave_barrier();
+                        const float4 lo = *reinterpret_cast<const float4*>(xb), hi = *reinterpret_cast<const float4*>(xb + 4);
+                        xq[buf][0] = lo.x; xq[buf][1] = lo.y; xq[buf][2] = lo.z; xq[buf][3] = lo.w;
+                        xq[buf][4] = hi.x; xq[buf][5] = hi.y; xq[buf][6] = hi.z; xq[buf][7] = hi.w;
+                    }
+                };
 #pragma unroll
                 for (int b = 0; b < RING - 1; ++b) request(b, kmin + b * CHUNK);
                 weights(0, wv[0]);
+                stage_times(0, 0);
 
                 for (int k0 = kmin;; k0 += RING * CHUNK) {
                     bool stop = false;
@@ -978,16 +1018,22 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
                         if (any == 0) { stop = true; break; }
                         request((ph + RING - 1) % RING, k + (RING - 1) * CHUNK);
                         weights((ph + 1) % RING, wv[(ph + 1) % 2]);
+                        stage_times((ph + 1) % RING, (ph + 1) % 2);
                         // The requests above stay ahead of the arithmetic below: what this phase consumes
                         // was requested a phase or more ago, and what it requests has the whole phase to
                         // arrive.
                         __builtin_amdgcn_sched_barrier(0);
-                        const int xl = __float_as_int(rxl[ph % RING]), xh = __float_as_int(rxh[ph % RING]);
-                        const float x[CHUNK] = {
-                            __int_as_float(quad_broadcast<0>(xl)), __int_as_float(quad_broadcast<1>(xl)),
-                            __int_as_float(quad_broadcast<2>(xl)), __int_as_float(quad_broadcast<3>(xl)),
-                            __int_as_float(quad_broadcast<0>(xh)), __int_as_float(quad_broadcast<1>(xh)),
-                            __int_as_float(quad_broadcast<2>(xh)), __int_as_float(quad_broadcast<3>(xh))};
+                        float x[CHUNK];
+                        if constexpr (XLDS) {
+#pragma unroll
+                            for (int u = 0; u < CHUNK; ++u) x[u] = xq[ph % 2][u];
+                        } else {
+                            const int xl = __float_as_int(rxl[ph % RING]), xh = __float_as_int(rxh[ph % RING]);
+                            x[0] = __int_as_float(quad_broadcast<0>(xl)); x[1] = __int_as_float(quad_broadcast<1>(xl));
+                            x[2] = __int_as_float(quad_broadcast<2>(xl)); x[3] = __int_as_float(quad_broadcast<3>(xl));
+                            x[4] = __int_as_float(quad_broadcast<0>(xh)); x[5] = __int_as_float(quad_broadcast<1>(xh));
+                            x[6] = __int_as_float(quad_broadcast<2>(xh)); x[7] = __int_as_float(quad_broadcast<3>(xh));
+                        }
                         const float thrx = x[CHUNK - 1] * thr_w;
 #pragma unroll
                         for (int c = 0; c < CH; ++c)
@@ -1154,7 +1200,7 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     const int n_slices = (int)((J + COLS - 1) / COLS);
     const int64_t items = (S + SEGS - 1) / SEGS;
     // workgroups the chip holds at once (two per CU when two weight slices fit in its LDS)
-    const int wgs_per_cu = (lds_bytes + FILTER_RED_BYTES) * 2 <= (size_t)LDS_SCAN_BYTES ? 2 : 1;
+    const int wgs_per_cu = (lds_bytes + filter_extra_lds(COLS, 1, 16)) * 2 <= (size_t)LDS_SCAN_BYTES ? 2 : 1;
     const int64_t capacity = (int64_t)cus * wgs_per_cu;
     // A launch whose work items all find a wavefront of their own in workgroups of four (one
     // wavefront per SIMD of a CU, and four times the threads of a single wavefront for copying the
@@ -1183,12 +1229,17 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     const bool split = low_latency && items * n_slices <= (int64_t)cus && I >= 2 * CHUNK * SPLIT_WAVES &&
                        split_lds + SPLIT_STATIC_LDS <= (size_t)LDS_SCAN_BYTES;
     if (split) WAVES = 1;                                   // items per workgroup pass
+    const bool filt = !(split || low_latency);
+    if (filt) {
+        // the chunk buffers of the wavefronts share the LDS with the slice: fewer wavefronts where it is tight
+        // (LDS_SCAN_TARGET leaves room for four)
+        while (WAVES > 4 && lds_bytes + filter_extra_lds(COLS, multi ? CH : 1, WAVES) > (size_t)LDS_SCAN_BYTES) WAVES -= 4;
+    }
     // split the segments so that slices x groups covers the chip without a second round of workgroups
     int64_t n_groups = capacity / n_slices;
     const int64_t max_groups = (work_items + WAVES - 1) / WAVES;
     if (n_groups > max_groups) n_groups = max_groups;
     if (n_groups < 1) n_groups = 1;
-    const bool filt = !(split || low_latency);
     auto kern_k = filt ? (multi ? scan_filter_kernel<COLS, CH, true> : scan_filter_kernel<COLS, 1, true>)
                   : split ? scan_lds_split_kernel<COLS, true> : scan_lds_kernel<COLS, true>;
     auto kern = filt ? (multi ? scan_filter_kernel<COLS, CH, false> : scan_filter_kernel<COLS, 1, false>)
@@ -1196,7 +1247,7 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     dim3 grid((unsigned)(n_slices * n_groups)), block((unsigned)((split && !filt) ? LOW_LATENCY_THREADS : WAVES * kWave));
     {
         KernelTimerScope timer_("scan", stream);
-        const size_t dyn_lds = filt ? lds_bytes + FILTER_RED_BYTES : split ? split_lds : lds_bytes;
+        const size_t dyn_lds = filt ? lds_bytes + filter_extra_lds(COLS, multi ? CH : 1, WAVES) : split ? split_lds : lds_bytes;
         if (causal_k)
             hipLaunchKernelGGL(kern_k, grid, block, dyn_lds, stream, sorted, perm, n_real, w, y, rcp, causal_k,
                                (int)S, (int)I, (int)stride, (int)J, n_slices, (int)n_groups, np, copy);
