@@ -63,7 +63,7 @@ enum {
     SNNTC_ERR_TOO_LARGE = 2,      /* a tensor (or the patch matrix) exceeds INT32_MAX elements  */
     SNNTC_ERR_BAD_ARGUMENT = 3,   /* null pointer, negative size, kernel larger than the image  */
     SNNTC_ERR_WORKSPACE = 4,      /* workspace missing, misaligned or too small                  */
-    SNNTC_ERR_UNSUPPORTED = 5,    /* segment longer than the largest supported sort (8192)       */
+    SNNTC_ERR_UNSUPPORTED = 5,    /* segment longer than the largest supported one (2^24 inputs) */
     SNNTC_ERR_HIP = 6             /* a HIP runtime call or kernel launch failed                  */
 };
 

@@ -124,15 +124,16 @@ int fc_check(int64_t B, int64_t I, int64_t J, int64_t w_rows, const float* param
     if (B * I > kInt32Max) return fail(SNNTC_ERR_TOO_LARGE, "%s: Too many elements in input tensor", who);
     if (w_rows * J > kInt32Max) return fail(SNNTC_ERR_TOO_LARGE, "%s: Too many elements in weight tensor", who);
     if (2 * B * J > kInt32Max) return fail(SNNTC_ERR_TOO_LARGE, "%s: Too many elements in output tensor", who);
-    if (I > kMaxSegment)
+    if (I > kMaxLongSegment)
         return fail(SNNTC_ERR_UNSUPPORTED, "%s: input size %lld exceeds the largest supported segment (%d)", who,
-                    (long long)I, kMaxSegment);
+                    (long long)I, kMaxLongSegment);
     return SNNTC_OK;
 }
 
 // Forward scratch.  n_pix / pix_c > 0 adds the per-pixel sorted channels the conv merge path needs.
 struct FcFwdWs {
     float* sorted; int32_t* perm; int32_t* n_real; float* pix_z; int32_t* pix_c;
+    void* long_keys;                                      // merge passes of segments longer than one network
     int64_t stride, pix_stride; size_t bytes;
 };
 FcFwdWs fc_fwd_ws(void* ws, int64_t S, int64_t I, int64_t n_pix = 0, int64_t pix_c = 0) {
@@ -145,6 +146,8 @@ FcFwdWs fc_fwd_ws(void* ws, int64_t S, int64_t I, int64_t n_pix = 0, int64_t pix
     r.n_real = c.take<int32_t>(S);
     r.pix_z = c.take<float>(n_pix * r.pix_stride);
     r.pix_c = c.take<int32_t>(n_pix * r.pix_stride);
+    const size_t long_bytes = sort_long_workspace_bytes(S, I);
+    r.long_keys = long_bytes ? c.take<unsigned char>((int64_t)long_bytes) : nullptr;
     r.bytes = c.used;
     return r;
 }
@@ -153,7 +156,7 @@ FcFwdWs fc_fwd_ws(void* ws, int64_t S, int64_t I, int64_t n_pix = 0, int64_t pix
 int forward_chain(const SegmentSource& src, const FcFwdWs& ws, const float* w, float* out, float* sorted_z,
                   int32_t* perm, int32_t* causal_k, int64_t S, int64_t I, int64_t J, const NeuronParams& np,
                   const TimeCopy& copy, hipStream_t st) {
-    int rc = launch_sort(src, S, ws.sorted, ws.perm, ws.n_real, (int)ws.stride, np.max_cmp, st);
+    int rc = launch_sort(src, S, ws.sorted, ws.perm, ws.n_real, (int)ws.stride, np.max_cmp, ws.long_keys, st);
     if (rc) return rc;
     rc = launch_unpad_rows(ws.sorted, ws.perm, sorted_z, perm, S, I, ws.stride, st);
     if (rc) return rc;
@@ -235,9 +238,9 @@ int cv_geom(int64_t B, int64_t H, int64_t W, int64_t C, int64_t Kc, int64_t w_ro
     if (w_rows * Kc > kInt32Max) return fail(SNNTC_ERR_TOO_LARGE, "%s: Too many elements in weight tensor", who);
     if (2 * g->S * Kc > kInt32Max) return fail(SNNTC_ERR_TOO_LARGE, "%s: Too many elements in output tensor", who);
     if (g->S * w_rows > kInt32Max) return fail(SNNTC_ERR_TOO_LARGE, "%s: Too many elements in patched tensor", who);
-    if (g->P > kMaxSegment)
+    if (g->P > kMaxLongSegment)
         return fail(SNNTC_ERR_UNSUPPORTED, "%s: patch length %lld exceeds the largest supported segment (%d)", who,
-                    (long long)g->P, kMaxSegment);
+                    (long long)g->P, kMaxLongSegment);
     return SNNTC_OK;
 }
 
@@ -282,7 +285,7 @@ int cv_forward_impl(const float* xpad, const float* w, const float* params, floa
     // sort every pixel's channels once, then assemble the patches by rank merging
     SegmentSource pixels{};
     pixels.base = xpad; pixels.conv = 0; pixels.I = (int)C;
-    rc = launch_sort(pixels, B * H * W, ws.pix_z, ws.pix_c, nullptr, (int)ws.pix_stride, np.max_cmp, st);
+    rc = launch_sort(pixels, B * H * W, ws.pix_z, ws.pix_c, nullptr, (int)ws.pix_stride, np.max_cmp, nullptr, st);
     if (rc) return rc;
     rc = launch_merge_patches(ws.pix_z, ws.pix_c, ws.pix_stride, ws.sorted, ws.perm, ws.n_real, g, ws.stride,
                               np.max_cmp, st);

@@ -12,7 +12,8 @@
 namespace snntc {
 
 constexpr int kWave = 64;              // CDNA wavefront width
-constexpr int kMaxSegment = 8192;      // longest sortable segment (power-of-two padded)
+constexpr int kMaxSegment = 8192;      // longest segment one sorting network takes; longer ones are merged from pieces
+constexpr int kMaxLongSegment = 1 << 24;
 constexpr size_t kAlign = 256;         // workspace sub-buffer alignment
 constexpr int kMaxDevices = 64;        // device indices the per-device one-time state covers
 
@@ -138,8 +139,11 @@ inline int64_t padded_stride(int64_t I) { return (I + 15) / 16 * 16; }
 
 // Segmented stable ascending sort: sorted[S,out_stride] and perm[S,out_stride] (entries past the
 // segment length hold +inf / 0), n_real[S] = number of values <= max_cmp (may be NULL).
+// Segments longer than kMaxSegment are sorted in pieces and merged in global memory; they need
+// `long_ws`, sort_long_workspace_bytes(S, I) bytes of scratch (NULL otherwise).
+size_t sort_long_workspace_bytes(int64_t S, int64_t I);
 int launch_sort(const SegmentSource& src, int64_t S, float* sorted, int32_t* perm, int32_t* n_real,
-                int out_stride, float max_cmp, hipStream_t stream);
+                int out_stride, float max_cmp, void* long_ws, hipStream_t stream);
 
 // Conv patch sort by merging pre-sorted pixels (merge.hip): pix_z / pix_c are the [B*H*W, Cs] outputs
 // of launch_sort on the image's pixels.

@@ -28,10 +28,14 @@ __device__ __forceinline__ float key_to_float(uint32_t k) {
     return __uint_as_float(k ^ ((k >> 31) ? 0x80000000u : 0xffffffffu));
 }
 
-template <int EPT, int G, int BLOCK>
+// RUNS: segments longer than the network are cut into `runs` pieces of NPAD elements; a unit of work is
+// one piece, and its sorted keys (value image << 32 | index in the segment; padding keys sort last
+// and carry their own position) go to keys[seg][run][NPAD] for the merge passes below.
+template <int EPT, int G, int BLOCK, bool RUNS = false>
 __global__ void __launch_bounds__(BLOCK)
 sort_segments_kernel(SegmentSource src, float* __restrict__ sorted, int32_t* __restrict__ perm,
-                     int32_t* __restrict__ n_real, int S, int out_stride, float max_cmp) {
+                     int32_t* __restrict__ n_real, int S, int out_stride, float max_cmp,
+                     unsigned long long* __restrict__ keys = nullptr, int runs = 1) {
     constexpr int NPAD = EPT * G;
     constexpr int SEGS = BLOCK / G;
     constexpr bool CROSS_WAVE = G > kWave;
@@ -42,7 +46,13 @@ sort_segments_kernel(SegmentSource src, float* __restrict__ sorted, int32_t* __r
     __shared__ int wave_count[CROSS_WAVE ? G / kWave : 1];
 
     const int tseg = threadIdx.x % G;
-    const int seg = blockIdx.x * SEGS + threadIdx.x / G;
+    int seg = blockIdx.x * SEGS + threadIdx.x / G;
+    int e0 = 0;                                           // first element of the unit in its segment
+    if constexpr (RUNS) {
+        const int unit = seg;
+        seg = unit / runs;
+        e0 = (unit - seg * runs) * NPAD;
+    }
     const bool live = seg < S;
     const int I = src.I;
 
@@ -59,15 +69,15 @@ sort_segments_kernel(SegmentSource src, float* __restrict__ sorted, int32_t* __r
                 p += ((size_t)(a * src.H + nh * src.Sh) * src.W + (size_t)nw * src.Sw) * src.C;
                 span = src.Kw * src.C;          // contiguous floats per kernel row
                 row = src.W * src.C;            // floats per image row
-                kh = (tseg * EPT) / span;
-                rem = tseg * EPT - kh * span;
+                kh = (e0 + tseg * EPT) / span;
+                rem = e0 + tseg * EPT - kh * span;
             } else {
                 p += (size_t)seg * I;
             }
         }
 #pragma unroll
         for (int r = 0; r < EPT; ++r) {
-            const int e = tseg * EPT + r;
+            const int e = e0 + tseg * EPT + r;
             uint32_t key = 0xffffffffu;
             if (live && e < I) {
                 float f;
@@ -131,6 +141,14 @@ sort_segments_kernel(SegmentSource src, float* __restrict__ sorted, int32_t* __r
         }
     }
 
+    if constexpr (RUNS) {
+        if (live) {
+            u64* ko = keys + ((size_t)seg * runs) * NPAD + e0 + tseg * EPT;
+#pragma unroll
+            for (int r = 0; r < EPT; ++r) ko[r] = v[r];
+        }
+        return;
+    }
     // ---- store: rows are out_stride long; positions past the segment get (+inf, row 0) ------------
     int below = 0;                      // own elements that take part in the scan (value <= MAX-0.1)
     if (live) {
@@ -183,15 +201,114 @@ int launch_sort_t(const SegmentSource& src, int64_t S, float* sorted, int32_t* p
     return SNNTC_OK;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Segments longer than the largest network (kMaxSegment): the pieces sorted by the RUNS
+// instantiation above are merged pairwise, pass after pass, in global memory.  A wavefront
+// produces MERGE_TILE consecutive keys of a merged pair: every lane finds by binary search how
+// many of the keys before its share come from the first run (merge path) and then merges its
+// share step by step.  Keys are distinct (they contain the index), so the result is the stable
+// order whatever the pass structure.  The last pass writes the (value, index) rows the scan reads,
+// with (+inf, 0) past the segment's end.  Rare and long: written for simplicity, not for speed.
+// ---------------------------------------------------------------------------------------------
+constexpr int MERGE_TILE = 1024;
+constexpr int MERGE_PER_LANE = MERGE_TILE / kWave;
+
+__global__ void __launch_bounds__(256)
+merge_runs_kernel(const u64* __restrict__ in, u64* __restrict__ out, float* __restrict__ sorted,
+                  int32_t* __restrict__ perm, int S, int I, int total, int L, int out_stride, int last) {
+    const int lane = threadIdx.x % kWave;
+    const int64_t tile = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+    const int tiles_per_seg = total / MERGE_TILE;
+    const int seg = (int)(tile / tiles_per_seg);
+    if (seg >= S) return;
+    const int pos0 = (int)(tile - (int64_t)seg * tiles_per_seg) * MERGE_TILE;       // first output of the tile
+    const int base = pos0 / (2 * L) * (2 * L);                                      // first key of the pair
+    const int nA = min(L, total - base), nB = min(L, max(0, total - base - L));
+    const u64* A = in + (size_t)seg * total + base;
+    const u64* B = A + L;
+    const int d0 = pos0 - base + lane * MERGE_PER_LANE;
+    int lo = max(0, d0 - nB), hi = min(d0, nA);
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (A[mid] < B[d0 - mid - 1]) lo = mid + 1; else hi = mid;                 // A[mid] precedes B[j-1]: too few from A
+    }
+    int i = lo, j = d0 - lo;
+    for (int u = 0; u < MERGE_PER_LANE; ++u) {
+        const u64 a = i < nA ? A[i] : ~0ull, b = j < nB ? B[j] : ~0ull;
+        const bool take_a = a < b;
+        const u64 key = take_a ? a : b;
+        i += take_a ? 1 : 0;
+        j += take_a ? 0 : 1;
+        const int q = base + d0 + u;
+        if (!last) {
+            out[(size_t)seg * total + q] = key;
+        } else if (q < I) {
+            sorted[(size_t)seg * out_stride + q] = key_to_float((uint32_t)(key >> 32));
+            perm[(size_t)seg * out_stride + q] = (int32_t)(uint32_t)key;
+        } else if (q < out_stride) {
+            sorted[(size_t)seg * out_stride + q] = INFINITY;
+            perm[(size_t)seg * out_stride + q] = 0;
+        }
+    }
+}
+
+// n_real[seg] = entries of the sorted row that take part in the scan (value <= max_cmp)
+__global__ void __launch_bounds__(256)
+count_real_kernel(const float* __restrict__ sorted, int32_t* __restrict__ n_real, int I, int out_stride, float max_cmp) {
+    __shared__ int part[256 / kWave];
+    const float* row = sorted + (size_t)blockIdx.x * out_stride;
+    int n = 0;
+    for (int e = threadIdx.x; e < I; e += blockDim.x) n += row[e] <= max_cmp ? 1 : 0;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) n += __shfl_xor(n, d, kWave);
+    if (threadIdx.x % kWave == 0) part[threadIdx.x / kWave] = n;
+    __syncthreads();
+    if (threadIdx.x == 0) n_real[blockIdx.x] = part[0] + part[1] + part[2] + part[3];
+}
+
+int launch_sort_long(const SegmentSource& src, int64_t S, float* sorted, int32_t* perm, int32_t* n_real,
+                     int out_stride, float max_cmp, void* long_ws, hipStream_t stream) {
+    if (!long_ws) return fail(SNNTC_ERR_WORKSPACE, "sort: segments of %d inputs need the long-segment workspace", src.I);
+    const int runs = (src.I + kMaxSegment - 1) / kMaxSegment;
+    const int64_t total = (int64_t)runs * kMaxSegment;
+    if (S * total > 0x7fffffffLL * 8) return fail(SNNTC_ERR_TOO_LARGE, "sort: %lld segments of %d inputs", (long long)S, src.I);
+    u64* buf[2] = {static_cast<u64*>(long_ws), static_cast<u64*>(long_ws) + S * total};
+    if (S * runs > 0x7fffffffLL) return fail(SNNTC_ERR_TOO_LARGE, "sort: too many segments (%lld)", (long long)S);
+    KernelTimerScope timer_("sort_segments", stream);
+    hipLaunchKernelGGL((sort_segments_kernel<8, 1024, 1024, true>), dim3((unsigned)(S * runs)), dim3(1024), 0, stream, src,
+                       sorted, perm, nullptr, (int)S, out_stride, max_cmp, buf[0], runs);
+    const int64_t tiles = S * (total / MERGE_TILE);
+    const int64_t blocks = (tiles + 3) / 4;
+    if (blocks > 0x7fffffffLL) return fail(SNNTC_ERR_TOO_LARGE, "sort: grid too large");
+    int cur = 0;
+    for (int64_t L = kMaxSegment; L < total; L *= 2) {
+        const int last = 2 * L >= total;
+        hipLaunchKernelGGL(merge_runs_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, buf[cur], buf[cur ^ 1], sorted,
+                           perm, (int)S, src.I, (int)total, (int)L, out_stride, last);
+        cur ^= 1;
+    }
+    if (n_real)
+        hipLaunchKernelGGL(count_real_kernel, dim3((unsigned)S), dim3(256), 0, stream, sorted, n_real, src.I, out_stride,
+                           max_cmp);
+    SNNTC_HIP_CHECK(hipGetLastError());
+    return SNNTC_OK;
+}
+
 }  // namespace
 
+// Bytes of the extra workspace launch_sort needs for S segments of I inputs (0 up to kMaxSegment):
+// two key buffers for the merge passes.
+size_t sort_long_workspace_bytes(int64_t S, int64_t I) {
+    if (I <= kMaxSegment) return 0;
+    const int64_t runs = (I + kMaxSegment - 1) / kMaxSegment;
+    return (size_t)2 * S * runs * kMaxSegment * sizeof(u64);
+}
+
 int launch_sort(const SegmentSource& src, int64_t S, float* sorted, int32_t* perm, int32_t* n_real,
-                int out_stride, float max_cmp, hipStream_t stream) {
+                int out_stride, float max_cmp, void* long_ws, hipStream_t stream) {
     if (S <= 0 || src.I <= 0) return SNNTC_OK;
     const int I = src.I;
-    if (I > kMaxSegment)
-        return fail(SNNTC_ERR_UNSUPPORTED, "segment length %d exceeds the largest supported sort (%d)", I,
-                    kMaxSegment);
+    if (I > kMaxSegment) return launch_sort_long(src, S, sorted, perm, n_real, out_stride, max_cmp, long_ws, stream);
     if (I <= 32)   return launch_sort_t<2, 16>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
     if (I <= 64)   return launch_sort_t<2, 32>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
     if (I <= 128)  return launch_sort_t<2, 64>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);

@@ -68,8 +68,14 @@ def test_fc_forward_argument_errors(lib):
     assert b"output tensor" in lib.snntc_last_error()
     assert lib.snntc_fc_forward(FAKE, FAKE, _fp(p0), FAKE, 1, 8192, 1 << 19, 8192, FAKE, 1 << 20, None) == _lib.ERR_TOO_LARGE
     assert b"weight tensor" in lib.snntc_last_error()
-    # segments longer than the largest sort
-    assert lib.snntc_fc_forward(FAKE, FAKE, _fp(p0), FAKE, 2, 9000, 4, 9000, FAKE, 1 << 20, None) == _lib.ERR_UNSUPPORTED
+    # segments longer than the largest supported one (2^24 inputs)
+    assert lib.snntc_fc_forward(FAKE, FAKE, _fp(p0), FAKE, 2, (1 << 24) + 1, 4, (1 << 24) + 1, FAKE, 1 << 20, None) == _lib.ERR_UNSUPPORTED
+    # segments longer than one sorting network (8192) need room for the merge passes as well
+    need_short, need_long = ctypes.c_size_t(), ctypes.c_size_t()
+    assert lib.snntc_fc_forward_workspace_bytes(2, 8192, 4, ctypes.byref(need_short)) == _lib.OK
+    assert lib.snntc_fc_forward_workspace_bytes(2, 9000, 4, ctypes.byref(need_long)) == _lib.OK
+    assert need_long.value >= need_short.value + 2 * 2 * 16384 * 8
+    assert lib.snntc_fc_forward(FAKE, FAKE, _fp(p0), FAKE, 2, 9000, 4, 9000, FAKE, need_short.value, None) == _lib.ERR_WORKSPACE
     # workspace: missing, misaligned, too small
     assert lib.snntc_fc_forward(FAKE, FAKE, _fp(p0), FAKE, 4, 10, 5, 10, None, 0, None) == _lib.ERR_WORKSPACE
     assert lib.snntc_fc_forward(FAKE, FAKE, _fp(p0), FAKE, 4, 10, 5, 10, ctypes.c_void_p(0x1010), 1 << 20, None) == _lib.ERR_WORKSPACE

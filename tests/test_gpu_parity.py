@@ -65,7 +65,12 @@ DENSE_CASES = [
     (18, 3, 5117, 24, True, "baseline"),       # 5118 rows x 8 columns: the largest slice that is kept in LDS
     (19, 3, 5120, 24, False, "baseline"),      # 160 KB exactly: no room left beside the slice, streaming scan
     (20, 3, 5120, 70, True, "baseline"),       # first size past it: streaming scan, two column blocks
-    (21, 2, 8192, 33, True, "reftest"),        # the longest supported segment
+    (21, 2, 8192, 33, True, "reftest"),        # the longest segment one sorting network takes
+    # longer segments: sorted in pieces of 8192 and merged in global memory
+    (23, 3, 8193, 20, True, "reftest"),        # two pieces, the second with a single input
+    (24, 2, 12000, 70, False, "baseline"),     # two pieces, one merge pass
+    (25, 2, 20000, 24, True, "reftest"),       # three pieces: a pass with an unpaired run
+    (26, 1, 41000, 9, True, "baseline"),       # six pieces, three passes; narrow backward pass
     (22, 5, 6000, 7, False, "reftest"),        # streaming scan with a narrow layer (the narrow backward pass)
 ]
 
@@ -184,6 +189,7 @@ CONV_CASES = [
     (8, 2, 10, 9, 48, 20, 3, 2, 2, 1, True, True, "reftest"),       # channels not a power of two
     (9, 2, 9, 9, 32, 16, 3, 3, 2, 2, True, False, "baseline"),      # stride 2 with 32 channels
     (10, 1, 12, 7, 40, 8, 2, 3, 1, 2, False, True, "reftest"),      # VALID, ragged kernel and stride
+    (11, 1, 3, 4, 1024, 24, 3, 3, 1, 1, True, True, "baseline"),    # P = 9216: patches longer than one sorting network
 ]
 
 
@@ -229,6 +235,28 @@ def test_conv_sort_with_heavy_ties(C, Kh, Kw, Sh, Sw):
     p = capi.cv_params(Kh, Kw, Sh, Sw, same=True, biasvolt=1.0)
     ref_out, ref_k, ref_sorted, ref_perm = capi.cv_forward_dev(xpad, w, p, want_aux=True)
     out, sz, perm, ck = snn.snncv(t(xpad), t(w), p, return_aux=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(perm.cpu().numpy(), ref_perm), "permutation differs"
+    assert np.array_equal(sz.cpu().numpy(), ref_sorted)
+    assert np.array_equal(ck.cpu().numpy(), ref_k)
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), ref_out.view(np.uint32))
+
+
+@pytest.mark.parametrize("I", [8200, 16385, 30000])
+def test_long_segment_sort_with_heavy_ties(I):
+    """Segments longer than one sorting network, quantised so that equal values sit in different
+    pieces: the merge passes must keep them in index order; some inputs lie above MAX_SPIKE_TIME - 0.1
+    (they sort last and do not count as scan inputs), one row has none below it."""
+    import snntc_amd as snn
+    rng = np.random.default_rng(I)
+    B, J = 3, 5
+    x = (1.0 + rng.integers(0, 9, (B, I)) / 8.0).astype(np.float32)
+    x[0, rng.integers(0, I, 40)] = 2e5
+    x[2, :] = 3e5
+    w = (rng.standard_normal((I + 1, J)) * 0.05 + 4.0 / I).astype(np.float32)
+    p = capi.fc_params(1.0)
+    ref_out, ref_k, ref_sorted, ref_perm = capi.fc_forward_dev(x, w, p, want_aux=True)
+    out, sz, perm, ck = snn.snnfc(t(x), t(w), p, return_aux=True)
     torch.cuda.synchronize()
     assert np.array_equal(perm.cpu().numpy(), ref_perm), "permutation differs"
     assert np.array_equal(sz.cpu().numpy(), ref_sorted)
