@@ -274,10 +274,12 @@ __device__ __forceinline__ void accumulate_chunk(float& wsum, float& ysum, int& 
 // Copies columns [j0, j0 + COLS) of all `rows` rows of W[rows, J] into LDS as wl[row][COLS] (zeros
 // past column J).  Loads are issued in batches so that a small workgroup does not pay one memory
 // latency per element.
+// Returns the largest |w| among the values this thread copied (NaN entries skipped).
 template <int COLS>
-__device__ __forceinline__ void fill_weight_slice(float* __restrict__ wl, const float* __restrict__ w, int rows,
-                                                  int J, int j0) {
+__device__ __forceinline__ float fill_weight_slice(float* __restrict__ wl, const float* __restrict__ w, int rows,
+                                                   int J, int j0) {
     const int n_fill = rows * COLS;
+    float amax = 0.0f;
     if ((J & 3) == 0) {
         constexpr int C4 = COLS / 4, FILL = 4;
         for (int base = threadIdx.x; base < rows * C4; base += FILL * blockDim.x) {
@@ -293,6 +295,7 @@ __device__ __forceinline__ void fill_weight_slice(float* __restrict__ wl, const 
             for (int u = 0; u < FILL; ++u) {
                 const int idx = base + u * blockDim.x;
                 if (idx < rows * C4) reinterpret_cast<float4*>(wl)[idx] = v[u];
+                amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[u].x), fabsf(v[u].y)), fmaxf(fabsf(v[u].z), fabsf(v[u].w))));
             }
         }
     } else if (j0 == 0 && J > 1 && J < COLS && (reinterpret_cast<uintptr_t>(w) & 15) == 0 && rows * J < (1 << 24)) {
@@ -321,13 +324,16 @@ __device__ __forceinline__ void fill_weight_slice(float* __restrict__ wl, const 
                     for (int t = 0; t < 4; ++t) {
                         const unsigned e = 4u * idx + t, r = __umulhi(e, magic);
                         wl[r * COLS + (e - r * J)] = q[t];
+                        amax = fmaxf(amax, fabsf(q[t]));
                     }
                 }
             }
         }
         if ((int)threadIdx.x < n - 4 * n4) {
             const unsigned e = 4u * n4 + threadIdx.x, r = __umulhi(e, magic);
-            wl[r * COLS + (e - r * J)] = w[e];
+            const float v = w[e];
+            wl[r * COLS + (e - r * J)] = v;
+            amax = fmaxf(amax, fabsf(v));
         }
     } else {
         constexpr int FILL = 16;
@@ -343,9 +349,11 @@ __device__ __forceinline__ void fill_weight_slice(float* __restrict__ wl, const 
             for (int u = 0; u < FILL; ++u) {
                 const int idx = base + u * blockDim.x;
                 if (idx < n_fill) wl[idx] = v[u];
+                amax = fmaxf(amax, fabsf(v[u]));
             }
         }
     }
+    return amax;
 }
 
 // Launches with at most a couple of wavefronts per SIMD, where nothing hides a stall: workgroups of
@@ -776,15 +784,10 @@ __device__ __forceinline__ void filter_chunk(float& wsum, float& ysum, int& kfla
         : "vcc", "scc");
 }
 
-// Largest |w| of the slice in LDS (n4 float4 entries), the same value in every thread.  `red` is
-// room for one float per wavefront.  NaN entries are skipped (a NaN sum never closes a set, with
-// or without the filter).
-__device__ __forceinline__ float slice_abs_max(const float* __restrict__ wl, int n4, float* __restrict__ red) {
-    float m = 0.0f;
-    for (int idx = threadIdx.x; idx < n4; idx += blockDim.x) {
-        const float4 v = reinterpret_cast<const float4*>(wl)[idx];
-        m = fmaxf(m, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
-    }
+// Largest of the threads' `m` over the workgroup, the same value in every thread.  `red` is room for
+// one float per wavefront; the call contains the workgroup barrier that also publishes whatever the
+// threads wrote to LDS before it.
+__device__ __forceinline__ float block_max(float m, float* __restrict__ red) {
 #pragma unroll
     for (int d = kWave / 2; d > 0; d >>= 1) m = fmaxf(m, __shfl_xor(m, d, kWave));
     if (threadIdx.x % kWave == 0) red[threadIdx.x / kWave] = m;
@@ -851,9 +854,8 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
     const int group = block - slice * n_groups;
     const int j0 = slice * COLS;
     const int rows = I + np.bias;
-    fill_weight_slice<COLS>(wl, w, rows, J, j0);
-    __syncthreads();
-    const float thr_w = FILTER_W * slice_abs_max(wl, rows * COLS / 4, wl + rows * COLS);
+    // the slice, and the largest |w| in it (the threads' shares of the copy, then the workgroup's)
+    const float thr_w = FILTER_W * block_max(fill_weight_slice<COLS>(wl, w, rows, J, j0), wl + rows * COLS);
 
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
