@@ -89,7 +89,9 @@ SNNTC_API int snntc_init(int device);
  * ------------------------------------------------------------------------------------------- */
 
 /* Scratch sizes.  Replaces the reference's allocate_temp calls (snntc/snnfc_kernels.cu.cc:110-137,
- * snntc/snnfcgrad_kernels.cu.cc:159-164). */
+ * snntc/snnfcgrad_kernels.cu.cc:159-164).  Inputs longer than 8192 per segment (I here, Kh*Kw*C
+ * for conv layers) are sorted in pieces and merged in device memory; the forward size then includes
+ * two key buffers for the merge passes.  Segments beyond 2^24 inputs -> UNSUPPORTED. */
 SNNTC_API int snntc_fc_forward_workspace_bytes(int64_t B, int64_t I, int64_t J, size_t* bytes);
 SNNTC_API int snntc_fc_backward_workspace_bytes(int64_t B, int64_t I, int64_t J, size_t* bytes);
 
