@@ -1144,9 +1144,11 @@ unpad_rows_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ 
 }  // namespace
 
 namespace {
-// Neurons per lane of the instantiation for large launches (four need 151 registers: too few
-// wavefronts per SIMD, measured slower).
-constexpr int filter_ch(int cols) { return 2; }
+// Neurons per lane of the instantiation for large launches: two (four need 151 registers: too few
+// wavefronts per SIMD, measured slower), except with 8-column slices, whose 32-byte weight rows make
+// the 8-byte reads of two-neuron lanes collide in the LDS banks (sixteen rows per read on four bank
+// groups): one neuron per lane reads eight rows at 4 bytes a lane.
+constexpr int filter_ch(int cols) { return cols == 8 ? 1 : 2; }
 
 template <int COLS>
 int raise_scan_lds_limits() {
