@@ -11,7 +11,7 @@ runs, once per workload and from the repository root,
                                               -- (the same command without --calibration-copies)
 
 each pass a run of its own under a time limit (counters and traces are never combined), keeps the raw
-output under DIR (default gpurun_out/profiles_raw) and writes into --out (default profiles/):
+output under --raw DIR and writes into --out (default profiles/):
 
     <W>_step_kernel_trace.txt     top kernels by total time, with the bench line of the traced run
     <W>_hbm_traffic_pmc.txt       FETCH_SIZE / WRITE_SIZE per launch, scaled by what the plain 256 MiB device

@@ -223,6 +223,7 @@ def test_gradients_against_the_literal_tolerance(name, kind, shape):
         assert share_hip <= max(1.5 * share_seq, 1e-3), (label, stats[label])
         assert worst_hip <= max(2.0 * worst_seq, 1.0), (label, stats[label])
     print(json.dumps(stats))
-    if os.path.isdir("gpurun_out"):
-        with open(os.path.join("gpurun_out", f"literal_bar_{kind}.json"), "w") as f:
+    stats_dir = os.environ.get("SNNTC_STATS_DIR")
+    if stats_dir and os.path.isdir(stats_dir):
+        with open(os.path.join(stats_dir, f"literal_bar_{kind}.json"), "w") as f:
             json.dump(stats, f, indent=1)
