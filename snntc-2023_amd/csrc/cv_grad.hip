@@ -7,6 +7,7 @@
 // Both kernels put the channel (dX) or the output channel (dW) on the lanes, so everything that
 // depends only on the patch is wave-uniform and is fetched through the scalar path.
 #include "snntc_common.h"
+#include <type_traits>
 
 namespace snntc {
 namespace {
@@ -297,29 +298,30 @@ cv_grad_weight_wide_kernel(const float* __restrict__ xpad, const float* __restri
         const float* yp = ym + (size_t)s_lo * Kc + jc;
         const float* up = upm + (size_t)s_lo * Kc + jc;
         float y_next = *yp, u_next = *up;
-        const int s_fast = (FULL || n_rows == R) ? s_hi : min(s_hi, s_safe);
-        for (int s = s_lo; s < s_hi; ++s) {
-            const float yv = y_next * -neg_s, uv = u_next;
-            if (s + 1 < s_hi) { yp += Kc; up += Kc; }
-            y_next = *yp; u_next = *up;
-            if (FULL || s < s_fast) {
+        // A block at the end of a kernel row fetches past its rows (the values are discarded), except
+        // for the last few patches of the tensor, where that fetch could leave it: there the unused
+        // rows re-read the block's last row.  Two loops, so that neither carries the other's code.
+        const int s_fast = (FULL || n_rows == R) ? s_hi : max(s_lo, min(s_hi, s_safe));
+        auto patches = [&](int s_from, int s_to, auto clamp_rows) {
+            for (int s = s_from; s < s_to; ++s) {
+                const float yv = y_next * -neg_s, uv = u_next;
+                if (s + 1 < s_hi) { yp += Kc; up += Kc; }
+                y_next = *yp; u_next = *up;
 #pragma unroll
-                for (int r = 0; r < R; ++r) acc[r] = __fmaf_rn(scaled_lead(xb[r], neg_s, yv), uv, acc[r]);
-            } else {
-                // A block at the end of a kernel row fetches past its rows (the values are discarded),
-                // except for the last few patches of the tensor, where that fetch could leave it: there
-                // the unused rows re-read the block's last row.
-#pragma unroll
-                for (int r = 0; r < R; ++r)
-                    acc[r] = __fmaf_rn(scaled_lead(xb[min(r, n_rows - 1)], neg_s, yv), uv, acc[r]);
+                for (int r = 0; r < R; ++r) {
+                    const float xv = decltype(clamp_rows)::value ? xb[min(r, n_rows - 1)] : xb[r];
+                    acc[r] = __fmaf_rn(scaled_lead(xv, neg_s, yv), uv, acc[r]);
+                }
+                if (with_bias) acc_bias = __fmaf_rn(scaled_lead(biasvolt, neg_s, yv), uv, acc_bias);
+                xb += step_w;
+                if (++nw == Nw) {
+                    nw = 0; xb += wrap_w;
+                    if (++nh == Nh) { nh = 0; xb += wrap_h; }
+                }
             }
-            if (with_bias) acc_bias = __fmaf_rn(scaled_lead(biasvolt, neg_s, yv), uv, acc_bias);
-            xb += step_w;
-            if (++nw == Nw) {
-                nw = 0; xb += wrap_w;
-                if (++nh == Nh) { nh = 0; xb += wrap_h; }
-            }
-        }
+        };
+        patches(s_lo, s_fast, std::false_type{});
+        if (!FULL) patches(s_fast, s_hi, std::true_type{});
     }
     if (wave > 0) {
 #pragma unroll
