@@ -295,9 +295,17 @@ cv_grad_weight_wide_kernel(const float* __restrict__ xpad, const float* __restri
         const ptrdiff_t wrap_w = ((ptrdiff_t)Sh * W - (ptrdiff_t)Nw * Sw) * C;
         const ptrdiff_t wrap_h = ((ptrdiff_t)H - (ptrdiff_t)Nh * Sh) * W * C;
         // y and up of the next patch are requested before the current one is worked on
-        const float* yp = ym + (size_t)s_lo * Kc + jc;
-        const float* up = upm + (size_t)s_lo * Kc + jc;
-        float y_next = *yp, u_next = *up;
+        // (through buffer descriptors of the wavefront's patch range: a scalar running offset plus the
+        // lane's constant column offset, no vector address arithmetic)
+        const int range_bytes = (int)min((int64_t)(s_hi - s_lo) * Kc * (int64_t)sizeof(float), (int64_t)0x7ffffffc);
+        const __amdgpu_buffer_rsrc_t ybuf =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(ym + (size_t)s_lo * Kc), 0, range_bytes, 0x00020000);
+        const __amdgpu_buffer_rsrc_t ubuf =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(upm + (size_t)s_lo * Kc), 0, range_bytes, 0x00020000);
+        const int col_bytes = (int)(jc * sizeof(float)), patch_bytes = Kc * (int)sizeof(float);
+        int next_bytes = 0;
+        float y_next = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ybuf, col_bytes, 0, 0));
+        float u_next = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ubuf, col_bytes, 0, 0));
         // A block at the end of a kernel row fetches past its rows (the values are discarded), except
         // for the last few patches of the tensor, where that fetch could leave it: there the unused
         // rows re-read the block's last row.  Two loops, so that neither carries the other's code.
@@ -305,14 +313,18 @@ cv_grad_weight_wide_kernel(const float* __restrict__ xpad, const float* __restri
         auto patches = [&](int s_from, int s_to, auto clamp_rows) {
             for (int s = s_from; s < s_to; ++s) {
                 const float yv = y_next * -neg_s, uv = u_next;
-                if (s + 1 < s_hi) { yp += Kc; up += Kc; }
-                y_next = *yp; u_next = *up;
+                if (s + 1 < s_hi) next_bytes += patch_bytes;
+                y_next = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ybuf, col_bytes, next_bytes, 0));
+                u_next = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ubuf, col_bytes, next_bytes, 0));
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     const float xv = decltype(clamp_rows)::value ? xb[min(r, n_rows - 1)] : xb[r];
                     acc[r] = __fmaf_rn(scaled_lead(xv, neg_s, yv), uv, acc[r]);
                 }
-                if (with_bias) acc_bias = __fmaf_rn(scaled_lead(biasvolt, neg_s, yv), uv, acc_bias);
+                if (with_bias) {                          // block-uniform: a branch, not a select
+                    asm volatile("");
+                    acc_bias = __fmaf_rn(scaled_lead(biasvolt, neg_s, yv), uv, acc_bias);
+                }
                 xb += step_w;
                 if (++nw == Nw) {
                     nw = 0; xb += wrap_w;
