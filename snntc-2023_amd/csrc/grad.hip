@@ -96,7 +96,7 @@ __device__ __forceinline__ const float* segment_base(const SegmentSource& src, i
 // and are summed through LDS in a fixed order.
 // ---------------------------------------------------------------------------------------------
 constexpr int DX_RB = 4;
-constexpr int DX_UNROLL = 8;
+constexpr int DX_STEP = 4;
 
 // PATCHES: the "samples" are the implicit patches of a conv layer (src.conv) and the result is the
 // gradient per patch element, dx[S, P], which cv_col2im_kernel then folds back onto the image.
@@ -128,27 +128,76 @@ fc_grad_input_kernel(const SegmentSource src, const float* __restrict__ wt,
     const int j_lo = wave * jq, j_hi = min(J, j_lo + jq);
     const float* __restrict__ wcol = wt + ic;
     int j = j_lo;
-    // DX_UNROLL columns at a time: their weights are requested together, the y / up values of the
-    // block's samples are wave-uniform and arrive through the scalar path.
-    for (; j + DX_UNROLL <= j_hi; j += DX_UNROLL) {
-        float wv[DX_UNROLL];
+    // DX_STEP columns at a time.  The y / up values of the block's samples are wave-uniform and arrive
+    // through the scalar path; scalar loads return in no fixed order, so a wavefront can only wait for
+    // all of them, and a load issued right before its use costs a round trip every time.  The loop
+    // therefore runs one step ahead: wait for the values of this step (requested a step ago), request
+    // those of the next into the other set of registers, then do this step's arithmetic.  The
+    // weights (vector loads, which return in order) run one step ahead as well.
+    {
+        typedef float f4 __attribute__((ext_vector_type(4)));
+        auto request = [&](f4 (&yv)[DX_RB], f4 (&uv)[DX_RB], int jj) {
+            const int off = jj * (int)sizeof(float);
 #pragma unroll
-        for (int u = 0; u < DX_UNROLL; ++u) wv[u] = wcol[(size_t)(j + u) * wt_stride];
-#pragma unroll
-        for (int r = 0; r < DX_RB; ++r) {
-#pragma unroll
-            for (int u = 0; u < DX_UNROLL; ++u) {
-                const float t = xr[r] <= yrow[r][j + u] ? wv[u] : 0.0f;
-                acc[r] = __fmaf_rn(urow[r][j + u], t, acc[r]);
+            for (int r = 0; r < DX_RB; ++r) {
+                asm volatile("s_load_dwordx4 %0, %1, %2" : "=s"(yv[r]) : "s"(yrow[r]), "s"(off));
+                asm volatile("s_load_dwordx4 %0, %1, %2" : "=s"(uv[r]) : "s"(urow[r]), "s"(off));
             }
+        };
+        auto arrived = [&](f4 (&yv)[DX_RB], f4 (&uv)[DX_RB]) {
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+s"(yv[0]), "+s"(yv[1]), "+s"(yv[2]), "+s"(yv[3]), "+s"(uv[0]), "+s"(uv[1]), "+s"(uv[2]),
+                           "+s"(uv[3]));
+        };
+        auto weights = [&](float (&wv)[DX_STEP], int jj) {
+#pragma unroll
+            for (int u = 0; u < DX_STEP; ++u) wv[u] = (wt + (size_t)(jj + u) * wt_stride)[ic];
+        };
+        // acc[r] += up * w where x <= y; the others are skipped, as in the reference
+        // (snnfcgrad_kernels.cu.cc:60), not added as zeros.  (Writing the compare into EXEC and running
+        // the multiply-add under it saves the select but no time: the EXEC round trip stalls the issue.)
+        auto macs = [&](const f4 (&yv)[DX_RB], const f4 (&uv)[DX_RB], const float (&wv)[DX_STEP]) {
+#pragma unroll
+            for (int r = 0; r < DX_RB; ++r) {
+#pragma unroll
+                for (int u = 0; u < DX_STEP; ++u)
+                    acc[r] = xr[r] <= yv[r][u] ? __fmaf_rn(uv[r][u], wv[u], acc[r]) : acc[r];
+            }
+        };
+        static_assert(DX_RB == 4 && DX_STEP == 4, "register sets of the pipelined loop");
+        const int steps = (j_hi - j_lo) / DX_STEP;
+        if (steps > 0) {
+            f4 ya[DX_RB], ua[DX_RB], yb[DX_RB], ub[DX_RB];
+            float wa[DX_STEP], wb[DX_STEP];
+            const int j_last = j_lo + (steps - 1) * DX_STEP;      // requests past the last step re-read it
+            request(ya, ua, j);
+            weights(wa, j);
+            for (int sidx = 0; sidx + 2 <= steps; sidx += 2) {
+                const int jn = j + DX_STEP, jnn = min(j + 2 * DX_STEP, j_last);
+                arrived(ya, ua);
+                request(yb, ub, jn);
+                weights(wb, jn);
+                __builtin_amdgcn_sched_barrier(0);                 // requests first, then the arithmetic
+                macs(ya, ua, wa);
+                __builtin_amdgcn_sched_barrier(0);
+                arrived(yb, ub);
+                request(ya, ua, jnn);
+                weights(wa, jnn);
+                __builtin_amdgcn_sched_barrier(0);
+                macs(yb, ub, wb);
+                __builtin_amdgcn_sched_barrier(0);
+                j += 2 * DX_STEP;
+            }
+            arrived(ya, ua);                                       // nothing stays in flight
+            if (steps & 1) macs(ya, ua, wa);
+            j = j_lo + steps * DX_STEP;
         }
     }
     for (; j < j_hi; ++j) {
         const float wv = wcol[(size_t)j * wt_stride];
 #pragma unroll
         for (int r = 0; r < DX_RB; ++r) {
-            const float t = xr[r] <= yrow[r][j] ? wv : 0.0f;
-            acc[r] = __fmaf_rn(urow[r][j], t, acc[r]);
+            acc[r] = xr[r] <= yrow[r][j] ? __fmaf_rn(urow[r][j], wv, acc[r]) : acc[r];
         }
     }
     if (wave > 0) {
@@ -291,9 +340,15 @@ grad_weight_dense_kernel(const float* __restrict__ x, const float* __restrict__ 
     const unsigned jc = (unsigned)min(j, J - 1);
     const int i0 = blockIdx.y * DW_RI;
     const int s_begin = blockIdx.z * seg_per_slice;
-    const int s_end = min(S, s_begin + seg_per_slice);
-    const float* __restrict__ ycol = ym + jc;
-    const float* __restrict__ ucol = upm + jc;
+    const int s_end = __builtin_amdgcn_readfirstlane(min(S, s_begin + seg_per_slice));
+    // ym / upm of the slice through buffer descriptors: the sample's row is a scalar offset, the lane's
+    // column a constant one, and no address is computed per lane (the launcher keeps a slice below 2 GB)
+    const int slice_bytes = max(s_end - s_begin, 0) * J * (int)sizeof(float);
+    const __amdgpu_buffer_rsrc_t ybuf =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(ym + (size_t)s_begin * J), 0, slice_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t ubuf =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(upm + (size_t)s_begin * J), 0, slice_bytes, 0x00020000);
+    const int col_bytes = (int)(jc * sizeof(float)), row_bytes = J * (int)sizeof(float);
 
     float acc[DW_RI];
 #pragma unroll
@@ -317,6 +372,31 @@ grad_weight_dense_kernel(const float* __restrict__ x, const float* __restrict__ 
         for (int k = 0; k < DW_RI; ++k) xt[buf][st_smp + 32 * k][st_row] = pending[k];
     };
 
+    // ym / upm of DWD_BATCH samples are requested together, then the batch is worked on.  (Requesting a
+    // batch ahead of the arithmetic changes nothing: alone, the requests of a launch keep L2 busy for
+    // about as long as the arithmetic keeps the vector units busy, and the two overlap only in part.)
+    auto load_batch = [&](float (&yv)[DWD_BATCH], float (&uv)[DWD_BATCH], int sb) {
+#pragma unroll
+        for (int q = 0; q < DWD_BATCH; ++q) {
+            const int sc = __builtin_amdgcn_readfirstlane(min(sb + q, s_end - 1));   // past the end: the last sample again
+            const int off = (sc - s_begin) * row_bytes;
+            yv[q] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ybuf, col_bytes, off, 0));
+            uv[q] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ubuf, col_bytes, off, 0));
+        }
+    };
+    auto run_batch = [&](const float (&yv)[DWD_BATCH], const float (&uv)[DWD_BATCH], int sb, int buf, int h) {
+#pragma unroll
+        for (int q = 0; q < DWD_BATCH; ++q) {
+            const float4* xq = reinterpret_cast<const float4*>(&xt[buf][wave * (DWD_TILE / 4) + h + q][0]);
+            const float4 xa = xq[0], xb = xq[1];
+            const float xr[DW_RI] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+            const float ys = yv[q] * -neg_s;
+            const float u = sb + q < s_end ? uv[q] : 0.0f;  // the surplus of the last batch weighs nothing
+#pragma unroll
+            for (int r = 0; r < DW_RI; ++r) acc[r] = __fmaf_rn(scaled_lead(xr[r], neg_s, ys), u, acc[r]);
+        }
+    };
+
     if (s_begin < s_end) {
         fetch_tile(s_begin);
         store_tile(0);
@@ -331,22 +411,8 @@ grad_weight_dense_kernel(const float* __restrict__ x, const float* __restrict__ 
                 const int sb = w0 + h;
                 if (sb >= s_end) break;                     // wavefront-uniform
                 float yv[DWD_BATCH], uv[DWD_BATCH];
-#pragma unroll
-                for (int q = 0; q < DWD_BATCH; ++q) {
-                    const int sc = min(sb + q, s_end - 1);
-                    yv[q] = ycol[(size_t)sc * J];
-                    uv[q] = ucol[(size_t)sc * J];
-                }
-#pragma unroll
-                for (int q = 0; q < DWD_BATCH; ++q) {
-                    const float4* xq = reinterpret_cast<const float4*>(&xt[buf][wave * (DWD_TILE / 4) + h + q][0]);
-                    const float4 xa = xq[0], xb = xq[1];
-                    const float xr[DW_RI] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
-                    const float ys = yv[q] * -neg_s;
-                    const float u = sb + q < s_end ? uv[q] : 0.0f;
-#pragma unroll
-                    for (int r = 0; r < DW_RI; ++r) acc[r] = __fmaf_rn(scaled_lead(xr[r], neg_s, ys), u, acc[r]);
-                }
+                load_batch(yv, uv, sb);
+                run_batch(yv, uv, sb, buf, h);
             }
             if (more) store_tile(buf ^ 1);
         }
@@ -649,7 +715,8 @@ int launch_grad_weight_rows(const SegmentSource& src, const float* upm, const fl
     {
         KernelTimerScope timer_(row_start ? "grad_weight_tail" : "grad_weight", stream);
         const LeadScale ls = lead_scale(np.max_time);
-        if (!src.conv && row_start == 0)
+        // (the dense kernel addresses a slice of ym / upm with 32-bit byte offsets)
+        if (!src.conv && row_start == 0 && ((int64_t)seg_per_slice + DWD_TILE) * J * (int64_t)sizeof(float) < 0x7fffffffLL)
             hipLaunchKernelGGL(grad_weight_dense_kernel, grid, dim3(256), 0, stream, src.base, upm, ym, dst, (int)S,
                                (int)src.I, (int)J, (int)rows, seg_per_slice, np.biasvolt, ls.neg_s, ls.post);
         else
