@@ -1051,7 +1051,7 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
             // eight inputs (positions are multiples of eight inside the full chunks of the row).  A scan
             // that closes is finished.  One that does not goes back to the fast loop if its fired state is
             // the plain one; otherwise (fired on a negative weight sum, say) it keeps stepping here, chunk
-            // by chunk, with the entries of its next chunk requested while the current one is worked on.
+            // by chunk.
             bool need[CH], any_need = false, any_armed = false;
             Chunk pc[CH];
 #pragma unroll
@@ -1063,9 +1063,11 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
                 any_armed |= armed[c];
             }
             if (__builtin_amdgcn_ballot_w64(any_need) != 0) {
-#pragma unroll
-                for (int c = 0; c < CH; ++c) load_chunk_flat(pc[c], xs, pr, need[c] ? kcur[c] : 0);
                 do {
+                    // (fetched on demand: a second round is rare, requesting its entries ahead of time
+                    // would cost every item eight more loads per scan)
+#pragma unroll
+                    for (int c = 0; c < CH; ++c) load_chunk_flat(pc[c], xs, pr, need[c] ? kcur[c] : 0);
                     any_need = false;
 #pragma unroll
                     for (int c = 0; c < CH; ++c) {
@@ -1075,8 +1077,6 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
                             pw[u] = wcol[pc[c].p[u] * COLS + c];
                             px[u] = pc[c].x[u];
                         }
-                        const int knext = kcur[c] + CHUNK;
-                        load_chunk_flat(pc[c], xs, pr, (need[c] && knext + CHUNK <= n_full) ? knext : 0);
                         float ya = wsum[c] < 0.0f ? -ysum[c] : ysum[c];
                         float yg = fired_cur[c] ? ya : INFINITY;
                         uint64_t exited = 0;
