@@ -24,6 +24,7 @@ output under --raw DIR and writes into --out (default profiles/):
 `summarise` redoes the text files and the table from raw output that is already there (kept with --keep-raw).
 """
 import argparse
+import tempfile
 import collections
 import json
 import os
@@ -234,11 +235,15 @@ def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("action", choices=["collect", "summarise"])
     ap.add_argument("--workloads", nargs="+", default=["cfg2", "cfg3", "cfg4", "cfg5"])
-    ap.add_argument("--raw", default=os.path.join(ROOT, "gpurun_out", "profiles_raw"))
+    ap.add_argument("--raw", default=None, help="folder for the raw rocprofv3 output (collect: a temporary one by default)")
     ap.add_argument("--out", default=os.path.join(ROOT, "profiles"))
     ap.add_argument("--keep-raw", action="store_true", help="keep the rocprofv3 databases after summarising")
     ap.add_argument("--commit", default=None, help="commit the measured tree is at (default: git rev-parse HEAD here)")
     args = ap.parse_args()
+    if args.raw is None:
+        if args.action == "summarise":
+            ap.error("summarise needs --raw (the folder a collect run with --keep-raw left)")
+        args.raw = tempfile.mkdtemp(prefix="snntc_profiles_")
     if args.action == "collect":
         collect(args.workloads, args.raw)
     summarise(args.workloads, args.raw, args.out, args.commit)
