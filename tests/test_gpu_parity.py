@@ -264,6 +264,28 @@ def test_long_segment_sort_with_heavy_ties(I):
     assert np.array_equal(out.cpu().numpy().view(np.uint32), ref_out.view(np.uint32))
 
 
+@pytest.mark.parametrize("I", [147, 200, 256])
+def test_many_short_segments_take_the_two_per_wavefront_sort(I):
+    """65 536 and more segments of 129..256 inputs (the patches of a 7x7x3 stem) are sorted two per
+    wavefront with eight elements per thread; quantised values make ties that must keep index order,
+    a few rows carry inputs above MAX_SPIKE_TIME - 0.1.  Everything bit for bit against the oracle."""
+    import snntc_amd as snn
+    rng = np.random.default_rng(I)
+    B, J = 65536 + 3, 4
+    x = (1.0 + rng.integers(0, 40, (B, I)) / 16.0).astype(np.float32)
+    x[5, rng.integers(0, I, 9)] = 2e5
+    x[B - 1, :] = 3e5
+    w = (rng.standard_normal((I + 1, J)) * 0.1 + 4.0 / I).astype(np.float32)
+    p = capi.fc_params(1.0)
+    ref_out, ref_k, ref_sorted, ref_perm = capi.fc_forward_dev(x, w, p, want_aux=True)
+    out, sz, perm, ck = snn.snnfc(t(x), t(w), p, return_aux=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(perm.cpu().numpy(), ref_perm), "permutation differs"
+    assert np.array_equal(sz.cpu().numpy(), ref_sorted)
+    assert np.array_equal(ck.cpu().numpy(), ref_k)
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), ref_out.view(np.uint32))
+
+
 def test_layer_autograd_matches_op_level_chain():
     """SNN_dense / SNN_conv hand the [B,...] upstream gradient to the backward op directly; the result
     must equal slicing the full op output under autograd (zero-extended gradient), bit for bit."""
