@@ -415,29 +415,44 @@ cv_grad_weight_narrow_kernel(const float* __restrict__ xpad, const float* __rest
 
     if (s_lo < s_hi) {
         const int per_img = Nh * Nw;
-        // this lane's patch: s_lo + half, then every second one; (a, nh, nw) follow it incrementally
+        // This lane's patch: s_lo + half, then every second one.  Its two inputs, ym and upm are followed
+        // by pointers that move by adds alone (a step of two patches, plus the wraps at the end of an
+        // output row and of an image), and the values of the next patch are requested before the
+        // current one is worked on.  A lane past its last patch keeps pointing at it, with upm = 0.
         int s = s_lo + half;
-        int sc = min(s, s_hi - 1);
-        int a = sc / per_img;
-        int r2 = sc - a * per_img;
+        const int sc = min(s, s_hi - 1);
+        const int a = sc / per_img;
+        const int r2 = sc - a * per_img;
         int nh = r2 / Nw, nw = r2 - nh * Nw;
+        const int l16 = lane & 15;                       // rows past the block's last one re-read it
+        const float* px0 = xpad + ((size_t)(a * H + nh * Sh + kh) * W + (size_t)(nw * Sw)) * C + q0 + min(l16, n_rows - 1);
+        const ptrdiff_t second = min(l16 + 16, n_rows - 1) - min(l16, n_rows - 1);
+        const float* py = ym + (size_t)sc * Kc + jc;
+        const float* pu = upm + (size_t)sc * Kc + jc;
+        const ptrdiff_t step_w = (ptrdiff_t)Sw * C;
+        const ptrdiff_t wrap_w = ((ptrdiff_t)Sh * W - (ptrdiff_t)Nw * Sw) * C;
+        const ptrdiff_t wrap_h = ((ptrdiff_t)H - (ptrdiff_t)Nh * Sh) * W * C;
         const int n_iter = (s_hi - s_lo + 1) / 2;
+        float x0n = px0[0], x1n = px0[second], yn = *py, un = s < s_hi ? *pu : 0.0f;
         for (int it = 0; it < n_iter; ++it) {
-            const bool have = s < s_hi;
-            const size_t xo = ((size_t)(a * H + nh * Sh + kh) * W + (size_t)(nw * Sw)) * C + q0;
-            const int l16 = lane & 15;                   // rows past the block's last one re-read it
-            const float x0 = xpad[xo + min(l16, n_rows - 1)], x1 = xpad[xo + min(l16 + 16, n_rows - 1)];
-            const float yv = ym[(size_t)sc * Kc + jc];
-            const float uv = have ? upm[(size_t)sc * Kc + jc] : 0.0f;
+            const float x0 = x0n, x1 = x1n, yv = yn, uv = un;
+            s += 2;
+            if (s < s_hi) {
+                py += 2 * Kc; pu += 2 * Kc;
+                px0 += 2 * step_w;
+                nw += 2;
+                while (nw >= Nw) {
+                    nw -= Nw; px0 += wrap_w;
+                    if (++nh == Nh) { nh = 0; px0 += wrap_h; }
+                }
+            }
+            if (it + 1 < n_iter) {                        // wavefront-uniform
+                x0n = px0[0]; x1n = px0[second]; yn = *py;
+                un = s < s_hi ? *pu : 0.0f;
+            }
             dw_rows16(acc, 0, x0, yv, uv);
             if (n_rows > 16) dw_rows16(acc, 16, x1, yv, uv);     // block-uniform
             if (with_bias) acc_bias = __fmaf_rn(fminf(biasvolt - yv, 0.0f), uv, acc_bias);
-            s += 2;
-            if (s < s_hi) {                               // a lane past its last patch keeps pointing at it
-                sc = s;
-                nw += 2;
-                while (nw >= Nw) { nw -= Nw; if (++nh == Nh) { nh = 0; ++a; } }
-            }
         }
     }
 #pragma unroll
