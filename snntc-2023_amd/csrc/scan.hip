@@ -1099,32 +1099,64 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
             if (__builtin_amdgcn_ballot_w64(any_armed) == 0) break;
         }
 
-        // Whatever is left of a row -- fewer than eight inputs behind the full chunks, as a rule -- step by
-        // step, then the output.
+        // Whatever is left of a row -- fewer than eight inputs behind the full chunks -- step by step,
+        // then the output.  The leftover entries and their weights are fetched in one go for the
+        // lane's CH scans (a load per step would put a memory round trip into every one of them); rows
+        // are padded beyond their length, so the eight entries from n_full on can always be read.
+        LaneState st[CH];
+        int kc[CH];
+        bool still[CH], any_left = false;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            st[c].wsum = wsum[c]; st[c].ysum = ysum[c]; st[c].wa = fabsf(wsum[c]);
+            st[c].ya = wsum[c] < 0.0f ? -ysum[c] : ysum[c];
+            st[c].fired = fired_cur[c];
+            kc[c] = kcur[c];
+            still[c] = live[c] && !fin[c];
+            any_left |= still[c] && kc[c] < n_seg;
+        }
+        if (__builtin_amdgcn_ballot_w64(any_left) != 0) {
+            Chunk tc;
+            load_chunk_flat(tc, xs, pr, n_full < n_seg ? n_full : 0);
+            float tw[CH][CHUNK];
+#pragma unroll
+            for (int c = 0; c < CH; ++c)
+#pragma unroll
+                for (int u = 0; u < CHUNK; ++u) tw[c][u] = wcol[tc.p[u] * COLS + c];
+#pragma unroll
+            for (int u = 0; u < CHUNK - 1; ++u) {
+                bool any_step = false;
+#pragma unroll
+                for (int c = 0; c < CH; ++c) {
+                    const bool step = still[c] && kc[c] == n_full + u && n_full + u < n_seg;
+                    if (step) {
+                        still[c] = scan_step(st[c], tc.x[u], tw[c][u]);
+                        if (still[c]) ++kc[c];
+                    }
+                    any_step |= step;
+                }
+                if (__builtin_amdgcn_ballot_w64(any_step) == 0) break;
+            }
+        }
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
             if (!live[c]) continue;
-            LaneState st;
-            st.wsum = wsum[c]; st.ysum = ysum[c]; st.wa = fabsf(wsum[c]);
-            st.ya = wsum[c] < 0.0f ? -ysum[c] : ysum[c];
-            int kc = kcur[c];
-            st.fired = fired_cur[c];
-            bool still = !fin[c];
-            for (int k = kc; k < n_seg && still; ++k) {
-                still = scan_step(st, xs[k], wcol[pr[k] * COLS + c]);
-                if (still) ++kc;
+            // (a scan that stands before the full chunks' end here does not occur; it would be walked like this)
+            for (int k = kc[c]; k < n_seg && still[c]; ++k) {
+                still[c] = scan_step(st[c], xs[k], wcol[pr[k] * COLS + c]);
+                if (still[c]) ++kc[c];
             }
             float y = np.max_time, r = 0.0f;
-            if (st.fired) {
-                r = 1.0f / st.wsum;
-                y = st.ysum * r;
+            if (st[c].fired) {
+                r = 1.0f / st[c].wsum;
+                y = st[c].ysum * r;
                 if (y >= np.max_time) { y = np.max_time; r = 0.0f; }
             }
             const size_t o = (size_t)seg * J + j + c;
             y_out[o] = y;
             rcp_out[o] = r;
             if (copy.dst) copy.dst[time_copy_pixel(copy, seg) * J + j + c] = y;
-            if (WANT_K) k_out[o] = (st.fired && r != 0.0f) ? kc : -1;
+            if (WANT_K) k_out[o] = (st[c].fired && r != 0.0f) ? kc[c] : -1;
         }
     }
 }
