@@ -1063,6 +1063,7 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
                 any_armed |= armed[c];
             }
             if (__builtin_amdgcn_ballot_w64(any_need) != 0) {
+                int round = 0;
                 do {
                     // (fetched on demand: a second round is rare, requesting its entries ahead of time
                     // would cost every item eight more loads per scan)
@@ -1077,11 +1078,37 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
                             pw[u] = wcol[pc[c].p[u] * COLS + c];
                             px[u] = pc[c].x[u];
                         }
+                        // Later rounds are for the rare scan that missed its close by a rounding: weight
+                        // sum positive, not fired (D < 0).  It cannot fire, let alone close, before the
+                        // weight sum has been negative long enough for D to come back up to zero, and it
+                        // walks on here, a chunk per round, usually in a wavefront that is alone by then.
+                        // While every scan of the round is in that state, a chunk is only accumulated and
+                        // bounded: with all t = ysum - x*wsum below -thr (the fast loop's margin) and all
+                        // weight sums positive, the reference's `fired` test is false after each of the
+                        // eight inputs, and that is all it evaluates for a scan that has not fired.
+                        bool walked = false;
+                        if (round > 0) {
+                            const bool stuck = need[c] && !fired_cur[c] && wsum[c] > 0.0f && px[0] >= 0.0f;
+                            if (__builtin_amdgcn_ballot_w64(need[c] && !stuck) == 0) {
+                                float wb = wsum[c], yb = ysum[c], tmax = -INFINITY, wmin = INFINITY;
+#pragma unroll
+                                for (int u = 0; u < CHUNK; ++u) {
+                                    wb += pw[u];
+                                    yb = __fmaf_rn(px[u], pw[u], yb);
+                                    tmax = fmaxf(tmax, __fmaf_rn(-px[u], wb, yb));
+                                    wmin = fminf(wmin, wb);
+                                }
+                                const float thr = __fmaf_rn(FILTER_REL, fabsf(yb), px[CHUNK - 1] * thr_w);
+                                walked = stuck && tmax < -thr && wmin > 0.0f;
+                                wsum[c] = walked ? wb : wsum[c];
+                                ysum[c] = walked ? yb : ysum[c];
+                            }
+                        }
                         float ya = wsum[c] < 0.0f ? -ysum[c] : ysum[c];
                         float yg = fired_cur[c] ? ya : INFINITY;
                         uint64_t exited = 0;
-                        int kc = kcur[c];
-                        const uint64_t run = __builtin_amdgcn_ballot_w64(need[c]);
+                        int kc = kcur[c] + (walked ? CHUNK : 0);
+                        const uint64_t run = __builtin_amdgcn_ballot_w64(need[c] && !walked);
                         if (run != 0) scan_chunk_vector<true>(wsum[c], ysum[c], ya, yg, kc, exited, run, px, pw);
                         const bool closed_here = (exited >> lane) & 1;
                         kcur[c] = kc;                       // inputs consumed
@@ -1094,6 +1121,7 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
                         need[c] = more && !plain;
                         any_need |= need[c];
                     }
+                    ++round;
                 } while (__builtin_amdgcn_ballot_w64(any_need) != 0);
             }
             if (__builtin_amdgcn_ballot_w64(any_armed) == 0) break;
