@@ -469,86 +469,144 @@ scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ pe
 }
 
 // Launches of a few dozen work items (the 10-wide head of a classifier): one item per workgroup,
-// its four wavefronts sharing the item instead of taking one each.  The running sums of a scan are
-// inherently sequential, its tests are not.  Wavefront 0 (the producer) only accumulates: two
-// instructions per input, and after every chunk of eight it leaves the sums in LDS and advances a
-// progress counter.  Wavefronts 1..3 (the testers) take every third chunk: they wait for the sums
-// before their chunk, recompute the fired state from them and the last input before the chunk, and
-// run the ordinary eight-step block with all its tests.  Each tester records the first close it
-// sees; the earliest of all is the scan's (a close found in a chunk is exact as long as no earlier
-// step closed, and an earlier close wins the minimum anyway).  The producer walks the trailing
-// inputs (fewer than eight) and supplies the result of a scan that never closes.
-// The item's sorted rows and row indices are copied into LDS first: at this pace chunks fetched
-// from memory a few ahead would not cover the memory latency.
-constexpr int SPLIT_WAVES = 4, SPLIT_TESTERS = SPLIT_WAVES - 1;
+// its wavefronts sharing the item instead of taking one each.  The running sums of a scan are
+// inherently sequential, its tests are not, and a lone wavefront pays about five clocks for every
+// instruction it issues, whatever the instruction.  So the sequential part is stripped to the two
+// additions per input and the reads that feed them:
+//   * before the scan all wavefronts gather the item's weights in scan order, w[lane][k] =
+//     W[perm[seg][k]][j], straight from memory into LDS (every entry is independent), next to the
+//     sorted rows; the scans then read times and weights as 16-byte runs with no address
+//     arithmetic, and the row indices never enter LDS;
+//   * wavefront 0 (the producer) only accumulates; after every chunk of eight inputs it leaves
+//     the sums in LDS and advances a progress counter.  While every scan of the item still has a
+//     full round of four chunks ahead no lane is masked and nothing is compared;
+//   * the testers take every SPLIT_TESTERS-th chunk: they wait for the sums before their chunk,
+//     recompute the fired state from them and the last input before the chunk, and run the ordinary
+//     eight-step block with all its tests.  Each tester records the first close it sees; the
+//     earliest of all is the scan's (a close found in a chunk is exact as long as no earlier step
+//     closed, and an earlier close wins the minimum anyway).  The producer walks the trailing
+//     inputs (fewer than eight) and supplies the result of a scan that never closes.
+// An item is SPLIT lanes wide: 32 lanes (the upper half of the wavefronts mirrors the lower) keep
+// the gathered weights of rows of 800 inputs within LDS; 64-column slices use all 64.
+constexpr int SPLIT_WAVES = 8;
+// Wavefronts are handed to the four SIMDs of a CU in turn: wavefront 4 would share the producer's and
+// sits the scan out, so the producer has its SIMD to itself and the testers run two to a SIMD.
+constexpr int SPLIT_IDLE_WAVE = 4, SPLIT_TESTERS = SPLIT_WAVES - 2;
+constexpr int SPLIT_THREADS = SPLIT_WAVES * kWave;
 constexpr int SPLIT_STATIC_LDS = 3 * SPLIT_WAVES * kWave * 4 + 16;
 constexpr int SPLIT_SPIN_LIMIT = 1 << 20;                  // polls of the progress counter before a tester gives up
+constexpr int SPLIT_PAD = 4;                               // floats between the weight rows of two lanes: the 16-byte
+                                                           // reads of eight neighbouring lanes fall on distinct banks
+constexpr int SPLIT_ROUND = 4;                             // chunks per round of the producer
+constexpr int split_lanes(int cols) { return cols == 64 ? 64 : 32; }
 
-// dynamic LDS of the split kernel: weight slice, rows, sums after every chunk
-__host__ __device__ inline size_t split_lds_bytes(size_t slice_bytes, int segs, int stride) {
-    return slice_bytes + (size_t)segs * stride * 8 + (size_t)(stride / CHUNK) * 2 * kWave * 4;
+// dynamic LDS of the split kernel: gathered weights [lanes][stride + pad], sorted rows [segs][stride],
+// sums after every chunk [chunks + round][2][lanes].  Reads run up to a round past the end of a row
+// (into whatever follows, never used); the sums behind the rows keep them inside the allocation.
+__host__ __device__ inline size_t split_lds_bytes(int lanes, int segs, int stride) {
+    return ((size_t)lanes * (stride + SPLIT_PAD) + (size_t)segs * stride +
+            (size_t)(stride / CHUNK + SPLIT_ROUND) * 2 * lanes) * sizeof(float);
 }
 
 template <int COLS, bool WANT_K>
-__global__ void __launch_bounds__(LOW_LATENCY_THREADS)
+__global__ void __launch_bounds__(SPLIT_THREADS)
 scan_lds_split_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ perm,
                       const int32_t* __restrict__ n_real, const float* __restrict__ w, float* __restrict__ y_out,
                       float* __restrict__ rcp_out, int32_t* __restrict__ k_out, int S, int I, int stride, int J,
                       int n_slices, int n_groups, NeuronParams np, TimeCopy copy) {
-    extern __shared__ __align__(16) float wl[];                          // [I + bias][COLS], rows, sums
+    extern __shared__ __align__(16) float wg[];            // [LANES][stride + SPLIT_PAD], rows, sums
     __shared__ int k_found[SPLIT_WAVES][kWave];
     __shared__ float w_found[SPLIT_WAVES][kWave], y_found[SPLIT_WAVES][kWave];
     __shared__ int progress;                               // chunks whose sums are in LDS
-    constexpr int SEGS = kWave / COLS;
+    constexpr int LANES = split_lanes(COLS), SEGS = LANES / COLS;
     constexpr int NONE = 0x7fffffff;
     const int block = xcd_contiguous(blockIdx.x, gridDim.x);
     const int slice = block / n_groups;
     const int group = block - slice * n_groups;
     const int j0 = slice * COLS;
-    const int rows = I + np.bias;
-    float* __restrict__ xrows = wl + rows * COLS;          // [SEGS][stride]
-    int32_t* __restrict__ prows = reinterpret_cast<int32_t*>(xrows + SEGS * stride);
-    float* __restrict__ sums = reinterpret_cast<float*>(prows + SEGS * stride);   // [chunk][wsum|ysum][lane]
-
-    fill_weight_slice<COLS>(wl, w, rows, J, j0);
+    const int wstride = stride + SPLIT_PAD;
+    float* __restrict__ xrows = wg + LANES * wstride;      // [SEGS][stride]
+    float* sums = xrows + SEGS * stride;                   // [chunk][wsum|ysum][LANES]
 
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    const int sub = lane / COLS, col = lane - sub * COLS;
+    const int la = lane % LANES;                           // lanes past LANES mirror the lower ones
+    const int sub = la / COLS, col = la - sub * COLS;
     const int j = j0 + col;
-    const float* __restrict__ wcol = wl + col;
-    const int last_chunk = stride - CHUNK;
+    const float* __restrict__ wrow = wg + la * wstride;
+    const float w_bias = np.bias && j < J ? w[(size_t)I * J + j] : 0.0f;
 
     for (int item = group; item * SEGS < S; item += n_groups) {
         const int seg0 = item * SEGS;
         const int n_segs = S - seg0 < SEGS ? S - seg0 : SEGS;
-        {
-            const float4* __restrict__ gx = reinterpret_cast<const float4*>(sorted + (size_t)seg0 * stride);
-            const int4* __restrict__ gp = reinterpret_cast<const int4*>(perm + (size_t)seg0 * stride);
-            const int n4 = n_segs * stride / 4;            // stride is a multiple of 16 entries
-            for (int e = threadIdx.x; e < n4; e += blockDim.x) {
-                reinterpret_cast<float4*>(xrows)[e] = gx[e];
-                reinterpret_cast<int4*>(prows)[e] = gp[e];
-            }
-            if (threadIdx.x == 0) progress = 0;
-        }
-        __syncthreads();                                    // rows (and, the first time, the weights) are in place
-
         const int seg_raw = seg0 + sub;
-        const bool live = seg_raw < S && j < J;
+        // mirror lanes scan along with the lane they mirror (same inputs, same sums, stored to the
+        // same place) and only stay out of the output
+        const bool scans = seg_raw < S && j < J;
+        const bool live = scans && lane < LANES;
         const int seg = seg_raw < S ? seg_raw : S - 1;
         const int row = seg - seg0;                         // idle lanes shadow the item's last segment
         const float* __restrict__ xs = xrows + row * stride;
-        const int32_t* __restrict__ pr = prows + row * stride;
-        const int n = live ? n_real[seg] : 0;
+        const int n = scans ? n_real[seg] : 0;              // (requested before the rows: one round trip less)
+        {
+            // Weights in scan order: a thread keeps its column and takes four consecutive entries of a
+            // row at a time (one 16-byte read of row indices, four weights, one 16-byte LDS write);
+            // COLS neighbours read one row of W together.  All row indices of a thread are requested
+            // first, then the sorted rows, then all its weights: two memory round trips for the usual
+            // item.  (Offsets into W as 24-bit multiply-adds: the launcher checks that rows and row
+            // pitch allow it.  Groups past the end repeat the last one.)
+            constexpr int KSTEP = SPLIT_THREADS / COLS, GB = 13;
+            const int gc = threadIdx.x % COLS, gk = threadIdx.x / COLS;
+            const bool col_live = j0 + gc < J;
+            const int groups = n_segs * stride / 4;        // stride is a multiple of 16 entries
+            const int4* __restrict__ gp = reinterpret_cast<const int4*>(perm + (size_t)seg0 * stride);
+            const __amdgpu_buffer_rsrc_t wbuf = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<float*>(w), 0, (int)((size_t)(I + np.bias) * J * sizeof(float)), 0x00020000);
+            const unsigned pitch = (unsigned)J * 4u, col_bytes = (unsigned)(j0 + gc) * 4u;
+            const int seg_skip = COLS * wstride - stride;  // from entry k of a column to entry k of the next segment
+            float* __restrict__ wcol = wg + gc * wstride;
+            auto weight = [&](int32_t r) {
+                return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                     wbuf, __umul24((unsigned)r, pitch) + col_bytes, 0, 0));
+            };
+            int4 pv[GB];
+            auto request_rows = [&](int g0) {
+#pragma unroll
+                for (int t = 0; t < GB; ++t) pv[t] = gp[min(g0 + t * KSTEP, groups - 1)];
+            };
+            request_rows(gk);
+            __builtin_amdgcn_sched_barrier(0);
+            const float4* __restrict__ gx = reinterpret_cast<const float4*>(sorted + (size_t)seg0 * stride);
+            for (int e = threadIdx.x; e < groups; e += SPLIT_THREADS) reinterpret_cast<float4*>(xrows)[e] = gx[e];
+            for (int g0 = gk;;) {
+                float4 wv[GB];
+#pragma unroll
+                for (int t = 0; t < GB; ++t)
+                    wv[t] = col_live ? make_float4(weight(pv[t].x), weight(pv[t].y), weight(pv[t].z), weight(pv[t].w))
+                                     : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+                for (int t = 0; t < GB; ++t) {
+                    const int f = 4 * min(g0 + t * KSTEP, groups - 1);
+                    int sl = 0;
+#pragma unroll
+                    for (int q = 1; q < SEGS; ++q) sl += f >= q * stride;
+                    *reinterpret_cast<float4*>(wcol + f + sl * seg_skip) = wv[t];
+                }
+                g0 += GB * KSTEP;
+                if (g0 >= groups) break;
+                request_rows(g0);
+            }
+            if (threadIdx.x == 0) progress = 0;
+        }
+        __syncthreads();                                    // rows and weights are in place
+
         const int n_full = n & ~(CHUNK - 1);
 
         float wsum = -np.theta, ysum = 0.0f, ya = 0.0f;
         bool fired0 = false;
         if (np.bias) {
-            const float wb = wcol[I * COLS];
-            wsum += wb;
-            ysum = np.biasvolt * wb;
+            wsum += w_bias;
+            ysum = np.biasvolt * w_bias;
             ya = wsum < 0.0f ? -ysum : ysum;
             fired0 = ya > fabsf(wsum) * np.biasvolt;
         }
@@ -557,59 +615,80 @@ scan_lds_split_kernel(const float* __restrict__ sorted, const int32_t* __restric
 
         if (wave == 0) {
             // ---- producer -----------------------------------------------------------------------
-            int kcnt = 0;
-            // chunk c is consumed from xp[c % NBUF] / wv[c % 2]; after it, chunk c+NBUF is read into its
-            // place and the weights of chunk c+2 are fetched
-            constexpr int NBUF = 4;
-            Chunk xp[NBUF];
-            float wv[2][CHUNK];
+            // chunk c is consumed from buf[c % NBUF]; after it, chunk c + NBUF is read into its place
+            constexpr int NBUF = SPLIT_ROUND;
+            float bx[NBUF][CHUNK], bw[NBUF][CHUNK];
+            auto fetch = [&](float (&x)[CHUNK], float (&wv)[CHUNK], int k) {
+                const float4 x0 = *reinterpret_cast<const float4*>(xs + k), x1 = *reinterpret_cast<const float4*>(xs + k + 4);
+                const float4 w0 = *reinterpret_cast<const float4*>(wrow + k), w1 = *reinterpret_cast<const float4*>(wrow + k + 4);
+                x[0] = x0.x; x[1] = x0.y; x[2] = x0.z; x[3] = x0.w; x[4] = x1.x; x[5] = x1.y; x[6] = x1.z; x[7] = x1.w;
+                wv[0] = w0.x; wv[1] = w0.y; wv[2] = w0.z; wv[3] = w0.w; wv[4] = w1.x; wv[5] = w1.y; wv[6] = w1.z; wv[7] = w1.w;
+            };
 #pragma unroll
-            for (int b = 0; b < NBUF; ++b) load_chunk_flat(xp[b], xs, pr, b * CHUNK <= last_chunk ? b * CHUNK : 0);
+            for (int b = 0; b < NBUF; ++b) fetch(bx[b], bw[b], b * CHUNK);
+            // chunks of this item: the longest row decides the counter's final value, the shortest how
+            // long no lane needs a mask
+            int n_full_max = n_full, n_full_min = scans ? n_full : NONE;
 #pragma unroll
-            for (int b = 0; b < 2; ++b)
+            for (int d = kWave / 2; d > 0; d >>= 1) {
+                n_full_max = max(n_full_max, __shfl_xor(n_full_max, d, kWave));
+                n_full_min = min(n_full_min, __shfl_xor(n_full_min, d, kWave));
+            }
+            n_full_max = __builtin_amdgcn_readfirstlane(n_full_max);
+            n_full_min = __builtin_amdgcn_readfirstlane(n_full_min);
+            // Order inside a phase: accumulate, store the sums, move the counter to the chunks before
+            // this one, then issue the reads for a later chunk.  The counter is a relaxed store and is
+            // not waited for: LDS serves a wavefront's requests in order, so the sums it covers, stored
+            // a phase earlier, are in place before it.  Nothing moves across a phase boundary (the
+            // compiler would otherwise wait for every outstanding request before each accumulation).
+            auto publish = [&](int k) {
+                asm volatile("" ::: "memory");
+                float* out = sums + (k / CHUNK) * 2 * LANES;
+                out[la] = wsum;
+                out[LANES + la] = ysum;
+                asm volatile("" ::: "memory");
+                __hip_atomic_store(&progress, k / CHUNK, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                asm volatile("" ::: "memory");
+            };
+            int k0 = 0;
+            for (; k0 + NBUF * CHUNK <= n_full_min; k0 += NBUF * CHUNK) {
 #pragma unroll
-                for (int u = 0; u < CHUNK; ++u) wv[b][u] = wcol[xp[b].p[u] * COLS];
-            // chunks of this item (the longest row decides): the counter's final value
-            int n_full_max = n_full;
+                for (int ph = 0; ph < NBUF; ++ph) {
+                    const int k = k0 + ph * CHUNK;
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int d = kWave / 2; d > 0; d >>= 1) n_full_max = max(n_full_max, __shfl_xor(n_full_max, d, kWave));
-            // Order inside a phase: accumulate, store the sums, then issue the LDS reads for later
-            // chunks.  The counter is moved two phases late and without waiting: LDS serves a
-            // wavefront's requests in order, and the weights the accumulation of chunk c consumes were
-            // requested right after the sums of chunk c-2 were stored -- once they have arrived,
-            // those sums are in place.
-            for (int k0 = 0;; k0 += NBUF * CHUNK) {
-                bool stop = false;
+                    for (int u = 0; u < CHUNK; ++u) {
+                        wsum += bw[ph][u];
+                        ysum = __fmaf_rn(bx[ph][u], bw[ph][u], ysum);
+                    }
+                    publish(k);
+                    fetch(bx[ph], bw[ph], k + NBUF * CHUNK);
+                }
+            }
+            for (; k0 < n_full_max; k0 += NBUF * CHUNK) {
 #pragma unroll
                 for (int ph = 0; ph < NBUF; ++ph) {
                     const int k = k0 + ph * CHUNK;
                     const uint64_t run = __ballot(k < n_full);
-                    if (run == 0) { stop = true; break; }
-                    accumulate_chunk(wsum, ysum, kcnt, run, xp[ph % NBUF].x, wv[ph % 2]);
-                    asm volatile("" ::: "memory");
-                    if (k >= 2 * CHUNK) __hip_atomic_store(&progress, k / CHUNK - 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                    float* __restrict__ out = sums + (size_t)(k / CHUNK) * 2 * kWave;
-                    out[lane] = wsum;
-                    out[kWave + lane] = ysum;
-                    asm volatile("" ::: "memory");
-                    const int kn = k + NBUF * CHUNK;
-                    load_chunk_flat(xp[ph % NBUF], xs, pr, kn <= last_chunk ? kn : 0);
-#pragma unroll
-                    for (int u = 0; u < CHUNK; ++u) wv[ph % 2][u] = wcol[xp[(ph + 2) % NBUF].p[u] * COLS];
+                    int unused = 0;
+                    __builtin_amdgcn_sched_barrier(0);
+                    accumulate_chunk(wsum, ysum, unused, run, bx[ph], bw[ph]);
+                    publish(k);
+                    fetch(bx[ph], bw[ph], k + NBUF * CHUNK);
                 }
-                if (stop) break;
             }
             // the last chunk's sums: wait for them, then let the counter reach its final value
             __hip_atomic_store(&progress, (n_full_max + CHUNK - 1) / CHUNK, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
             // the trailing inputs, for a scan that no tester closes
-            if (live) {
+            int kcnt = n_full;
+            if (scans) {
                 LaneState st;
                 st.wsum = wsum; st.ysum = ysum; st.wa = fabsf(wsum);
                 st.ya = wsum < 0.0f ? -ysum : ysum;
                 st.fired = n_full > 0 ? st.ya > xs[n_full - 1] * st.wa : fired0;
                 bool open = true;
                 for (int k = n_full; k < n && open; ++k) {
-                    open = scan_step(st, xs[k], wcol[pr[k] * COLS]);
+                    open = scan_step(st, xs[k], wrow[k]);
                     if (open) ++kcnt;
                 }
                 if (!open) k_close = kcnt;
@@ -620,47 +699,61 @@ scan_lds_split_kernel(const float* __restrict__ sorted, const int32_t* __restric
             w_found[0][lane] = wsum;
             y_found[0][lane] = ysum;
             consumed = kcnt;                                // all n inputs when nothing closed
+        } else if (wave == SPLIT_IDLE_WAVE) {
+            k_found[wave][lane] = NONE;
+            w_found[wave][lane] = 0.0f;
+            y_found[wave][lane] = 0.0f;
         } else {
-            // ---- tester: chunks wave-1, wave-1+3, ... ---------------------------------------------
+            // ---- tester t of SPLIT_TESTERS: chunks t, t + SPLIT_TESTERS, ... --------------------------
             uint64_t closed = 0;
             float w_close = 0.0f, y_close = 0.0f;
             float yg = fired0 ? ya : INFINITY;
-            Chunk cur, nxt;
-            float wcur[CHUNK];
-            int c = wave - 1;
-            load_chunk_flat(cur, xs, pr, c * CHUNK <= last_chunk ? c * CHUNK : 0);
-#pragma unroll
-            for (int u = 0; u < CHUNK; ++u) wcur[u] = wcol[cur.p[u] * COLS];
+            float xc[CHUNK], wc[CHUNK], xn[CHUNK], wn[CHUNK];
+            auto fetch = [&](float (&x)[CHUNK], float (&wv)[CHUNK], int k) {
+                const float4 x0 = *reinterpret_cast<const float4*>(xs + k), x1 = *reinterpret_cast<const float4*>(xs + k + 4);
+                const float4 w0 = *reinterpret_cast<const float4*>(wrow + k), w1 = *reinterpret_cast<const float4*>(wrow + k + 4);
+                x[0] = x0.x; x[1] = x0.y; x[2] = x0.z; x[3] = x0.w; x[4] = x1.x; x[5] = x1.y; x[6] = x1.z; x[7] = x1.w;
+                wv[0] = w0.x; wv[1] = w0.y; wv[2] = w0.z; wv[3] = w0.w; wv[4] = w1.x; wv[5] = w1.y; wv[6] = w1.z; wv[7] = w1.w;
+            };
+            int c = wave < SPLIT_IDLE_WAVE ? wave - 1 : wave - 2;
+            const int last_chunk = stride - CHUNK;
+            fetch(xc, wc, c * CHUNK <= last_chunk ? c * CHUNK : 0);
             for (;; c += SPLIT_TESTERS) {
                 const int k = c * CHUNK;
                 const uint64_t run = __ballot(k < n_full) & ~closed;
                 if (run == 0) break;                        // every lane closed here or past its inputs
                 const int kn = k + SPLIT_TESTERS * CHUNK;
-                load_chunk_flat(nxt, xs, pr, kn <= last_chunk ? kn : 0);
+                fetch(xn, wn, kn <= last_chunk ? kn : 0);
                 if (c > 0) {
-                    // bounded wait: if the sums never arrive the tester goes on with what is there and
-                    // the result is marked invalid (no early exit: every wavefront reaches the barriers)
+                    // Bounded wait: if the sums never arrive the tester goes on with what is there and
+                    // the result is marked invalid (no early exit: every wavefront reaches the barriers).
+                    // The counter and the sums are requested together and waited for once: LDS serves
+                    // a wavefront's requests in order, so sums read after a counter that had reached c
+                    // are the finished ones; a poll that came too early is repeated as a whole.
                     int spins = 0;
-                    while (__builtin_amdgcn_readfirstlane(__hip_atomic_load(&progress, __ATOMIC_ACQUIRE,
-                                                                            __HIP_MEMORY_SCOPE_WORKGROUP)) < c &&
-                           spins < SPLIT_SPIN_LIMIT) {
+                    const float* in = sums + (c - 1) * 2 * LANES;
+                    float x_prev;
+                    for (;;) {
+                        const int seen = __hip_atomic_load(&progress, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        asm volatile("" ::: "memory");
+                        wsum = in[la];
+                        ysum = in[LANES + la];
+                        x_prev = xs[k - 1];
+                        asm volatile("" ::: "memory");
+                        if (__builtin_amdgcn_readfirstlane(seen) >= c || spins >= SPLIT_SPIN_LIMIT) break;
                         __builtin_amdgcn_s_sleep(1);
                         ++spins;
                     }
                     failed |= spins >= SPLIT_SPIN_LIMIT;
-                    const float* __restrict__ in = sums + (size_t)(c - 1) * 2 * kWave;
-                    wsum = in[lane];
-                    ysum = in[kWave + lane];
                     ya = wsum < 0.0f ? -ysum : ysum;        // fired state after input k-1, from the sums
-                    yg = ya > xs[k - 1] * fabsf(wsum) ? ya : INFINITY;
+                    yg = ya > x_prev * fabsf(wsum) ? ya : INFINITY;
                 }
                 const uint64_t before = closed;
                 int kc = k;
-                scan_chunk_vector<true>(wsum, ysum, ya, yg, kc, closed, run, cur.x, wcur);
+                scan_chunk_vector<true>(wsum, ysum, ya, yg, kc, closed, run, xc, wc);
                 if (((closed & ~before) >> lane) & 1) { k_close = kc; w_close = wsum; y_close = ysum; }
 #pragma unroll
-                for (int u = 0; u < CHUNK; ++u) wcur[u] = wcol[nxt.p[u] * COLS];
-                cur = nxt;
+                for (int u = 0; u < CHUNK; ++u) { xc[u] = xn[u]; wc[u] = wn[u]; }
             }
             k_found[wave][lane] = failed ? -1 : k_close;    // -1 poisons the result below
             w_found[wave][lane] = w_close;
@@ -1283,16 +1376,20 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     constexpr int CH = filter_ch(COLS);
     const int64_t multi_items = (S + CH * SEGS - 1) / (CH * SEGS);
     const bool multi = !low_latency && multi_items * n_slices >= (int64_t)cus * 4 * 4;
-    const int64_t work_items = multi ? multi_items : items;
     if (multi) {
         const int64_t per_wg = (multi_items * n_slices + capacity - 1) / capacity;
         WAVES = (int)(per_wg >= 16 ? 16 : (per_wg + 3) / 4 * 4);
     }
     // Fewer items than CUs: a whole workgroup per item, its wavefronts sharing the item's tests.
-    const size_t split_lds = split_lds_bytes(lds_bytes, SEGS, (int)stride);
-    const bool split = low_latency && items * n_slices <= (int64_t)cus && I >= 2 * CHUNK * SPLIT_WAVES &&
-                       split_lds + SPLIT_STATIC_LDS <= (size_t)LDS_SCAN_BYTES;
+    constexpr int SPLIT_SEGS = split_lanes(COLS) / COLS;
+    const int64_t split_items = (S + SPLIT_SEGS - 1) / SPLIT_SEGS;
+    const size_t split_lds = split_lds_bytes(split_lanes(COLS), SPLIT_SEGS, (int)stride);
+    const bool split = low_latency && split_items * n_slices <= (int64_t)cus && I >= 2 * CHUNK * SPLIT_WAVES &&
+                       split_lds + SPLIT_STATIC_LDS <= (size_t)LDS_SCAN_BYTES &&
+                       // the gather addresses W by 24-bit multiplies and a 32-bit byte offset
+                       I + np.bias < (1 << 24) && J < (1 << 22) && (I + np.bias) * J * 4 < 0x7fffffffLL;
     if (split) WAVES = 1;                                   // items per workgroup pass
+    const int64_t work_items = split ? split_items : multi ? multi_items : items;
     const bool filt = !(split || low_latency);
     if (filt) {
         // the chunk buffers of the wavefronts share the LDS with the slice: fewer wavefronts where it is tight
@@ -1308,7 +1405,7 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
                   : split ? scan_lds_split_kernel<COLS, true> : scan_lds_kernel<COLS, true>;
     auto kern = filt ? (multi ? scan_filter_kernel<COLS, CH, false> : scan_filter_kernel<COLS, 1, false>)
                 : split ? scan_lds_split_kernel<COLS, false> : scan_lds_kernel<COLS, false>;
-    dim3 grid((unsigned)(n_slices * n_groups)), block((unsigned)((split && !filt) ? LOW_LATENCY_THREADS : WAVES * kWave));
+    dim3 grid((unsigned)(n_slices * n_groups)), block((unsigned)((split && !filt) ? SPLIT_THREADS : WAVES * kWave));
     {
         KernelTimerScope timer_("scan", stream);
         const size_t dyn_lds = filt ? lds_bytes + filter_extra_lds(COLS, multi ? CH : 1, WAVES) : split ? split_lds : lds_bytes;

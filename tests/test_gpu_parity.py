@@ -350,6 +350,10 @@ HEAD_CASES = [
     (22, 33, 2048, 5, True),
     (23, 130, 264, 16, True),      # J equal to the slice width (vector weight copy)
     (24, 6, 72, 3, True),
+    (25, 40, 300, 5, True),        # 8-column slice: four samples per work item
+    (26, 50, 200, 24, False),      # 32-column slice
+    (27, 20, 136, 40, True),       # 64-column slice, rows barely long enough to be shared
+    (28, 100, 264, 70, True),      # two column slices, the second mostly empty
 ]
 
 
