@@ -480,7 +480,7 @@ scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ pe
 //   * wavefront 0 (the producer) only accumulates; after every chunk of eight inputs it leaves
 //     the sums in LDS and advances a progress counter.  While every scan of the item still has a
 //     full round of four chunks ahead no lane is masked and nothing is compared;
-//   * the testers take every SPLIT_TESTERS-th chunk: they wait for the sums before their chunk,
+//   * the other wavefronts (the testers) take every SPLIT_TESTERS-th chunk: they wait for the sums before their chunk,
 //     recompute the fired state from them and the last input before the chunk, and run the ordinary
 //     eight-step block with all its tests.  Each tester records the first close it sees; the
 //     earliest of all is the scan's (a close found in a chunk is exact as long as no earlier step
@@ -488,10 +488,9 @@ scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ pe
 //     inputs (fewer than eight) and supplies the result of a scan that never closes.
 // An item is SPLIT lanes wide: 32 lanes (the upper half of the wavefronts mirrors the lower) keep
 // the gathered weights of rows of 800 inputs within LDS; 64-column slices use all 64.
-constexpr int SPLIT_WAVES = 8;
-// Wavefronts are handed to the four SIMDs of a CU in turn: wavefront 4 would share the producer's and
-// sits the scan out, so the producer has its SIMD to itself and the testers run two to a SIMD.
-constexpr int SPLIT_IDLE_WAVE = 4, SPLIT_TESTERS = SPLIT_WAVES - 2;
+// (Seven testers: leaving the wavefront that shares the producer's SIMD idle, or 11 or 15 testers,
+// measured no faster.)
+constexpr int SPLIT_WAVES = 8, SPLIT_TESTERS = SPLIT_WAVES - 1;
 constexpr int SPLIT_THREADS = SPLIT_WAVES * kWave;
 constexpr int SPLIT_STATIC_LDS = 3 * SPLIT_WAVES * kWave * 4 + 16;
 constexpr int SPLIT_SPIN_LIMIT = 1 << 20;                  // polls of the progress counter before a tester gives up
@@ -699,10 +698,6 @@ scan_lds_split_kernel(const float* __restrict__ sorted, const int32_t* __restric
             w_found[0][lane] = wsum;
             y_found[0][lane] = ysum;
             consumed = kcnt;                                // all n inputs when nothing closed
-        } else if (wave == SPLIT_IDLE_WAVE) {
-            k_found[wave][lane] = NONE;
-            w_found[wave][lane] = 0.0f;
-            y_found[wave][lane] = 0.0f;
         } else {
             // ---- tester t of SPLIT_TESTERS: chunks t, t + SPLIT_TESTERS, ... --------------------------
             uint64_t closed = 0;
@@ -715,7 +710,7 @@ scan_lds_split_kernel(const float* __restrict__ sorted, const int32_t* __restric
                 x[0] = x0.x; x[1] = x0.y; x[2] = x0.z; x[3] = x0.w; x[4] = x1.x; x[5] = x1.y; x[6] = x1.z; x[7] = x1.w;
                 wv[0] = w0.x; wv[1] = w0.y; wv[2] = w0.z; wv[3] = w0.w; wv[4] = w1.x; wv[5] = w1.y; wv[6] = w1.z; wv[7] = w1.w;
             };
-            int c = wave < SPLIT_IDLE_WAVE ? wave - 1 : wave - 2;
+            int c = wave - 1;
             const int last_chunk = stride - CHUNK;
             fetch(xc, wc, c * CHUNK <= last_chunk ? c * CHUNK : 0);
             for (;; c += SPLIT_TESTERS) {
