@@ -87,3 +87,45 @@ def test_random_shapes_and_parameters(seed0):
         except AssertionError as e:
             fails.append(f"case {seed0}/{case}: {desc}: {str(e)[:300]}")
     assert not fails, "\n".join(fails)
+
+
+@pytest.mark.parametrize("seed0", [21, 22])
+def test_random_classifier_heads(seed0):
+    """Layers with few work items (few outputs, moderate batch), where the wavefronts of a workgroup share
+    one scan: random row lengths 128..1000, every column-slice width, one or more slices, batches up to
+    what the kernel takes, ragged numbers of real inputs, rows without any, ties, weights of both signs,
+    columns that never fire.  y, 1/S and the causal-set sizes bit-exact, with and without the extra outputs."""
+    import snntc_amd as snn
+    n_cases, fails = 100, []
+    for case in range(n_cases):
+        rng = np.random.default_rng(seed0 * 100000 + case)
+        biasvolt = float(rng.choice([0.0, 1.0, 1.0, 0.6]))
+        theta = float(rng.choice([1.0, 1.0, 0.5, 2.0]))
+        max_time = float(rng.choice([1e5, 1e5, 30.0]))
+        I = int(rng.choice([128, 129, 136, 200, 264, 511, 512, 784, 800, 900, int(rng.integers(128, 1000))]))
+        J = int(rng.choice([1, 3, 5, 8, 9, 10, 16, 17, 24, 32, 33, 40, 64, 70, 100]))
+        cols = 64                                            # the library's slice width for this J
+        while cols > 8 and cols // 2 >= J:
+            cols //= 2
+        segs = (64 if cols == 64 else 32) // cols            # samples per work item
+        slices = (J + cols - 1) // cols
+        B = int(rng.integers(1, min(max(1, 256 // slices * segs), 300) + 1))
+        rows = I + (1 if biasvolt > 1e-8 else 0)
+        x = np.exp(1.5 * rng.random((B, I))).astype(np.float32)
+        if rng.random() < 0.3: x = (np.round(x * 4) / 4).astype(np.float32)
+        if rng.random() < 0.5: x[rng.random((B, I)) < rng.random((B, 1)) * 0.6] = np.float32(max_time)
+        if rng.random() < 0.3: x[int(rng.integers(0, B))] = np.float32(max_time)
+        w = ((3.0 / I + np.sqrt(2.0 / I) * rng.standard_normal((rows, J))) * theta * rng.choice([1.0, 0.3, 3.0])).astype(np.float32)
+        if rng.random() < 0.2: w = rng.standard_normal((rows, J)).astype(np.float32)
+        if rng.random() < 0.3: w[:, int(rng.integers(0, J))] = -np.abs(w[:, 0])
+        p = capi.fc_params(biasvolt, max_time=max_time, theta=theta)
+        ref_out, ref_k, _, _ = capi.fc_forward_dev(x, w, p, want_aux=True)
+        out, _, _, ck = snn.snnfc(t(x), t(w), p, return_aux=True)
+        out2 = snn.snnfc(t(x), t(w), p)
+        torch.cuda.synchronize()
+        out, ck, out2 = out.cpu().numpy(), ck.cpu().numpy(), out2.cpu().numpy()
+        desc = f"case {seed0}/{case}: B={B} I={I} J={J} bias={biasvolt} theta={theta} max={max_time}"
+        if not np.array_equal(ck, ref_k): fails.append(desc + ": k")
+        elif not np.array_equal(out.view(np.uint32), ref_out.view(np.uint32)): fails.append(desc + ": y/r")
+        elif not np.array_equal(out2.view(np.uint32), ref_out.view(np.uint32)): fails.append(desc + ": y/r (plain)")
+    assert not fails, "\n".join(fails)
