@@ -13,8 +13,9 @@
 //                          chunk of eight inputs proves that none of them can close the set;
 //   scan_lds_kernel        small launches (a couple of wavefronts per SIMD): weight slice in LDS, every
 //                          step with its tests, written for latency;
-//   scan_lds_split_kernel  fewer work items than CUs: one item per workgroup, its wavefronts sharing
-//                          the item's tests;
+//   scan_lds_split_kernel  fewer work items than CUs: one item per workgroup, its weights gathered
+//                          into LDS in scan order first, then one wavefront accumulating and the
+//                          others sharing the item's tests;
 //   scan_kernel            segments so long that not even eight weight columns fit in LDS: weight
 //                          rows streamed from memory, one wavefront per (segment, 64 neurons).
 // In all of them lanes run across neurons, so a weight row is read coalesced (or conflict-free from
