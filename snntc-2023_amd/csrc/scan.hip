@@ -23,6 +23,8 @@
 // (segment rows are padded to a multiple of 16 entries so that they are fetched eight at a time
 // without bounds checks).
 #include <atomic>
+#include <type_traits>
+#include <utility>
 
 #include "snntc_common.h"
 
@@ -862,15 +864,19 @@ __device__ __forceinline__ void filter_chunk(float& wsum, float& ysum, int& kfla
     }
     const float thr = __fmaf_rn(FILTER_REL, fabsf(yb), thrx);
     uint64_t stop;
+    // (two statements: the first has scalar results only, so the masks stay uniform values for the compiler
+    // also where no branch depends on them)
     asm("v_cmp_gt_f32_e32 vcc, %[m], %[thr]\n"                       // pass: false for NaN on either side
         "s_andn2_b64 %[stop], %[open], vcc\n"
         "s_and_b64 %[open], %[open], vcc\n"
-        "v_cndmask_b32_e64 %[ws], %[ws], %[wb], %[open]\n"
+        : [open] "+s"(open), [stop] "=&s"(stop)
+        : [m] "v"(m), [thr] "v"(thr)
+        : "vcc", "scc");
+    asm("v_cndmask_b32_e64 %[ws], %[ws], %[wb], %[open]\n"
         "v_cndmask_b32_e64 %[ys], %[ys], %[yb], %[open]\n"
         "v_cndmask_b32_e64 %[kf], %[kf], %[vk], %[stop]\n"
-        : [ws] "+v"(wsum), [ys] "+v"(ysum), [kf] "+v"(kflag), [open] "+s"(open), [stop] "=&s"(stop)
-        : [m] "v"(m), [thr] "v"(thr), [wb] "v"(wb), [yb] "v"(yb), [vk] "v"(k)
-        : "vcc", "scc");
+        : [ws] "+v"(wsum), [ys] "+v"(ysum), [kf] "+v"(kflag)
+        : [open] "s"(open), [stop] "s"(stop), [wb] "v"(wb), [yb] "v"(yb), [vk] "v"(k));
 }
 
 // Largest of the threads' `m` over the workgroup, the same value in every thread.  `red` is room for
@@ -914,6 +920,17 @@ __device__ __forceinline__ void quad_row_addresses(int row, unsigned base, unsig
 }
 
 typedef __attribute__((address_space(3))) const float lds_cfloat;
+
+// f(integral_constant<int, 0>), f(<1>), ... f(<N-1>) until one returns false; true if none did.  The
+// phase number reaches f as a type, so ring slots and buffers stay compile-time register choices.
+template <class F, int... PH>
+__device__ __forceinline__ bool for_each_phase_impl(F&& f, std::integer_sequence<int, PH...>) {
+    return (f(std::integral_constant<int, PH>{}) && ...);
+}
+template <int N, class F>
+__device__ __forceinline__ bool for_each_phase(F&& f) {
+    return for_each_phase_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 // Segments a wavefront of the filter kernel works on, and whether their input times go through
 // LDS: they do unless every quad has a segment of its own (then the quad broadcast is all there is
@@ -1091,14 +1108,43 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
 #pragma unroll
                 for (int b = 0; b < RING - 1; ++b) request(b, kmin + b * CHUNK);
                 weights(0, wv[0]);
+                // (every lane "uses" the first chunk's times here: otherwise the compiler moves their loads
+                // under the writers' branch of stage_times and waits for all 28 requests there)
+                if constexpr (XLDS) asm volatile("" : "+v"(rxl[0]), "+v"(rxh[0]));
                 stage_times(0, 0);
 
-                for (int k0 = kmin;; k0 += RING * CHUNK) {
-                    bool stop = false;
-                    rotate_wave_priority(k0 / (RING * CHUNK) + (wave >> 2));
+                // One phase; its number is a compile-time value.  (The phases of a round are chained by a fold
+                // expression, not by a loop with a break: behind such a loop the compiler waits in every
+                // phase for all but the last four row loads, which makes the ring one chunk deep in effect.)
+                auto phase = [&](auto ph_c, int k) {
+                    constexpr int ph = decltype(ph_c)::value;
+                    request((ph + RING - 1) % RING, k + (RING - 1) * CHUNK);
+                    weights((ph + 1) % RING, wv[(ph + 1) % 2]);
+                    stage_times((ph + 1) % RING, (ph + 1) % 2);
+                    // The requests above stay ahead of the arithmetic below: what this phase consumes
+                    // was requested a phase or more ago, and what it requests has the whole phase to
+                    // arrive.
+                    __builtin_amdgcn_sched_barrier(0);
+                    float x[CHUNK];
+                    if constexpr (XLDS) {
 #pragma unroll
-                    for (int ph = 0; ph < RING; ++ph) {
-                        const int k = k0 + ph * CHUNK;
+                        for (int u = 0; u < CHUNK; ++u) x[u] = xq[ph % 2][u];
+                    } else {
+                        const int xl = __float_as_int(rxl[ph % RING]), xh = __float_as_int(rxh[ph % RING]);
+                        x[0] = __int_as_float(quad_broadcast<0>(xl)); x[1] = __int_as_float(quad_broadcast<1>(xl));
+                        x[2] = __int_as_float(quad_broadcast<2>(xl)); x[3] = __int_as_float(quad_broadcast<3>(xl));
+                        x[4] = __int_as_float(quad_broadcast<0>(xh)); x[5] = __int_as_float(quad_broadcast<1>(xh));
+                        x[6] = __int_as_float(quad_broadcast<2>(xh)); x[7] = __int_as_float(quad_broadcast<3>(xh));
+                    }
+                    const float thrx = x[CHUNK - 1] * thr_w;
+#pragma unroll
+                    for (int c = 0; c < CH; ++c)
+                        filter_chunk(wsum[c], ysum[c], kflag[c], open[c], k, thrx, x, wv[ph % 2][c]);
+                };
+                for (int k0 = kmin;; k0 += RING * CHUNK) {
+                    rotate_wave_priority(k0 / (RING * CHUNK) + (wave >> 2));
+                    const bool stop = !for_each_phase<RING>([&](auto ph_c) {
+                        const int k = k0 + decltype(ph_c)::value * CHUNK;
                         const uint64_t inside = __builtin_amdgcn_ballot_w64(k < n_full);
                         uint64_t any = 0;
 #pragma unroll
@@ -1106,30 +1152,10 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
                             open[c] &= inside;
                             any |= open[c];
                         }
-                        if (any == 0) { stop = true; break; }
-                        request((ph + RING - 1) % RING, k + (RING - 1) * CHUNK);
-                        weights((ph + 1) % RING, wv[(ph + 1) % 2]);
-                        stage_times((ph + 1) % RING, (ph + 1) % 2);
-                        // The requests above stay ahead of the arithmetic below: what this phase consumes
-                        // was requested a phase or more ago, and what it requests has the whole phase to
-                        // arrive.
-                        __builtin_amdgcn_sched_barrier(0);
-                        float x[CHUNK];
-                        if constexpr (XLDS) {
-#pragma unroll
-                            for (int u = 0; u < CHUNK; ++u) x[u] = xq[ph % 2][u];
-                        } else {
-                            const int xl = __float_as_int(rxl[ph % RING]), xh = __float_as_int(rxh[ph % RING]);
-                            x[0] = __int_as_float(quad_broadcast<0>(xl)); x[1] = __int_as_float(quad_broadcast<1>(xl));
-                            x[2] = __int_as_float(quad_broadcast<2>(xl)); x[3] = __int_as_float(quad_broadcast<3>(xl));
-                            x[4] = __int_as_float(quad_broadcast<0>(xh)); x[5] = __int_as_float(quad_broadcast<1>(xh));
-                            x[6] = __int_as_float(quad_broadcast<2>(xh)); x[7] = __int_as_float(quad_broadcast<3>(xh));
-                        }
-                        const float thrx = x[CHUNK - 1] * thr_w;
-#pragma unroll
-                        for (int c = 0; c < CH; ++c)
-                            filter_chunk(wsum[c], ysum[c], kflag[c], open[c], k, thrx, x, wv[ph % 2][c]);
-                    }
+                        if (any == 0) return false;
+                        phase(ph_c, k);
+                        return true;
+                    });
                     if (stop) break;
                 }
 #pragma unroll
