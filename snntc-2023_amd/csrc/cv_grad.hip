@@ -136,35 +136,30 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
             for (int kc0 = ks * kc_share; kc0 < (ks + 1) * kc_share; kc0 += KCB) {
                 // stage the patch row: slots whose patch does not exist are never read
                 __builtin_amdgcn_wave_barrier();
-                // The loads of a round are issued together: one slot at a time would cost a memory
-                // latency per slot, and nothing of this wavefront overlaps with it.  A round covers
-                // STAGE * (64 / KCB) slots -- with fewer than 64 output channels per slot the lanes
-                // share out neighbouring slots -- which is the whole row for a 3-wide kernel.
-                constexpr int STAGE = 10, PER = kWave / KCB;
+                // The rows go from memory straight into LDS (buffer loads with the LDS bit: lane l of a load
+                // writes dword l behind the load's LDS base).  A load covers 64 / KCB neighbouring slots --
+                // with fewer than 64 output channels per slot the lanes share them out -- and all loads of
+                // a round are in flight together.  No registers are involved, which the compiler used to
+                // free by spilling the accumulators around this loop.
+                constexpr int PER = kWave / KCB;
                 const int sub = lane / KCB, kcl = lane - sub * KCB;
-                for (int d0 = 0; d0 < n_slots; d0 += STAGE * PER) {
-                    float yv[STAGE], uv[STAGE];
-                    bool have[STAGE];
-#pragma unroll
-                    for (int k = 0; k < STAGE; ++k) {
-                        const int d = d0 + k * PER + sub;
-                        const int ww = w0 - Kw + 1 + d;
-                        have[k] = d < n_slots && ww >= 0 && ww % Sw == 0 && ww / Sw < Nw;
-                        if (have[k]) {
-                            const size_t so = (row0 + ww / Sw) * Kc + kc0 + kcl;
-                            yv[k] = ym[so];
-                            uv[k] = upm[so];
-                        }
-                    }
-#pragma unroll
-                    for (int k = 0; k < STAGE; ++k) {
-                        if (have[k]) {
-                            const int d = d0 + k * PER + sub;
-                            ys[d * KCB + kcl] = yv[k];
-                            us[d * KCB + kcl] = uv[k];
-                        }
+                const int row_bytes = (int)(((size_t)Nw * Kc - kc0) * sizeof(float));
+                const __amdgpu_buffer_rsrc_t ybuf = __builtin_amdgcn_make_buffer_rsrc(
+                    const_cast<float*>(ym + row0 * Kc + kc0), 0, row_bytes, 0x00020000);
+                const __amdgpu_buffer_rsrc_t ubuf = __builtin_amdgcn_make_buffer_rsrc(
+                    const_cast<float*>(upm + row0 * Kc + kc0), 0, row_bytes, 0x00020000);
+                typedef __attribute__((address_space(3))) void lds_void;
+                for (int d0 = 0; d0 < n_slots; d0 += PER) {
+                    const int d = d0 + sub;
+                    const int ww = w0 - Kw + 1 + d;
+                    const int col = Sw == 1 ? ww : ww / Sw;
+                    if (d < n_slots && ww >= 0 && (Sw == 1 || ww % Sw == 0) && col < Nw) {
+                        const int so = (col * Kc + kcl) * (int)sizeof(float);
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(ybuf, (lds_void*)(ys + d0 * KCB), 4, so, 0, 0, 0);
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(ubuf, (lds_void*)(us + d0 * KCB), 4, so, 0, 0, 0);
                     }
                 }
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
                 __builtin_amdgcn_wave_barrier();
                 for (int kw = 0; kw < Kw; ++kw) {
@@ -477,7 +472,8 @@ cv_grad_weight_narrow_kernel(const float* __restrict__ xpad, const float* __rest
 bool cv_grad_input_chan_supported(const ConvGeom& g) {
     // the staging buffer (four wavefronts, up to 2 * TILE + Kw patches) has to fit the default 64 KB of LDS
     // (plus the 6 KB the output-channel split keeps for its partial sums)
-    return g.C >= 32 && g.Kc % 16 == 0 && (2 * DX_TILE + g.Kw) * 64 * 8 * 4 + 3 * DX_TILE * kWave * 4 <= 64 * 1024;
+    return g.C >= 32 && g.Kc % 16 == 0 && (2 * DX_TILE + g.Kw) * 64 * 8 * 4 + 3 * DX_TILE * kWave * 4 <= 64 * 1024 &&
+           g.Nw * g.Kc * 4 < 0x7fffffffLL;               // an output row of ym / upm behind one buffer descriptor
 }
 
 // wq: the weights regrouped by launch_backward_prologue (mode 2)
