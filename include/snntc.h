@@ -99,7 +99,11 @@ SNNTC_API int snntc_fc_backward_workspace_bytes(int64_t B, int64_t I, int64_t J,
  * rows [B,2B) = 1/(sum_{causal set} w - Spike_Threshold) (0 for a neuron that never fires).
  * Errors: w_rows not in {I, I+1} or inconsistent with biasvolt -> DIM_MISMATCH
  *         (snntc/snnfc_kernels.cc:171-172); B*I, w_rows*J or 2*B*J > INT32_MAX -> TOO_LARGE
- *         (snntc/snnfc_kernels.cc:194-203). */
+ *         (snntc/snnfc_kernels.cc:194-203).
+ * Layers with a handful of outputs (fewer work items than compute units) run a kernel whose
+ * wavefronts hand each other running sums through LDS behind a bounded wait; should that wait ever
+ * run out, the affected (sample, neuron) entries of both halves of `out` are NaN and the call still
+ * returns SNNTC_OK (the library never synchronises with the device).  It has not been observed. */
 SNNTC_API int snntc_fc_forward(const float* x, const float* w, const float* params_host, float* out,
                      int64_t B, int64_t I, int64_t J, int64_t w_rows,
                      void* workspace, size_t workspace_bytes, void* stream);
