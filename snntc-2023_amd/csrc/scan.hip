@@ -1394,10 +1394,13 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     }
     // With at least four wavefronts of multi-neuron lanes for every SIMD, CH neurons per lane (CH times
     // the segments per wavefront) is the cheaper instruction stream; in between, one neuron per
-    // lane in 16-wave workgroups balances better.
+    // lane in 16-wave workgroups balances better -- as long as those workgroups fit the chip in one
+    // go: once one-neuron lanes would need a second round of workgroups, the multi-neuron form, which
+    // still fits, is the faster one (800 x 800 at B = 384: 55 against 79 us).
     constexpr int CH = filter_ch(COLS);
     const int64_t multi_items = (S + CH * SEGS - 1) / (CH * SEGS);
-    const bool multi = !low_latency && multi_items * n_slices >= (int64_t)cus * 4 * 4;
+    const bool multi = !low_latency && (multi_items * n_slices >= (int64_t)cus * 4 * 4 ||
+                                        (CH > 1 && items * n_slices > capacity * 16));
     if (multi) {
         const int64_t per_wg = (multi_items * n_slices + capacity - 1) / capacity;
         WAVES = (int)(per_wg >= 16 ? 16 : (per_wg + 3) / 4 * 4);
