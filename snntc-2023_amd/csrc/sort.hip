@@ -347,11 +347,15 @@ int launch_sort(const SegmentSource& src, int64_t S, float* sorted, int32_t* per
     // (401408 segments of 147: 417 us against 465 us)
     if (I <= 256 && I > 128 && S >= 65536) return launch_sort_t<8, 32>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
     if (I <= 256)  return launch_sort_t<4, 64>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
+    // Few long segments (a dense batch): several wavefronts per segment with two or four elements per
+    // thread instead of one wavefront with eight or more -- the chip fills, and a lone wavefront's long
+    // network is what such a launch waits for.  Rows of 257..512: 7 against 12 us up to 512 rows, the
+    // same from 2048 rows on; rows of 513..1024: 29 against 58 us at 2048 rows, 148 against 183 us at
+    // 16384, so at every count; rows of 1025..2048: 12 against 15 us up to 128 rows, behind from 8192 on.
+    if (I <= 512 && S <= 2048) return launch_sort_t<2, 256>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
     if (I <= 512)  return launch_sort_t<8, 64>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
-    // few long segments (a dense batch): eight wavefronts per segment instead of one fill the chip
-    // (B = 256 rows of 800: 10.7 us against 11.6 us with four, 11.8 us with sixteen)
-    if (I <= 1024 && I > 512 && S < 2048) return launch_sort_t<2, 512>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
-    if (I <= 1024) return launch_sort_t<16, 64>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
+    if (I <= 1024) return launch_sort_t<2, 512>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
+    if (I <= 2048 && S <= 512) return launch_sort_t<4, 512>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
     if (I <= 2048) return launch_sort_t<8, 256>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
     if (I <= 4096) return launch_sort_t<8, 512>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);
     return launch_sort_t<8, 1024>(src, S, sorted, perm, n_real, out_stride, max_cmp, stream);

@@ -286,6 +286,28 @@ def test_many_short_segments_take_the_two_per_wavefront_sort(I):
     assert np.array_equal(out.cpu().numpy().view(np.uint32), ref_out.view(np.uint32))
 
 
+@pytest.mark.parametrize("B,I", [(2100, 600), (40, 400), (2049, 400), (60, 1500), (600, 1500)])
+def test_row_sorts_on_either_side_of_their_shape_switches(B, I):
+    """Rows of 257..512, 513..1024 and 1025..2048 inputs are sorted by several wavefronts per row
+    while the batch is small (for 513..1024 always) and by one or four beyond; both sides of every
+    switch, with ties and rows that carry inputs above MAX_SPIKE_TIME - 0.1, bit for bit against the oracle."""
+    import snntc_amd as snn
+    rng = np.random.default_rng(B + I)
+    J = 3
+    x = (1.0 + rng.integers(0, 60, (B, I)) / 16.0).astype(np.float32)
+    x[3, rng.integers(0, I, 11)] = 2e5
+    x[B - 1, :] = 3e5
+    w = (rng.standard_normal((I + 1, J)) * 0.1 + 4.0 / I).astype(np.float32)
+    p = capi.fc_params(1.0)
+    ref_out, ref_k, ref_sorted, ref_perm = capi.fc_forward_dev(x, w, p, want_aux=True)
+    out, sz, perm, ck = snn.snnfc(t(x), t(w), p, return_aux=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(perm.cpu().numpy(), ref_perm), "permutation differs"
+    assert np.array_equal(sz.cpu().numpy(), ref_sorted)
+    assert np.array_equal(ck.cpu().numpy(), ref_k)
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), ref_out.view(np.uint32))
+
+
 def test_layer_autograd_matches_op_level_chain():
     """SNN_dense / SNN_conv hand the [B,...] upstream gradient to the backward op directly; the result
     must equal slicing the full op output under autograd (zero-extended gradient), bit for bit."""
