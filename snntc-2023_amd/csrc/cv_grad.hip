@@ -489,7 +489,10 @@ int launch_cv_grad_input_chan(const float* xpad, const float* wq, const float* u
     // small images with at least four chunks of output channels: split the channels over the
     // wavefronts of a workgroup.  Decided by the layer's geometry alone, never by the batch: the
     // order of the additions, and with it the last bits of dX, must not depend on the batch size.
-    const int ksplit = (halves == 1 && g.H * tiles_w * c_blocks <= 160 && g.Kc % (4 * kcb) == 0) ? 4 : 1;
+    // (Up to 1024 tiles per image: with 256 output channels a tile's wavefront walks 36 taps, and at small
+    // batches too few tiles exist to hide that -- 256 -> 256 at 16 x 16, one image: 55 against 174 us;
+    // at 32 images the split still is a little ahead, 437 against 491 us.)
+    const int ksplit = (halves == 1 && g.H * tiles_w * c_blocks <= 1024 && g.Kc % (4 * kcb) == 0) ? 4 : 1;
     // One item per workgroup.  Without the split a workgroup is a single wavefront: the
     // wavefronts do not cooperate, their running times differ (border tiles, rows outside the window),
     // and a CU takes a new workgroup only when a whole one has left, so in larger workgroups the slots
