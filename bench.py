@@ -3,7 +3,8 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|cfg1|cfg2|cfg3|cfg4|cfg5|dense]
 
-Prints ONE JSON line.  A "step" is one pass of a workload over one synthetic batch that is already
+The last line of stdout is ONE short JSON record (under 1500 bytes); the per-kernel tables of every workload
+go to stderr as a second JSON line (and to --detail-file).  A "step" is one pass of a workload over one synthetic batch that is already
 resident in HBM.  The workloads are the five BASELINE configurations (and the north-star dense layer):
 
   cfg1   single SNN_dense 784->800 with bias, forward + backward, B=128.
@@ -15,13 +16,13 @@ resident in HBM.  The workloads are the five BASELINE configurations (and the no
   dense  single SNN_dense 784->800 with bias, forward + backward, B=256.
 
 The default, `--workload all`, times every one of them for K steps after W warm-up steps in this one
-process.  The top-level fields of the line (value, ms_per_step, config, roofline, cpu_baseline,
-kernels) are those of cfg5, the largest configuration that runs on one GPU; `per_config` holds the
-same fields for every workload.  With a single workload named, the top level is that workload.
+process.  The top-level fields of the record (value, ms_per_step, config, roofline, cpu_baseline) are
+those of cfg5, the largest configuration that runs on one GPU; `per_config` holds one row per workload
+(`per_config_fields` names the columns).  With a single workload named, the top level is that workload.
 
 `value` is samples/s of the whole step.  `roofline` prices the kernel with the largest share of the
 step against the MI355X peak that bounds it (algorithmic flops or bytes / its measured launch time,
-HIP events recorded by the library on the launch stream); `kernels` carries the same fraction for
+HIP events recorded by the library on the launch stream); the detail line carries the same fraction for
 every library kernel whose algorithmic work is defined.  `cpu_baseline` times the CPU restatement of
 the reference's single-threaded host functors on this machine's cores, on a bounded sample.
 """
@@ -342,7 +343,7 @@ def carried_counters(workload_key, kernel):
         return {}
     entry = dict(table.get("workloads", {}).get(workload_key, {}).get(kernel, {}))
     if entry:
-        entry["source"] = f"profiles/counters.json, measured at commit {table.get('commit', '?')}"
+        entry["source"] = f"profiles/counters.json at commit {table.get('commit', '?')}"
     return entry
 
 
@@ -416,7 +417,7 @@ def cpu_baseline(workload_key, seed=0):
         what = "the same conv/dense layers (pooling and loss left out)"
     dt = time.perf_counter() - t0
     return {"value": n_samples / dt, "unit": "samples/s", "cores": 1, "kind": "port",
-            "sample": f"B={B} through {what}, fwd+bwd, reference host functors restated in C (gcc -O3), 1 thread",
+            "sample": f"B={B}, {what}, fwd+bwd; reference host functors restated in C, gcc -O3, 1 thread",
             "seconds": dt, "host_cpus": os.cpu_count()}
 
 
@@ -509,6 +510,58 @@ def measure(torch, snn, _lib, dev, key, steps, warmup, use_graph=True, want_cpu=
     return res
 
 
+def _sig(v, digits=5):
+    """Numbers rounded to `digits` significant digits (the record line is read by machines with a size limit)."""
+    if isinstance(v, bool) or v is None or isinstance(v, (str, int)):
+        return v
+    if isinstance(v, float):
+        return float(f"{v:.{digits}g}")
+    if isinstance(v, dict):
+        return {k: _sig(x, digits) for k, x in v.items()}
+    if isinstance(v, (list, tuple)):
+        return [_sig(x, digits) for x in v]
+    return v
+
+
+ROOFLINE_KEYS = ("bound", "kernel", "achieved", "peak", "unit", "frac", "traffic", "valu_busy", "avg_launch_us",
+                 "launches_per_step", "algorithmic_flops_per_step", "algorithmic_bytes_per_step", "counters_source")
+CPU_KEYS = ("value", "unit", "cores", "kind", "sample", "seconds", "host_cpus")
+PER_CONFIG_FIELDS = ["ms_per_step", "samples_per_s", "dominant_kernel", "frac", "cpu_samples_per_s", "gpu_kernel_us"]
+LINE_BUDGET = 1500           # bytes; the record line must stay below this
+
+
+def headline(head, per_config, steps, warmup, device):
+    """The one record line: the fields of the headline workload, its dominant kernel's roofline, its CPU
+    baseline, and per workload a row of PER_CONFIG_FIELDS.  Everything else measure() returns (per-kernel
+    tables) is printed elsewhere."""
+    cfg = head["config"]
+    result = {
+        "metric": "SNN layer fwd+bwd samples/sec at 1 GPU; achieved HBM GB/s & % roofline",
+        "value": head["value"],
+        "unit": "samples/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": cfg["workload"], "batch": cfg["batch"], "launch": cfg["launch"], "device": device},
+        "roofline": {k: head["roofline"].get(k) for k in ROOFLINE_KEYS},
+    }
+    if "cpu_baseline" in head:
+        result["cpu_baseline"] = {k: head["cpu_baseline"].get(k) for k in CPU_KEYS}
+    if per_config:
+        result["per_config_fields"] = PER_CONFIG_FIELDS
+        result["per_config"] = {
+            key: [r["ms_per_step"], r["value"], r["roofline"]["kernel"], r["roofline"]["frac"],
+                  r.get("cpu_baseline", {}).get("value"), r["library_kernel_us_per_step"]]
+            for key, r in per_config.items()}
+    return _sig(result)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -520,6 +573,7 @@ def main():
     ap.add_argument("--calibration-copies", type=int, default=0,
                     help="first do this many plain 256 MiB device copies: a kernel of known traffic to scale "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings of the same run by")
+    ap.add_argument("--detail-file", default="", help="also write the per-kernel tables (JSON) to this file")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -548,31 +602,17 @@ def main():
                                   use_graph=not args.no_graph, want_cpu=not args.no_cpu_baseline)
     head = per_config[HEADLINE if args.workload == "all" else keys[0]]
 
-    result = {
-        "metric": "SNN layer fwd+bwd samples/sec at 1 GPU; achieved HBM GB/s & % roofline",
-        "value": head["value"],
-        "unit": "samples/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": head["ms_per_step"],
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "f32",
-        "data": "synthetic",
-        "config": dict(head["config"], device=torch.cuda.get_device_name(0)),
-        "eager_ms_per_step": head["eager_ms_per_step"],
-        "graph_ms_per_step": head["graph_ms_per_step"],
-        "roofline": head["roofline"],
-        "kernels": head["kernels"],
-        "library_kernel_us_per_step": head["library_kernel_us_per_step"],
-    }
-    if "cpu_baseline" in head:
-        result["cpu_baseline"] = head["cpu_baseline"]
-    if args.workload == "all":
-        result["per_config"] = per_config
-    print(json.dumps(result))
+    result = headline(head, per_config if args.workload == "all" else None, args.steps, args.warmup,
+                      torch.cuda.get_device_name(0))
+    # the per-kernel tables of every workload: one line on stderr (and a file, if asked for), so that the
+    # last line of stdout stays a short record
+    detail = json.dumps({"per_config": per_config})
+    print(detail, file=sys.stderr)
+    if args.detail_file:
+        with open(args.detail_file, "w") as f:
+            f.write(detail + "\n")
+    sys.stderr.flush()
+    print(json.dumps(result, separators=(",", ":")))
 
 
 if __name__ == "__main__":

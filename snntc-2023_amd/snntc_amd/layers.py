@@ -3,8 +3,10 @@
 Constructor argument names, order and defaults, the weight layout ``[in_size + bias, out_size]``,
 the two ``Params`` vectors and the padding rules are the reference's; only the framework differs
 (``torch.nn.Module`` + ``torch.autograd.Function`` instead of ``tf.keras.layers.Layer`` +
-``RegisterGradient``).  ``SNN_dense`` and ``SNN_conv`` run the gfx950 ops; pooling, LRN and the
-loss are thin compositions of stock PyTorch ops, exactly as they are stock TF ops in the reference.
+``RegisterGradient``).  ``SNN_dense``, ``SNN_conv``, the earliest-spike pooling layers, the SAME padding
+and the loss run gfx950 kernels and, like the four ops, take float32 tensors on a ROCm device only: there
+is no host fallback.  ``SNN_avgpool2d`` and ``SNN_LRN`` are compositions of stock PyTorch ops, as they are
+stock TF ops in the reference.
 """
 import math
 
@@ -12,6 +14,7 @@ import numpy as np
 import torch
 import torch.nn.functional as F
 
+from ._lib import SnntcLibraryError
 from .ops import SnnCvSame, SnnCvTimes, SnnFcTimes, SnnMinPool, SnnPadTime, SoftmaxTimeLoss
 
 # Mirrors the reference's module-level switch (SNN_TC_Modules.py:11): when True the layers keep
@@ -41,18 +44,29 @@ def _same_pad(size, kernel, stride):
     return before, total - before
 
 
+def _require_device(t, what):
+    """The kernels behind these layers exist for float32 NHWC tensors on a ROCm device only."""
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{what} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise SnntcLibraryError(f"{what} lives on {t.device}: this layer runs on a ROCm GPU only (no CPU fallback)")
+    if t.dtype != torch.float32:
+        raise TypeError(f"{what} must be float32, got {t.dtype}")
+
+
 def _pad_hw(x, kh, kw, sh, sw, value):
-    """Pads NHWC ``x`` for SAME mode with ``value`` (a negative total crops, as tf.pad would fail
-    there the reference never reaches that case)."""
+    """Pads NHWC ``x`` for SAME mode with ``value`` in one kernel pass (a negative total is refused: tf.pad
+    would fail there and the reference never reaches that case)."""
+    _require_device(x, "input")
+    if x.dim() != 4:
+        raise ValueError(f"input must be [B,H,W,C], got shape {tuple(x.shape)}")
     H, W = x.shape[1], x.shape[2]
     top, bottom = _same_pad(H, kh, sh)
     left, right = _same_pad(W, kw, sw)
     if min(top, bottom, left, right) < 0:
         raise ValueError("negative SAME padding: kernel smaller than stride is not supported")
     if top or bottom or left or right:
-        if x.is_cuda and x.dtype == torch.float32 and x.dim() == 4:
-            return SnnPadTime.apply(x.contiguous(), top, bottom, left, right, float(value))    # one pass
-        x = F.pad(x, (0, 0, left, right, top, bottom), mode="constant", value=float(value))
+        return SnnPadTime.apply(x.contiguous(), top, bottom, left, right, float(value))
     return x
 
 
@@ -172,9 +186,11 @@ class SNN_conv(torch.nn.Module, _CostsMixin):
     def forward(self, input, prefilled=False, feed=None):
         """prefilled: the layer before has written `input` into this layer's padded_input_buffer.
         feed: the SNN_conv that follows; its padded input buffer receives this layer's output as well."""
+        _require_device(input, "input")
+        if input.dim() != 4:
+            raise ValueError(f"input must be [B,H,W,C], got shape {tuple(input.shape)}")
         B = input.shape[0]
-        on_device = input.is_cuda and input.dtype == torch.float32 and input.dim() == 4
-        if self.padding == 'SAME' and on_device:
+        if self.padding == 'SAME':
             H, W = input.shape[1], input.shape[2]
             xpad = self.padded_input_buffer(B, H, W, input.device)[0] if prefilled else None
             next_xpad, next_offset = None, (0, 0)
@@ -186,7 +202,7 @@ class SNN_conv(torch.nn.Module, _CostsMixin):
             return SnnCvSame.apply(input.contiguous(), self.weight, self.Params, self.same_pads(H, W), xpad, next_xpad,
                                    next_offset)
         if prefilled or feed is not None:
-            raise ValueError("chaining needs SAME padding and float32 device tensors")
+            raise ValueError("chaining needs SAME padding")
         X = self.prepare_input(input)
         if Check_Dim:
             self.maxD[0] = max(self.maxD[0], int(B))
@@ -224,8 +240,13 @@ class _Pool2d(torch.nn.Module):
         self.name = name
 
     def _padded_nchw(self, input):
+        """Stock-op padding (any device), for the layers that are stock ops in the reference too."""
         if self.padding == 'SAME':
-            input = _pad_hw(input, self.Kh, self.Kw, self.Sh, self.Sw, self.padvalue)
+            top, bottom = _same_pad(input.shape[1], self.Kh, self.Sh)
+            left, right = _same_pad(input.shape[2], self.Kw, self.Sw)
+            if min(top, bottom, left, right) < 0:
+                raise ValueError("negative SAME padding: kernel smaller than stride is not supported")
+            input = F.pad(input, (0, 0, left, right, top, bottom), mode="constant", value=float(self.padvalue))
         return input.permute(0, 3, 1, 2)
 
 
@@ -234,27 +255,24 @@ class SNN_maxpool2d(_Pool2d):
 
     def forward(self, input, feed=None):
         """feed: the SNN_conv that follows; its padded input buffer receives the pooled times as well."""
-        if feed is not None and not (input.is_cuda and input.dtype == torch.float32 and input.dim() == 4):
-            raise ValueError("chaining needs float32 device tensors")
-        if input.is_cuda and input.dtype == torch.float32 and input.dim() == 4:
-            # one kernel each way: the padding is implicit and the minimum is taken directly
-            H, W = input.shape[1], input.shape[2]
-            top = bottom = left = right = 0
-            if self.padding == 'SAME':
-                top, bottom = _same_pad(H, self.Kh, self.Sh)
-                left, right = _same_pad(W, self.Kw, self.Sw)
-                if min(top, bottom, left, right) < 0:
-                    raise ValueError("negative SAME padding: kernel smaller than stride is not supported")
-            nh = (H + top + bottom - self.Kh) // self.Sh + 1
-            nw = (W + left + right - self.Kw) // self.Sw + 1
-            next_xpad, next_offset = None, (0, 0)
-            if feed is not None:
-                next_xpad, next_offset = feed.padded_input_buffer(input.shape[0], nh, nw, input.device)
-            return SnnMinPool.apply(input.contiguous(), (self.Kh, self.Kw), (self.Sh, self.Sw), (top, left), (nh, nw),
-                                    float(self.padvalue), next_xpad, next_offset)
-        x = self._padded_nchw(input)                         # host tensors: the reference's formula itself
-        y = -F.max_pool2d(-x, (self.Kh, self.Kw), (self.Sh, self.Sw))
-        return y.permute(0, 2, 3, 1)
+        _require_device(input, "input")
+        if input.dim() != 4:
+            raise ValueError(f"input must be [B,H,W,C], got shape {tuple(input.shape)}")
+        # one kernel each way: the padding is implicit and the minimum is taken directly
+        H, W = input.shape[1], input.shape[2]
+        top = bottom = left = right = 0
+        if self.padding == 'SAME':
+            top, bottom = _same_pad(H, self.Kh, self.Sh)
+            left, right = _same_pad(W, self.Kw, self.Sw)
+            if min(top, bottom, left, right) < 0:
+                raise ValueError("negative SAME padding: kernel smaller than stride is not supported")
+        nh = (H + top + bottom - self.Kh) // self.Sh + 1
+        nw = (W + left + right - self.Kw) // self.Sw + 1
+        next_xpad, next_offset = None, (0, 0)
+        if feed is not None:
+            next_xpad, next_offset = feed.padded_input_buffer(input.shape[0], nh, nw, input.device)
+        return SnnMinPool.apply(input.contiguous(), (self.Kh, self.Kw), (self.Sh, self.Sw), (top, left), (nh, nw),
+                                float(self.padvalue), next_xpad, next_offset)
 
 
 class SNN_globalminpool2d(torch.nn.Module):
@@ -269,11 +287,10 @@ class SNN_globalminpool2d(torch.nn.Module):
         self.name = name
 
     def forward(self, input):
+        _require_device(input, "input")
         B, H, W, C = input.shape
-        if input.is_cuda and input.dtype == torch.float32:
-            y = SnnMinPool.apply(input.contiguous(), (H, W), (H, W), (0, 0), (1, 1), float(self.padvalue))
-            return y.reshape(B, C)
-        return input.amin(dim=(1, 2))                       # host tensors: the definition itself
+        y = SnnMinPool.apply(input.contiguous(), (H, W), (H, W), (0, 0), (1, 1), float(self.padvalue))
+        return y.reshape(B, C)
 
 
 class SNN_flatten(torch.nn.Module):
@@ -296,8 +313,10 @@ class SNN_avgpool2d(_Pool2d):
 def loss_func(logit=None, label=None):
     """Mean categorical cross-entropy of one-hot ``label`` against softmax(-logit): the earliest
     output spike is the predicted class (SNN_TC_Modules.py:286-288)."""
-    if (logit.is_cuda and logit.dim() == 2 and logit.dtype == torch.float32 and label.dtype == torch.float32
-            and not label.requires_grad):
-        return SoftmaxTimeLoss.apply(logit, label)           # one fused kernel for loss and gradient
-    logp = F.log_softmax(-logit, dim=-1)                      # host tensors / other layouts: the formula itself
-    return torch.mean(-torch.sum(label * logp, dim=-1))
+    _require_device(logit, "logit")
+    _require_device(label, "label")
+    if logit.dim() != 2 or label.shape != logit.shape:
+        raise ValueError(f"logit and label must both be [B, classes], got {tuple(logit.shape)} and {tuple(label.shape)}")
+    if label.requires_grad:
+        raise ValueError("label must not require a gradient: the loss kernel differentiates the spike times only")
+    return SoftmaxTimeLoss.apply(logit, label)               # one fused kernel for loss and gradient

@@ -35,10 +35,24 @@ def test_conv_layer_contract():
     assert v.name == 'convkernel' and v.rates == [1, 1]
 
 
-@pytest.mark.parametrize("H,W,K,S", [(32, 32, 3, 1), (224, 224, 7, 2), (9, 7, 5, 3), (8, 8, 2, 2), (5, 6, 4, 1)])
+SAME_CASES = [(32, 32, 3, 1), (224, 224, 7, 2), (9, 7, 5, 3), (8, 8, 2, 2), (5, 6, 4, 1)]
+
+
+@pytest.mark.parametrize("H,W,K,S", SAME_CASES)
+def test_conv_same_padding_rule(H, W, K, S):
+    """The split of the SAME padding (SNN_TC_Modules.py:147-158) against the closed form the reference's
+    tests recompute (test-snn-cv-forward.py:70-75), and the op's output size on the padded image."""
+    c = snn.SNN_conv(2, 3, K, S, 'SAME')
+    (t, b), (l, r) = cf.same_pad(H, K, S), cf.same_pad(W, K, S)
+    assert c.same_pads(H, W) == (t, b, l, r)
+    assert (H + t + b - K) // S + 1 == -(-H // S) and c.output_hw(H, W) == (-(-H // S), -(-W // S))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,W,K,S", SAME_CASES)
 def test_conv_same_padding_uses_max_spike_time(H, W, K, S):
     c = snn.SNN_conv(2, 3, K, S, 'SAME')
-    x = torch.rand(2, H, W, 2) + 1
+    x = torch.rand(2, H, W, 2, device="cuda:0") + 1
     xp = c.prepare_input(x)
     (t, b), (l, r) = cf.same_pad(H, K, S), cf.same_pad(W, K, S)
     assert xp.shape == (2, H + t + b, W + l + r, 2)
@@ -102,14 +116,8 @@ def test_cost_gradients_against_closed_forms_on_the_gpu():
     _cost_gradient_check("cuda:0")
 
 
-def test_min_time_pool_and_avg_pool():
+def test_avg_pool_is_the_stock_op():
     x = torch.rand(2, 5, 7, 3) + 1
-    mp = snn.SNN_maxpool2d(2, 2, 'SAME')
-    y = mp(x)
-    assert y.shape == (2, 3, 4, 3)
-    xn = np.pad(x.numpy(), ((0, 0), (0, 1), (0, 1), (0, 0)), constant_values=1e5)
-    want = xn.reshape(2, 3, 2, 4, 2, 3).min(axis=(2, 4))               # earliest spike in each window
-    assert np.allclose(y.numpy(), want)
     ap = snn.SNN_avgpool2d(2, 2, 'VALID')
     ya = ap(x)
     assert ya.shape == (2, 2, 3, 3)
@@ -124,11 +132,25 @@ def test_lrn_matches_its_formula():
     assert np.allclose(y, x.numpy() / scale ** 0.75, rtol=1e-6)
 
 
+@pytest.mark.gpu
 def test_loss_is_cross_entropy_on_negated_times():
-    logit = torch.tensor([[1.0, 2.0, 4.0], [3.0, 1.5, 1.2]])
-    label = torch.tensor([[1.0, 0, 0], [0, 0, 1.0]])
+    logit = torch.tensor([[1.0, 2.0, 4.0], [3.0, 1.5, 1.2]], device="cuda:0")
+    label = torch.tensor([[1.0, 0, 0], [0, 0, 1.0]], device="cuda:0")
     want = np.mean([-np.log(np.exp(-1) / np.exp([-1, -2, -4]).sum()), -np.log(np.exp(-1.2) / np.exp([-3, -1.5, -1.2]).sum())])
     assert abs(float(snn.loss_func(logit, label)) - want) < 1e-6
+
+
+def test_glue_layers_refuse_cpu_tensors():
+    """Pooling, SAME padding and the loss run device kernels, like the four ops: no host path."""
+    x = torch.rand(2, 6, 6, 4) + 1
+    for layer in (snn.SNN_maxpool2d(2, 2, 'SAME'), snn.SNN_globalminpool2d(), snn.SNN_conv(4, 3, 3, 1, 'SAME'),
+                  snn.SNN_conv(4, 3, 3, 1, 'VALID')):
+        with pytest.raises(snn.SnntcLibraryError, match="no CPU fallback"):
+            layer(x)
+    with pytest.raises(snn.SnntcLibraryError, match="no CPU fallback"):
+        snn.SNN_conv(4, 3, 3, 1, 'SAME').prepare_input(x)
+    with pytest.raises(snn.SnntcLibraryError, match="no CPU fallback"):
+        snn.loss_func(torch.rand(3, 5), torch.eye(5)[:3])
 
 
 def test_ops_refuse_cpu_tensors():

@@ -76,16 +76,6 @@ def test_hip_pooling_matches_the_oracle(B, H, W, C, Kh, Kw, Sh, Sw, same):
     assert np.array_equal(arg2.cpu().numpy(), arg) and np.array_equal(y2.cpu().numpy(), y)
 
 
-def test_global_min_pool_on_the_host_is_the_definition():
-    """Host tensors take the definition itself: the minimum over the image, per channel."""
-    from snntc_amd.layers import SNN_globalminpool2d
-    rng = np.random.default_rng(1)
-    x = np.exp(rng.random((3, 5, 4, 6))).astype(np.float32)
-    y, _, _ = cf.min_pool(x, 5, 4, 5, 4, same=False)
-    got = SNN_globalminpool2d()(torch.from_numpy(x))
-    assert tuple(got.shape) == (3, 6) and np.array_equal(got.numpy(), y.reshape(3, 6))
-
-
 @pytest.mark.gpu
 @pytest.mark.parametrize("B,H,W,C", [(32, 7, 7, 512), (3, 5, 9, 7), (2, 1, 1, 4), (1, 14, 14, 256)])
 def test_hip_global_min_pool_matches_the_oracle(B, H, W, C):
