@@ -103,7 +103,8 @@ SNNTC_API int snntc_fc_backward_workspace_bytes(int64_t B, int64_t I, int64_t J,
  * Layers with a handful of outputs (fewer work items than compute units) run a kernel whose
  * wavefronts hand each other running sums through LDS behind a bounded wait; should that wait ever
  * run out, the affected (sample, neuron) entries of both halves of `out` are NaN and the call still
- * returns SNNTC_OK (the library never synchronises with the device).  It has not been observed. */
+ * returns SNNTC_OK (the library never synchronises with the device).  It has not been observed.
+ * snntc_scan_status() below reports it without a pass over the outputs. */
 SNNTC_API int snntc_fc_forward(const float* x, const float* w, const float* params_host, float* out,
                      int64_t B, int64_t I, int64_t J, int64_t w_rows,
                      void* workspace, size_t workspace_bytes, void* stream);
@@ -268,6 +269,22 @@ SNNTC_API int snntc_pad_time_backward(const float* dxpad, float* dx, int64_t B, 
  * ------------------------------------------------------------------------------------------- */
 SNNTC_API int snntc_sgd_update(float* const* w, const float* const* dw, const int64_t* n, int64_t count, float lr,
                      void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Health of the bounded wait described at snntc_fc_forward (no counterpart in the reference, whose scan
+ * has one thread per neuron and nothing to wait for).
+ *   snntc_scan_status(&giveups, stream)  number of wavefronts, on the current device since the process
+ *       started, whose wait ran out (each poisons the outputs of its work item with NaN).  0 = every scan
+ *       result so far is what the kernels computed.  The count is a 4-byte device word read with a copy on
+ *       `stream` followed by a wait for that stream: call it where the caller synchronises anyway (after a
+ *       training step's loss has been read, at the end of a batch of requests).
+ *   snntc_debug_set_scan_wait_polls(polls)  test hook: the number of polls a waiting wavefront spends from
+ *       the next launch on (process-wide; polls < 0 restores the default of 2^20).  With 0 every wait that
+ *       is not already satisfied at its first poll gives up, which drives the give-up path while every
+ *       kernel still runs to its end.
+ * ------------------------------------------------------------------------------------------- */
+SNNTC_API int snntc_scan_status(int64_t* giveups, void* stream);
+SNNTC_API int snntc_debug_set_scan_wait_polls(int polls);
 
 /* ---------------------------------------------------------------------------------------------
  * Per-kernel timing (no counterpart in the reference, which only times whole scripts with

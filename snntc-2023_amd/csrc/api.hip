@@ -83,6 +83,7 @@ NeuronParams neuron_params(float max_time, float theta, float biasvolt) {
     np.theta = theta;
     np.biasvolt = biasvolt;
     np.bias = biasvolt > 1e-8f ? 1 : 0;
+    np.wait_polls = 0;                                    // the scan launcher fills it in
     return np;
 }
 
@@ -464,6 +465,16 @@ int snntc_sgd_update(float* const* w, const float* const* dw, const int64_t* n, 
             return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_sgd_update: tensor %lld is a null pointer", (long long)t);
     }
     return launch_sgd_update(w, dw, n, (int)count, lr, static_cast<hipStream_t>(stream));
+}
+
+int snntc_scan_status(int64_t* giveups, void* stream) {
+    if (!giveups) return fail(SNNTC_ERR_BAD_ARGUMENT, "snntc_scan_status: giveups is NULL");
+    return read_scan_giveups(giveups, static_cast<hipStream_t>(stream));
+}
+
+int snntc_debug_set_scan_wait_polls(int polls) {
+    set_scan_wait_polls(polls);
+    return SNNTC_OK;
 }
 
 int snntc_profile_enable(int on) {

@@ -496,7 +496,11 @@ scan_lds_kernel(const float* __restrict__ sorted, const int32_t* __restrict__ pe
 constexpr int SPLIT_WAVES = 8, SPLIT_TESTERS = SPLIT_WAVES - 1;
 constexpr int SPLIT_THREADS = SPLIT_WAVES * kWave;
 constexpr int SPLIT_STATIC_LDS = 3 * SPLIT_WAVES * kWave * 4 + 16;
-constexpr int SPLIT_SPIN_LIMIT = 1 << 20;                  // polls of the progress counter before a tester gives up
+constexpr int SPLIT_SPIN_LIMIT = 1 << 20;                  // default number of polls of the progress counter before a
+                                                           // tester gives up (NeuronParams::wait_polls carries the one in force)
+// Tester wavefronts that gave up since the process started: one word per device, written (a vector
+// atomic) only on that path, read by read_scan_giveups().
+__device__ unsigned int g_scan_giveups = 0;
 constexpr int SPLIT_PAD = 4;                               // floats between the weight rows of two lanes: the 16-byte
                                                            // reads of eight neighbouring lanes fall on distinct banks
 constexpr int SPLIT_ROUND = 4;                             // chunks per round of the producer
@@ -731,6 +735,7 @@ scan_lds_split_kernel(const float* __restrict__ sorted, const int32_t* __restric
                     int spins = 0;
                     const float* in = sums + (c - 1) * 2 * LANES;
                     float x_prev;
+                    bool arrived;
                     for (;;) {
                         const int seen = __hip_atomic_load(&progress, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                         asm volatile("" ::: "memory");
@@ -738,11 +743,12 @@ scan_lds_split_kernel(const float* __restrict__ sorted, const int32_t* __restric
                         ysum = in[LANES + la];
                         x_prev = xs[k - 1];
                         asm volatile("" ::: "memory");
-                        if (__builtin_amdgcn_readfirstlane(seen) >= c || spins >= SPLIT_SPIN_LIMIT) break;
+                        arrived = __builtin_amdgcn_readfirstlane(seen) >= c;
+                        if (arrived || spins >= np.wait_polls) break;
                         __builtin_amdgcn_s_sleep(1);
                         ++spins;
                     }
-                    failed |= spins >= SPLIT_SPIN_LIMIT;
+                    failed |= !arrived;
                     ya = wsum < 0.0f ? -ysum : ysum;        // fired state after input k-1, from the sums
                     yg = ya > x_prev * fabsf(wsum) ? ya : INFINITY;
                 }
@@ -753,6 +759,7 @@ scan_lds_split_kernel(const float* __restrict__ sorted, const int32_t* __restric
 #pragma unroll
                 for (int u = 0; u < CHUNK; ++u) { xc[u] = xn[u]; wc[u] = wn[u]; }
             }
+            if (failed && lane == 0) atomicAdd(&g_scan_giveups, 1u);
             k_found[wave][lane] = failed ? -1 : k_close;    // -1 poisons the result below
             w_found[wave][lane] = w_close;
             y_found[wave][lane] = y_close;
@@ -1367,10 +1374,26 @@ int scan_prepare_device(int dev, int* cu_count_out) {
     return SNNTC_OK;
 }
 
+namespace {
+std::atomic<int> g_wait_polls{SPLIT_SPIN_LIMIT};
+}
+
+void set_scan_wait_polls(int polls) { g_wait_polls.store(polls < 0 ? SPLIT_SPIN_LIMIT : polls, std::memory_order_relaxed); }
+
+int read_scan_giveups(int64_t* count, hipStream_t stream) {
+    unsigned int v = 0;
+    SNNTC_HIP_CHECK(hipMemcpyFromSymbolAsync(&v, HIP_SYMBOL(g_scan_giveups), sizeof(v), 0, hipMemcpyDeviceToHost, stream));
+    SNNTC_HIP_CHECK(hipStreamSynchronize(stream));
+    *count = (int64_t)v;
+    return SNNTC_OK;
+}
+
 template <int COLS>
 int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_real, const float* w, float* y,
                     float* rcp, int32_t* causal_k, int64_t S, int64_t I, int64_t stride, int64_t J,
-                    const NeuronParams& np, const TimeCopy& copy, size_t lds_bytes, hipStream_t stream) {
+                    const NeuronParams& np_in, const TimeCopy& copy, size_t lds_bytes, hipStream_t stream) {
+    NeuronParams np = np_in;
+    np.wait_polls = g_wait_polls.load(std::memory_order_relaxed);
     int dev = 0, cus = 0;
     SNNTC_HIP_CHECK(hipGetDevice(&dev));
     const int prep = scan_prepare_device(dev, &cus);
@@ -1434,6 +1457,9 @@ int launch_scan_lds(const float* sorted, const int32_t* perm, const int32_t* n_r
     {
         KernelTimerScope timer_("scan", stream);
         const size_t dyn_lds = filt ? lds_bytes + filter_extra_lds(COLS, multi ? CH : 1, WAVES) : split ? split_lds : lds_bytes;
+        if (dyn_lds > (size_t)LDS_SCAN_BYTES)
+            return fail(SNNTC_ERR_UNSUPPORTED, "scan: %zu bytes of LDS for %d rows x %d columns exceed the %d available",
+                        dyn_lds, (int)(I + np.bias), COLS, LDS_SCAN_BYTES);
         if (causal_k)
             hipLaunchKernelGGL(kern_k, grid, block, dyn_lds, stream, sorted, perm, n_real, w, y, rcp, causal_k,
                                (int)S, (int)I, (int)stride, (int)J, n_slices, (int)n_groups, np, copy);
@@ -1454,7 +1480,9 @@ int launch_scan(const float* sorted, const int32_t* perm, const int32_t* n_real,
     int cols = 64;
     while (cols > 8 && (rows * cols * sizeof(float) > (size_t)LDS_SCAN_TARGET || cols / 2 >= J)) cols >>= 1;
     const size_t lds_bytes = rows * cols * sizeof(float);
-    if (lds_bytes <= (size_t)LDS_SCAN_BYTES) {
+    // (LDS_SCAN_TARGET, not the full 160 KB: whichever LDS kernel the launch shape selects must find room for
+    // its chunk buffers behind the slice -- 8-column slices of 5055..5120 rows would fit on their own only)
+    if (lds_bytes <= (size_t)LDS_SCAN_TARGET) {
         switch (cols) {
             case 64: return launch_scan_lds<64>(sorted, perm, n_real, w, y, rcp, causal_k, S, I, stride, J, np, copy, lds_bytes, stream);
             case 32: return launch_scan_lds<32>(sorted, perm, n_real, w, y, rcp, causal_k, S, I, stride, J, np, copy, lds_bytes, stream);

@@ -73,6 +73,8 @@ struct NeuronParams {
     float theta;      // Spike_Threshold
     float biasvolt;   // input value of the bias row
     int bias;         // biasvolt > 1e-8
+    int wait_polls;   // scan_lds_split_kernel: polls a tester wavefront spends on the producer's sums before it
+                      // gives up (set by the scan launcher, see scan_wait_polls)
 };
 
 // The weight-gradient kernels add up u * min(x - y, 0) over the segments.  They evaluate the second
@@ -160,6 +162,12 @@ int launch_unpad_rows(const float* sorted, const int32_t* perm, float* sorted_ou
 int launch_scan(const float* sorted, const int32_t* perm, const int32_t* n_real, const float* w, float* y,
                 float* rcp, int32_t* causal_k, int64_t S, int64_t I, int64_t stride, int64_t J,
                 const NeuronParams& np, const TimeCopy& copy, hipStream_t stream);
+
+// Bounded wait of the classifier-head scan (scan_lds_split_kernel): the poll limit launches use from now on
+// (polls < 0 restores the default), and the number of tester wavefronts that ran out of it on the current
+// device since the process started (read with a copy on `stream` and a wait for that stream).
+void set_scan_wait_polls(int polls);
+int read_scan_giveups(int64_t* count, hipStream_t stream);
 
 // One-time set-up on device `dev`, which must be the current device: the dynamic-LDS limits of every
 // scan / merge instantiation (and the CU count the scan sizes its launches with).  The launchers call

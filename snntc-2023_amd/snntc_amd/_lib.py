@@ -31,6 +31,7 @@ EXPORTS = (
     "snntc_softmax_time_loss", "snntc_sgd_update",
     "snntc_min_pool_forward", "snntc_min_pool_backward",
     "snntc_pad_time_forward", "snntc_pad_time_backward",
+    "snntc_scan_status", "snntc_debug_set_scan_wait_polls",
     "snntc_profile_enable", "snntc_profile_collect", "snntc_profile_entry",
 )
 
@@ -104,6 +105,8 @@ def load():
     lib.snntc_min_pool_backward.argtypes = [vp, vp, vp] + [i64] * 12 + [vp]
     lib.snntc_pad_time_forward.argtypes = [vp, vp] + [i64] * 8 + [c.c_float, vp]
     lib.snntc_pad_time_backward.argtypes = [vp, vp] + [i64] * 8 + [vp]
+    lib.snntc_scan_status.argtypes = [c.POINTER(i64), vp]
+    lib.snntc_debug_set_scan_wait_polls.argtypes = [c.c_int]
     lib.snntc_profile_enable.argtypes = [c.c_int]
     lib.snntc_profile_collect.argtypes = []
     lib.snntc_profile_entry.argtypes = [c.c_int, c.POINTER(c.c_char_p), c.POINTER(i64), c.POINTER(c.c_double)]
@@ -141,3 +144,16 @@ def profile_collect():
         check(lib.snntc_profile_entry(i, ctypes.byref(name), ctypes.byref(cnt), ctypes.byref(ms)))
         out[name.value.decode()] = (cnt.value, ms.value)
     return out
+
+
+def scan_giveups(stream=None):
+    """Wavefronts of the classifier-head scan whose bounded wait ran out on the current device since the
+    process started (each leaves NaN in the outputs of its work item).  Waits for `stream`."""
+    n = ctypes.c_int64()
+    check(load().snntc_scan_status(ctypes.byref(n), ctypes.c_void_p(stream or 0)))
+    return n.value
+
+
+def set_scan_wait_polls(polls):
+    """Test hook: polls a waiting scan wavefront spends from the next launch on (< 0: the default)."""
+    check(load().snntc_debug_set_scan_wait_polls(int(polls)))

@@ -19,6 +19,23 @@ import torch
 from . import _lib
 
 _workspaces = {}
+_giveups_seen = {}
+
+
+def check_scan_health(device=None):
+    """Raises SnntcError if, since the last call for this device, a wavefront of the classifier-head scan
+    ran out of its bounded wait (the affected outputs are NaN).  Synchronises with the current stream of
+    the device: call it where the program waits for the GPU anyway (after reading a loss, at the end of
+    an epoch or of a batch of requests)."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    with torch.cuda.device(device):
+        n = _lib.scan_giveups(torch.cuda.current_stream(device).cuda_stream)
+    before = _giveups_seen.get(device.index, 0)
+    _giveups_seen[device.index] = n
+    if n > before:
+        raise _lib.SnntcError(_lib.ERR_HIP, f"{n - before} scan wavefront(s) gave up waiting for partial sums on "
+                                            f"{device}: the outputs of their work items are NaN")
+    return n
 
 
 def _params(params, n):

@@ -60,11 +60,14 @@ DENSE_CASES = [
     (15, 128, 2048, 512, True, "baseline"),    # CIFAR-shaped net, first dense layer
     (16, 128, 512, 10, True, "baseline"),      # CIFAR-shaped net, head
     (17, 32, 512, 1000, True, "baseline"),     # ImageNet-shaped net, classifier
-    # inputs so long that not even 8 weight columns fit in LDS: the scan streams the weight rows
-    # (I + bias > 5120), and the last size that still uses the LDS-resident slice
-    (18, 3, 5117, 24, True, "baseline"),       # 5118 rows x 8 columns: the largest slice that is kept in LDS
-    (19, 3, 5120, 24, False, "baseline"),      # 160 KB exactly: no room left beside the slice, streaming scan
-    (20, 3, 5120, 70, True, "baseline"),       # first size past it: streaming scan, two column blocks
+    # inputs so long that not even 8 weight columns fit in LDS beside the kernels' chunk buffers: the scan
+    # streams the weight rows (I + bias > 5054), and the last size that still uses the LDS-resident slice
+    (18, 3, 5053, 24, True, "baseline"),       # 5054 rows x 8 columns: the largest slice that is kept in LDS
+    (27, 2800, 5053, 24, True, "baseline"),    # the same slice under the filter kernel (a large batch)
+    (28, 3, 5054, 24, True, "baseline"),       # 5055 rows: first size that streams
+    (29, 2800, 5100, 24, True, "baseline"),    # 5055..5120 rows at a large batch: streaming scan
+    (19, 3, 5120, 24, False, "baseline"),      # 160 KB exactly: streaming scan
+    (20, 3, 5120, 70, True, "baseline"),       # streaming scan, two column blocks
     (21, 2, 8192, 33, True, "reftest"),        # the longest segment one sorting network takes
     # longer segments: sorted in pieces of 8192 and merged in global memory
     (23, 3, 8193, 20, True, "reftest"),        # two pieces, the second with a single input
@@ -404,6 +407,47 @@ def test_dense_head_forward_bit_exact(seed, B, I, J, bias):
     assert np.array_equal(out.view(np.uint32), ref_out.view(np.uint32)), "y / 1/S not bit-exact"
     assert np.array_equal(out2.view(np.uint32), ref_out.view(np.uint32)), "plain entry point not bit-exact"
     assert np.all(ref_k[:, 0] == -1) and (ref_k >= 0).any(), "the case should hold firing and silent neurons"
+
+
+def test_head_scan_bounded_wait_gives_up_visibly():
+    """The classifier-head scan hands running sums from one wavefront to the others behind a bounded
+    wait.  With the poll limit at zero (a host-side test hook; every kernel still runs to its end) a
+    waiting wavefront gives up on its first poll unless the sums are already there: the call still
+    returns SNNTC_OK, every output is either the oracle's bits or NaN in BOTH halves of `out`, the
+    status word counts the wavefronts that gave up, and check_scan_health() raises.  With the limit
+    restored the same call is bit-exact again and the count stays where it was."""
+    import snntc_amd as snn
+    from snntc_amd import _lib
+    rng = np.random.default_rng(5)
+    B, I, J = 32, 800, 10                                          # 16 work items of one workgroup each
+    x = np.exp(1.0 - rng.random((B, I))).astype(np.float32)
+    w = ((4.0 / I) + rng.standard_normal((I + 1, J)) * np.sqrt(1.0 / I)).astype(np.float32)
+    p = capi.fc_params(1.0)
+    ref = capi.fc_forward_dev(x, w, p)
+    xt, wt = t(x), t(w)
+    snn.check_scan_health(DEV)                                     # settles the count seen so far
+    before = _lib.scan_giveups()
+    _lib.set_scan_wait_polls(0)
+    try:
+        out = snn.snnfc(xt, wt, p)                                 # no exception: status SNNTC_OK
+        torch.cuda.synchronize()
+    finally:
+        _lib.set_scan_wait_polls(-1)
+    out = out.cpu().numpy()
+    gave_up = _lib.scan_giveups() - before
+    y, r = out[:B], out[B:]
+    poisoned = np.isnan(y)
+    assert np.array_equal(poisoned, np.isnan(r)), "a poisoned neuron must be NaN in both halves"
+    good = ~poisoned
+    assert np.array_equal(y[good].view(np.uint32), ref[:B][good].view(np.uint32))
+    assert np.array_equal(r[good].view(np.uint32), ref[B:][good].view(np.uint32))
+    # a lone wavefront needs microseconds for the first chunk's sums; the testers poll within nanoseconds
+    assert poisoned.any() and gave_up > 0, "the give-up path did not run"
+    with pytest.raises(snn.SnntcError, match="gave up"):
+        snn.check_scan_health(DEV)
+    out = snn.snnfc(xt, wt, p).cpu().numpy()
+    assert np.array_equal(out.view(np.uint32), ref.view(np.uint32)), "default wait: not bit-exact"
+    assert snn.check_scan_health(DEV) == before + gave_up
 
 
 def test_sgd_update_matches_numpy():
