@@ -114,14 +114,16 @@ fc_grad_input_kernel(const SegmentSource src, const float* __restrict__ wt,
     const int b0 = blockIdx.x * DX_RB;
 
     float xr[DX_RB], acc[DX_RB];
-    const float* __restrict__ yrow[DX_RB];
-    const float* __restrict__ urow[DX_RB];
+    // the y / up rows of the block's samples: one base pointer each and a byte offset per sample (eight
+    // scalar registers instead of sixteen for eight pointers; samples past the batch repeat the last row)
+    const float* __restrict__ ybase = ym + (size_t)b0 * J;
+    const float* __restrict__ ubase = upm + (size_t)b0 * J;
+    int row_bytes[DX_RB];
 #pragma unroll
     for (int r = 0; r < DX_RB; ++r) {
         const int brow = min(b0 + r, B - 1);
         xr[r] = PATCHES ? segment_base(src, brow)[row_offset(src, (int)ic)] : x[(size_t)brow * I + ic];
-        yrow[r] = ym + (size_t)brow * J;
-        urow[r] = upm + (size_t)brow * J;
+        row_bytes[r] = (brow - b0) * J * (int)sizeof(float);
         acc[r] = 0.0f;
     }
     const int jq = (J + 3) / 4;
@@ -140,8 +142,9 @@ fc_grad_input_kernel(const SegmentSource src, const float* __restrict__ wt,
             const int off = jj * (int)sizeof(float);
 #pragma unroll
             for (int r = 0; r < DX_RB; ++r) {
-                asm volatile("s_load_dwordx4 %0, %1, %2" : "=s"(yv[r]) : "s"(yrow[r]), "s"(off));
-                asm volatile("s_load_dwordx4 %0, %1, %2" : "=s"(uv[r]) : "s"(urow[r]), "s"(off));
+                const int o = row_bytes[r] + off;
+                asm volatile("s_load_dwordx4 %0, %1, %2" : "=s"(yv[r]) : "s"(ybase), "s"(o));
+                asm volatile("s_load_dwordx4 %0, %1, %2" : "=s"(uv[r]) : "s"(ubase), "s"(o));
             }
         };
         auto arrived = [&](f4 (&yv)[DX_RB], f4 (&uv)[DX_RB]) {
@@ -197,7 +200,8 @@ fc_grad_input_kernel(const SegmentSource src, const float* __restrict__ wt,
         const float wv = wcol[(size_t)j * wt_stride];
 #pragma unroll
         for (int r = 0; r < DX_RB; ++r) {
-            acc[r] = xr[r] <= yrow[r][j] ? __fmaf_rn(urow[r][j], wv, acc[r]) : acc[r];
+            const int e = row_bytes[r] / (int)sizeof(float) + j;
+            acc[r] = xr[r] <= ybase[e] ? __fmaf_rn(ubase[e], wv, acc[r]) : acc[r];
         }
     }
     if (wave > 0) {

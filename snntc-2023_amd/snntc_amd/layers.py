@@ -168,15 +168,26 @@ class SNN_conv(torch.nn.Module, _CostsMixin):
         """The layer's own padded input for B images of H x W (SAME mode): a tensor [B,Hp,Wp,C] that lives as
         long as the layer, its border filled with MAX_SPIKE_TIME once, and (top, left), where the image
         goes.  The layer before writes its output straight into the interior (`feed`), so no padding pass
-        runs between the two; the content belongs to the latest forward pass."""
+        runs between the two; the content belongs to the latest forward pass (a backward pass of an
+        earlier one is refused by autograd: the writes advance the buffer's version counter).  The
+        layer keeps the buffers of the MAX_PADDED_BUFFERS input shapes used last; release_buffers() drops
+        them all."""
         top, bottom, left, right = self.same_pads(H, W)
         key = (B, H, W, str(device))
-        buf = self._padded.get(key)
+        buf = self._padded.pop(key, None)
         if buf is None:
             buf = torch.full((B, top + H + bottom, left + W + right, self.C), float(self.Params[0]),
                              dtype=torch.float32, device=device)
-            self._padded[key] = buf
+            while len(self._padded) >= self.MAX_PADDED_BUFFERS:
+                self._padded.pop(next(iter(self._padded)))          # the shape used longest ago
+        self._padded[key] = buf                                     # most recently used last
         return buf, (top, left)
+
+    MAX_PADDED_BUFFERS = 4
+
+    def release_buffers(self):
+        """Drops the padded input buffers (they are re-created on demand)."""
+        self._padded.clear()
 
     def output_hw(self, H, W):
         if self.padding == 'SAME':

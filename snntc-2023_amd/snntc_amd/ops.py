@@ -75,6 +75,15 @@ def _workspace(device, nbytes):
     return buf
 
 
+def _written_behind_autograd(t):
+    """A kernel has written into `t` through its raw pointer.  Autograd counts in-place writes per tensor
+    and refuses to run a backward pass whose saved tensors have been written since they were saved; the
+    count is advanced here so that this protection also covers the padded input buffers the chained
+    layers fill (a second forward pass before the backward pass of the first would otherwise silently
+    differentiate against the second pass's input)."""
+    torch.autograd.graph.increment_version(t)
+
+
 def release_workspaces():
     """Drops the cached eager scratch buffers (they are re-created on demand)."""
     _workspaces.clear()
@@ -214,6 +223,7 @@ def snncv(X, W, Params, return_aux=False, next_xpad=None, next_offset=(0, 0)):
             _lib.check(lib.snntc_cv_forward_chained(_ptr(X), _ptr(W), pp, _ptr(out), _ptr(nx), nx.shape[1], nx.shape[2],
                                                     next_offset[0], next_offset[1], B, H, Wd, C, Kc, w_rows, _ptr(ws),
                                                     ws.numel(), _stream(X.device)))
+            _written_behind_autograd(next_xpad)
             return out
         _lib.check(lib.snntc_cv_forward(_ptr(X), _ptr(W), pp, _ptr(out), B, H, Wd, C, Kc, w_rows, _ptr(ws),
                                         ws.numel(), _stream(X.device)))
@@ -450,6 +460,7 @@ def min_pool(x, kernel, stride, pad, out_hw, pad_value=1e5, want_arg=True, next_
                                                           next_offset[0], next_offset[1], B, H, W, C, kernel[0],
                                                           kernel[1], stride[0], stride[1], pad[0], pad[1], out_hw[0],
                                                           out_hw[1], float(pad_value), _stream(x.device)))
+            _written_behind_autograd(next_xpad)
             return y, arg
         _lib.check(lib.snntc_min_pool_forward(_ptr(x), _ptr(y), _ptr(arg), B, H, W, C, kernel[0], kernel[1], stride[0],
                                               stride[1], pad[0], pad[1], out_hw[0], out_hw[1], float(pad_value),

@@ -99,3 +99,29 @@ def test_chained_network_matches_the_unchained_one_bit_for_bit():
     plain(zin).sum().backward()
     chained(zin2).sum().backward()
     assert torch.equal(zin.grad, zin2.grad)
+
+
+def test_backward_after_a_second_forward_of_a_chained_network_is_refused():
+    """The padded input buffers of chained layers belong to the latest forward pass.  A backward pass of
+    an earlier forward would differentiate against the later pass's inputs; autograd refuses it because
+    the kernels' writes advance the buffers' version counters.  Forward, backward, forward, backward (a
+    training loop) is unaffected, and the layers keep a bounded number of buffers."""
+    from snntc_amd import networks
+    rng = np.random.default_rng(7)
+    z1 = t(np.exp(1.0 - rng.random((2, 16, 16, 3))).astype(np.float32))
+    z2 = t(np.exp(1.0 - rng.random((2, 16, 16, 3))).astype(np.float32))
+    net = networks.build(SMALL_NET, weights=networks.draw_weights(SMALL_NET, rng), chain=True).to(DEV)
+    y1 = net(z1)
+    net(z2)                                                    # overwrites the padded buffers y1's graph saved
+    with pytest.raises(RuntimeError, match="modified by an inplace operation"):
+        y1.sum().backward()
+    for z in (z1, z2):                                         # the ordinary order still works
+        net.zero_grad(set_to_none=True)
+        net(z).sum().backward()
+        assert all(w.grad is not None and bool(torch.isfinite(w.grad).all()) for w in net.weights())
+    conv = [m for m in net if hasattr(m, "release_buffers")][1]
+    for B in range(1, 8):                                      # ragged batches: buffers do not pile up
+        net(z1[:1].expand(B, -1, -1, -1).contiguous())
+    assert len(conv._padded) <= conv.MAX_PADDED_BUFFERS
+    conv.release_buffers()
+    assert len(conv._padded) == 0
