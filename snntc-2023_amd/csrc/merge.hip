@@ -118,6 +118,32 @@ __device__ __forceinline__ void wave_merge(const u64* A, int nA, const u64* B, i
     if (lane == 0) out[n] = ~0ull;
 }
 
+// The same merge by a whole workgroup of `nthreads` threads (thread `tid` takes one run of consecutive
+// outputs): for patches so long that a buffer pair per wavefront does not fit in LDS.  The caller puts
+// a workgroup barrier behind it before anyone reads `out`.
+__device__ __forceinline__ void block_merge(const u64* A, int nA, const u64* B, int nB, u64 orB, u64* out, int tid,
+                                            int nthreads) {
+    const int n = nA + nB;
+    const int E = (n + nthreads - 1) / nthreads;
+    const int d0 = min(tid * E, n), d1 = min(d0 + E, n);
+    int lo = max(0, d0 - nB), hi = min(d0, nA);
+    while (lo < hi) {                                          // co-rank of the run's first output
+        const int mid = (lo + hi) >> 1;
+        const bool a_first = A[mid] < (B[d0 - mid - 1] | orB);
+        lo = a_first ? mid + 1 : lo;
+        hi = a_first ? hi : mid;
+    }
+    int i = lo, j = d0 - lo;
+    for (int e = d0; e < d1; ++e) {
+        const u64 a = A[i], b = B[j] | orB;                    // sentinels stand in for an exhausted list
+        const bool take_a = a < b;
+        out[e] = take_a ? a : b;
+        i += take_a ? 1 : 0;
+        j += take_a ? 0 : 1;
+    }
+    if (tid == 0) out[n] = ~0ull;
+}
+
 constexpr int MERGE_THREADS = 256;
 constexpr int MERGE_RUNS = 1;                             // runs of outputs a lane merges side by side
 constexpr int MERGE_WAVES = MERGE_THREADS / kWave;
@@ -125,7 +151,11 @@ constexpr int MERGE_WAVES = MERGE_THREADS / kWave;
 // One workgroup = TW consecutive patches of one output row.
 //   pix_z / pix_c : every pixel's channels sorted ascending and their channel ids, rows of Cs entries
 //   sorted / perm : [S, stride] outputs (entries past P padded with +inf / 0), n_real[S]
-__global__ void __launch_bounds__(MERGE_THREADS)
+// BLOCKWIDE = false: every wavefront merges patches of its own between two buffers private to it.
+// BLOCKWIDE = true (patches of thousands of entries, whose buffer pairs would not fit once per
+// wavefront): the workgroup merges one patch at a time between a single pair of buffers.
+template <int THREADS, bool BLOCKWIDE>
+__global__ void __launch_bounds__(THREADS)
 merge_patches_kernel(const float* __restrict__ pix_z, const int32_t* __restrict__ pix_c, int Cs,
                      float* __restrict__ sorted, int32_t* __restrict__ perm, int32_t* __restrict__ n_real,
                      int H, int W, int C, int Kh, int Kw, int Sh, int Sw, int Nh, int Nw, int TW, int tiles_w,
@@ -141,7 +171,7 @@ merge_patches_kernel(const float* __restrict__ pix_z, const int32_t* __restrict_
     // list before it (the merges of a patch alternate between the two)
     const int col_stride = KhC + 1, out_stride = P + 1 + (Kw > 2 ? P - KhC + 1 : 0);
     u64* col_keys = reinterpret_cast<u64*>(lds_raw);                                   // [tile_cols][KhC + 1]
-    u64* out_keys = col_keys + (size_t)tile_cols * col_stride;                         // [MERGE_WAVES][out_stride]
+    u64* out_keys = col_keys + (size_t)tile_cols * col_stride;                         // [buffer pairs][out_stride]
     float* px_z = reinterpret_cast<float*>(out_keys);                                  // [Kh][tile_cols][C]
     uint16_t* px_c = reinterpret_cast<uint16_t*>(px_z + (size_t)Kh * tile_cols * C);   // [Kh][tile_cols][C]
 
@@ -166,12 +196,12 @@ merge_patches_kernel(const float* __restrict__ pix_z, const int32_t* __restrict_
     // ---- stage the sorted pixels under the tile ------------------------------------------------
     // loads are issued in batches: one at a time would cost a memory latency per group
     constexpr int STAGE = 4;
-    for (int base = threadIdx.x; base < n_groups; base += STAGE * MERGE_THREADS) {
+    for (int base = threadIdx.x; base < n_groups; base += STAGE * THREADS) {
         float4 zv[STAGE];
         int4 cv[STAGE];
 #pragma unroll
         for (int u = 0; u < STAGE; ++u) {
-            const int g = base + u * MERGE_THREADS;
+            const int g = base + u * THREADS;
             int row, c, kh, col;
             split(g, row, c, kh, col);
             const int wp = w_first + col;
@@ -185,7 +215,7 @@ merge_patches_kernel(const float* __restrict__ pix_z, const int32_t* __restrict_
         }
 #pragma unroll
         for (int u = 0; u < STAGE; ++u) {
-            const int g = base + u * MERGE_THREADS;
+            const int g = base + u * THREADS;
             if (g < n_groups) {
                 reinterpret_cast<float4*>(px_z)[g] = zv[u];
                 reinterpret_cast<uint2*>(px_c)[g] = make_uint2((uint32_t)cv[u].x | ((uint32_t)cv[u].y << 16),
@@ -197,7 +227,7 @@ merge_patches_kernel(const float* __restrict__ pix_z, const int32_t* __restrict_
 
     // ---- column lists: merge the Kh pixels of every column -----------------------------------------
     // A thread ranks the NB = 4 elements of a group side by side.
-    for (int g = threadIdx.x; g < n_groups; g += MERGE_THREADS) {
+    for (int g = threadIdx.x; g < n_groups; g += THREADS) {
         int row, l0, kh, col;
         split(g, row, l0, kh, col);
         const float4 zq = reinterpret_cast<const float4*>(px_z)[g];
@@ -216,8 +246,49 @@ merge_patches_kernel(const float* __restrict__ pix_z, const int32_t* __restrict_
             col_keys[(size_t)col * col_stride + rank[i]] = ((u64)order_key(z[i]) << 32) | ((u64)kh << 24) | ch[i];
     }
     __syncthreads();                                          // the pixel lists are dead from here on
-    for (int col = threadIdx.x; col < tile_cols; col += MERGE_THREADS) col_keys[(size_t)col * col_stride + KhC] = ~0ull;
+    for (int col = threadIdx.x; col < tile_cols; col += THREADS) col_keys[(size_t)col * col_stride + KhC] = ~0ull;
     __syncthreads();
+
+    if constexpr (BLOCKWIDE) {
+        // ---- patches, one at a time, by the whole workgroup ------------------------------------------
+        __shared__ int below_count;
+        u64* other = out_keys + P + 1;
+        for (int j = 0; j < TW && nw0 + j < Nw; ++j) {
+            const u64* cols = col_keys + (size_t)(j * Sw) * col_stride;
+            const u64* acc = cols;
+            if (threadIdx.x == 0) below_count = 0;
+            for (int kw = 1; kw < Kw; ++kw) {
+                u64* dst = ((Kw - 1 - kw) & 1) ? other : out_keys;
+                block_merge(acc, kw * KhC, cols + (size_t)kw * col_stride, KhC, (u64)kw << 16, dst, threadIdx.x, THREADS);
+                __syncthreads();
+                acc = dst;
+            }
+            const size_t s = (size_t)(a * Nh + nh) * Nw + nw0 + j;
+            float* so = sorted + s * stride;
+            int32_t* po = perm + s * stride;
+            int below = 0;
+            for (int e = threadIdx.x; e < stride; e += THREADS) {
+                float z = INFINITY;
+                int32_t id = 0;
+                if (e < P) {
+                    const u64 key = acc[e];
+                    z = order_key_to_float((uint32_t)(key >> 32));
+                    const uint32_t low = (uint32_t)key;                    // kh | kw | c
+                    id = (int32_t)(((low >> 24) * Kw + ((low >> 16) & 0xffu)) * C + (low & 0xffffu));
+                }
+                below += (e < P && z <= max_cmp) ? 1 : 0;
+                so[e] = z;
+                po[e] = id;
+            }
+#pragma unroll
+            for (int d = kWave / 2; d > 0; d >>= 1) below += __shfl_xor(below, d, kWave);
+            if (threadIdx.x % kWave == 0 && below != 0) atomicAdd(&below_count, below);
+            __syncthreads();                                  // the buffers are free again, the count is complete
+            if (threadIdx.x == 0) n_real[s] = below_count;
+            __syncthreads();
+        }
+        return;
+    }
 
     // ---- patches: merge the Kw columns of every patch ----------------------------------------------
     // From here on a wavefront works alone: the column lists are read-only and its two buffers are
@@ -225,7 +296,7 @@ merge_patches_kernel(const float* __restrict__ pix_z, const int32_t* __restrict_
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
     u64* my_out = out_keys + (size_t)wave * out_stride;
-    for (int j = wave; j < TW && nw0 + j < Nw; j += MERGE_WAVES) {
+    for (int j = wave; j < TW && nw0 + j < Nw; j += THREADS / kWave) {
         // column 0 with 1, the result with 2, ...: the merge that takes in column kw writes the
         // patch buffer when Kw - 1 - kw is even and the other buffer otherwise, so that the last
         // one lands in the patch buffer
@@ -258,27 +329,53 @@ merge_patches_kernel(const float* __restrict__ pix_z, const int32_t* __restrict_
     }
 }
 
-size_t merge_lds_bytes(int C, int Kh, int Kw, int Sw, int TW) {
+// LDS of a workgroup with `pairs` buffer pairs for finished / half-finished patches.
+size_t merge_lds_bytes(int C, int Kh, int Kw, int Sw, int TW, int pairs = MERGE_WAVES) {
     const size_t tile_cols = (size_t)(TW - 1) * Sw + Kw;
     const size_t KhC = (size_t)Kh * C, P = KhC * Kw;
-    const size_t staging = (size_t)MERGE_WAVES * (P + 1 + (Kw > 2 ? P - KhC + 1 : 0)) * 8;
+    const size_t staging = (size_t)pairs * (P + 1 + (Kw > 2 ? P - KhC + 1 : 0)) * 8;
     const size_t pixels = (size_t)Kh * tile_cols * C * (4 + 2);
     return tile_cols * (KhC + 1) * 8 + (staging > pixels ? staging : pixels);
 }
 
-// Patches per tile: as many as fit in 52 KB of LDS (so three workgroups share a CU), at
-// most 16, never more than the row holds.  Layers with so many channels that not even two
-// patches fit in 52 KB take what fits in MERGE_LDS_CAP (one workgroup per CU).
 constexpr size_t MERGE_LDS_CAP = 160 * 1024;
-int merge_tile_width(const ConvGeom& g) {
+constexpr int MERGE_BLOCKWIDE_THREADS = 1024;
+
+// How a layer's patches are merged.  Patches per tile: as many as fit in 52 KB of LDS (so three
+// workgroups share a CU), at most 16, never more than the row holds.  Layers with so many channels
+// that not even two patches fit in 52 KB take what fits in MERGE_LDS_CAP (one workgroup per CU); where
+// that leaves a narrow tile or none at all (a buffer pair per wavefront is 31 KB for 3 x 3 x 256 and
+// 61 KB for 3 x 3 x 512), the workgroup -- of 16 wavefronts then -- keeps a single pair and merges one
+// patch at a time, the row cut into tiles of equal width.
+struct MergePlan {
+    bool ok, blockwide;
+    int tw;
+    size_t lds;
+};
+MergePlan merge_plan(const ConvGeom& g) {
+    const int C = (int)g.C, Kh = (int)g.Kh, Kw = (int)g.Kw, Sw = (int)g.Sw;
     const int tw_max = g.Nw < 16 ? (int)g.Nw : 16;
     int tw = tw_max;
-    while (tw > 1 && merge_lds_bytes((int)g.C, (int)g.Kh, (int)g.Kw, (int)g.Sw, tw) > 52 * 1024) --tw;
+    while (tw > 1 && merge_lds_bytes(C, Kh, Kw, Sw, tw) > 52 * 1024) --tw;
     if (tw < 2) {
+        // one workgroup per CU: worth it while the tile stays wide (3 x 3 x 128: 16 patches; with 256
+        // channels only 4 would fit, and the block-wide form below is faster: 145 against 186 us at 14 x 14)
         tw = tw_max;
-        while (tw > 1 && merge_lds_bytes((int)g.C, (int)g.Kh, (int)g.Kw, (int)g.Sw, tw) > MERGE_LDS_CAP) --tw;
+        while (tw > 1 && merge_lds_bytes(C, Kh, Kw, Sw, tw) > MERGE_LDS_CAP) --tw;
+        if (tw < (tw_max < 8 ? tw_max : 8)) tw = 1;
     }
-    return tw;
+    if (tw >= 2 && merge_lds_bytes(C, Kh, Kw, Sw, tw) <= MERGE_LDS_CAP)
+        return MergePlan{true, false, tw, merge_lds_bytes(C, Kh, Kw, Sw, tw)};
+    // (the block-wide form keeps a counter in static LDS next to the dynamic area)
+    constexpr size_t CAP1 = MERGE_LDS_CAP - 64;
+    tw = tw_max;
+    while (tw > 1 && merge_lds_bytes(C, Kh, Kw, Sw, tw, 1) > CAP1) --tw;
+    if (tw >= 2) {
+        const int tiles = ((int)g.Nw + tw - 1) / tw;
+        tw = ((int)g.Nw + tiles - 1) / tiles;
+    }
+    const size_t lds = merge_lds_bytes(C, Kh, Kw, Sw, tw, 1);
+    return MergePlan{tw >= 2 && lds <= CAP1, true, tw, lds};
 }
 
 }  // namespace
@@ -287,8 +384,7 @@ int merge_tile_width(const ConvGeom& g) {
 // footprint within reach; everything else goes through the bitonic network.
 bool merge_sort_supported(const ConvGeom& g) {
     if (g.C < 32 || g.C % NB != 0 || g.C > 4096 || g.Kw < 2 || g.Kh > 255 || g.Kw > 255) return false;
-    const int tw = merge_tile_width(g);
-    return merge_lds_bytes((int)g.C, (int)g.Kh, (int)g.Kw, (int)g.Sw, tw) <= MERGE_LDS_CAP && tw >= 2;
+    return merge_plan(g).ok;
 }
 
 // One-time set-up on device `dev` (the current device): the dynamic-LDS limit of every
@@ -297,8 +393,10 @@ int merge_prepare_device(int dev) {
     static std::atomic<bool> done[kMaxDevices];
     if (dev < 0 || dev >= kMaxDevices) return fail(SNNTC_ERR_UNSUPPORTED, "patch merge: device index %d not supported", dev);
     if (done[dev].load(std::memory_order_acquire)) return SNNTC_OK;
-    SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(merge_patches_kernel),
+    SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(merge_patches_kernel<MERGE_THREADS, false>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)MERGE_LDS_CAP));
+    SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(merge_patches_kernel<MERGE_BLOCKWIDE_THREADS, true>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)MERGE_LDS_CAP - 64));
     done[dev].store(true, std::memory_order_release);
     return SNNTC_OK;
 }
@@ -306,8 +404,9 @@ int merge_prepare_device(int dev) {
 int launch_merge_patches(const float* pix_z, const int32_t* pix_c, int64_t Cs, float* sorted, int32_t* perm,
                          int32_t* n_real, const ConvGeom& g, int64_t stride, float max_cmp,
                          hipStream_t stream) {
-    const int tw = merge_tile_width(g);
-    const size_t lds = merge_lds_bytes((int)g.C, (int)g.Kh, (int)g.Kw, (int)g.Sw, tw);
+    const MergePlan plan = merge_plan(g);
+    const int tw = plan.tw;
+    const size_t lds = plan.lds;
     const int tiles_w = (int)((g.Nw + tw - 1) / tw);
     const int64_t blocks = g.B * g.Nh * tiles_w;
     if (blocks > 0x7fffffffLL) return fail(SNNTC_ERR_TOO_LARGE, "patch merge: grid too large");
@@ -323,9 +422,16 @@ int launch_merge_patches(const float* pix_z, const int32_t* pix_c, int64_t Cs, f
     if (prep) return prep;
     {
         KernelTimerScope timer_("merge_patches", stream);
-        hipLaunchKernelGGL(merge_patches_kernel, dim3((unsigned)blocks), dim3(MERGE_THREADS), lds, stream, pix_z, pix_c, (int)Cs,
-                           sorted, perm, n_real, (int)g.H, (int)g.W, (int)g.C, (int)g.Kh, (int)g.Kw, (int)g.Sh,
-                           (int)g.Sw, (int)g.Nh, (int)g.Nw, tw, tiles_w, (int)stride, max_cmp, c4_shift, magic);
+        if (plan.blockwide)
+            hipLaunchKernelGGL((merge_patches_kernel<MERGE_BLOCKWIDE_THREADS, true>), dim3((unsigned)blocks),
+                               dim3(MERGE_BLOCKWIDE_THREADS), lds, stream, pix_z, pix_c, (int)Cs, sorted, perm, n_real,
+                               (int)g.H, (int)g.W, (int)g.C, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.Nh,
+                               (int)g.Nw, tw, tiles_w, (int)stride, max_cmp, c4_shift, magic);
+        else
+            hipLaunchKernelGGL((merge_patches_kernel<MERGE_THREADS, false>), dim3((unsigned)blocks), dim3(MERGE_THREADS),
+                               lds, stream, pix_z, pix_c, (int)Cs, sorted, perm, n_real, (int)g.H, (int)g.W, (int)g.C,
+                               (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.Nh, (int)g.Nw, tw, tiles_w,
+                               (int)stride, max_cmp, c4_shift, magic);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;

@@ -193,6 +193,10 @@ CONV_CASES = [
     (9, 2, 9, 9, 32, 16, 3, 3, 2, 2, True, False, "baseline"),      # stride 2 with 32 channels
     (10, 1, 12, 7, 40, 8, 2, 3, 1, 2, False, True, "reftest"),      # VALID, ragged kernel and stride
     (11, 1, 3, 4, 1024, 24, 3, 3, 1, 1, True, True, "baseline"),    # P = 9216: patches longer than one sorting network
+    # patches whose merge buffers fit in LDS only once per workgroup (merged by all its wavefronts together)
+    (12, 2, 7, 7, 512, 8, 3, 3, 1, 1, True, True, "baseline"),      # rows of 7 patches: tiles of 4 and 3
+    (13, 1, 6, 9, 512, 8, 3, 2, 2, 2, False, True, "reftest"),      # VALID, stride 2, two-column kernel
+    (14, 1, 4, 5, 640, 8, 3, 3, 1, 1, True, False, "reftest"),      # channel count not a power of two, P = 5760
 ]
 
 
@@ -223,7 +227,8 @@ def test_conv_forward_backward(seed, B, H, W, C, Kc, Kh, Kw, Sh, Sw, same, bias,
     assert np.all(dp == 0)
 
 
-@pytest.mark.parametrize("C,Kh,Kw,Sh,Sw", [(32, 3, 3, 1, 1), (64, 3, 3, 1, 1), (3, 3, 3, 1, 1), (40, 2, 3, 1, 2)])
+@pytest.mark.parametrize("C,Kh,Kw,Sh,Sw", [(32, 3, 3, 1, 1), (64, 3, 3, 1, 1), (3, 3, 3, 1, 1), (40, 2, 3, 1, 2),
+                                           (512, 3, 3, 1, 1)])
 def test_conv_sort_with_heavy_ties(C, Kh, Kw, Sh, Sw):
     """Quantised inputs: most values repeat inside a patch (and SAME padding adds runs of 1e5), so
     the permutation is decided by the stable tie rule (kh, kw, c) almost everywhere."""
