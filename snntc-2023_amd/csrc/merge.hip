@@ -351,6 +351,7 @@ struct MergePlan {
     bool ok, blockwide;
     int tw;
     size_t lds;
+    int waves = MERGE_WAVES;                               // wavefronts of a workgroup (each with a buffer pair)
 };
 MergePlan merge_plan(const ConvGeom& g) {
     const int C = (int)g.C, Kh = (int)g.Kh, Kw = (int)g.Kw, Sw = (int)g.Sw;
@@ -360,6 +361,17 @@ MergePlan merge_plan(const ConvGeom& g) {
     if (tw < 2) {
         // one workgroup per CU: worth it while the tile stays wide (3 x 3 x 128: 16 patches; with 256
         // channels only 4 would fit, and the block-wide form below is faster: 145 against 186 us at 14 x 14)
+        // (with eight wavefronts if their buffer pairs leave room for tiles of eight patches: 3 x 3 x 128 at
+        // 28 x 28, 32 images: 237 against 318 us with four)
+        int tw8 = tw_max;
+        while (tw8 > 1 && merge_lds_bytes(C, Kh, Kw, Sw, tw8, 8) > MERGE_LDS_CAP) --tw8;
+        if (tw8 >= (tw_max < 8 ? tw_max : 8)) {
+            const int tiles = ((int)g.Nw + tw8 - 1) / tw8;
+            tw8 = ((int)g.Nw + tiles - 1) / tiles;
+            MergePlan p8{true, false, tw8, merge_lds_bytes(C, Kh, Kw, Sw, tw8, 8)};
+            p8.waves = 8;
+            return p8;
+        }
         tw = tw_max;
         while (tw > 1 && merge_lds_bytes(C, Kh, Kw, Sw, tw) > MERGE_LDS_CAP) --tw;
         if (tw < (tw_max < 8 ? tw_max : 8)) tw = 1;
@@ -395,6 +407,8 @@ int merge_prepare_device(int dev) {
     if (done[dev].load(std::memory_order_acquire)) return SNNTC_OK;
     SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(merge_patches_kernel<MERGE_THREADS, false>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)MERGE_LDS_CAP));
+    SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(merge_patches_kernel<2 * MERGE_THREADS, false>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)MERGE_LDS_CAP));
     SNNTC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(merge_patches_kernel<MERGE_BLOCKWIDE_THREADS, true>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)MERGE_LDS_CAP - 64));
     done[dev].store(true, std::memory_order_release);
@@ -427,6 +441,11 @@ int launch_merge_patches(const float* pix_z, const int32_t* pix_c, int64_t Cs, f
                                dim3(MERGE_BLOCKWIDE_THREADS), lds, stream, pix_z, pix_c, (int)Cs, sorted, perm, n_real,
                                (int)g.H, (int)g.W, (int)g.C, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.Nh,
                                (int)g.Nw, tw, tiles_w, (int)stride, max_cmp, c4_shift, magic);
+        else if (plan.waves == 2 * MERGE_WAVES)
+            hipLaunchKernelGGL((merge_patches_kernel<2 * MERGE_THREADS, false>), dim3((unsigned)blocks),
+                               dim3(2 * MERGE_THREADS), lds, stream, pix_z, pix_c, (int)Cs, sorted, perm, n_real, (int)g.H,
+                               (int)g.W, (int)g.C, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.Nh, (int)g.Nw, tw,
+                               tiles_w, (int)stride, max_cmp, c4_shift, magic);
         else
             hipLaunchKernelGGL((merge_patches_kernel<MERGE_THREADS, false>), dim3((unsigned)blocks), dim3(MERGE_THREADS),
                                lds, stream, pix_z, pix_c, (int)Cs, sorted, perm, n_real, (int)g.H, (int)g.W, (int)g.C,
