@@ -342,6 +342,8 @@ def carried_counters(workload_key, kernel):
     except (OSError, ValueError):
         return {}
     entry = dict(table.get("workloads", {}).get(workload_key, {}).get(kernel, {}))
+    if "valu_busy" in entry:                 # share of the SIMDs' issue slots that hold a vector instruction
+        entry["valu_busy"] = min(1.0, entry["valu_busy"])
     if entry:
         entry["source"] = f"profiles/counters.json at commit {table.get('commit', '?')}"
     return entry

@@ -72,9 +72,9 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
     extern __shared__ __align__(16) float staged[];      // per wavefront: [2][n_slots + 1][KCB]; ksplit = 4: then `partial`
     constexpr int SPAN = DX_TILE * HALVES;               // pixels of one wavefront
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    // ksplit = 1: a tile per single-wavefront workgroup.  ksplit = 4 (layers with few tiles and many
-    // output channels): a tile per workgroup of four, its wavefronts take a quarter of the output
-    // channels each and their sums are added in wavefront order.
+    // ksplit = 1: a tile per single-wavefront workgroup.  ksplit = 2 or 4 (layers with few tiles and many
+    // output channels): a tile per workgroup of that many wavefronts, each takes its share of the output
+    // channels and their sums are added in wavefront order.
     // Items are (image, row, tile, channel block).  When the last tile of a row is a partial one, those
     // tiles form a second run of workgroups behind all others (`lead_blocks` workgroups, a multiple of
     // the XCD count, hold the `lead_items` others), so that the launch ends on its shortest items and
@@ -211,7 +211,7 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
         }
     }
     if (ksplit > 1) {                                     // block-uniform: all four wavefronts hold the same tile
-        // sums of wavefronts 1..3, [3][DX_TILE][64], behind the staging areas
+        // sums of wavefronts 1..ksplit-1, [ksplit - 1][DX_TILE][64], behind the staging areas
         float* __restrict__ partial = staged + (size_t)(blockDim.x / kWave) * 2 * (n_slots + 1) * KCB;
         if (ks > 0) {
 #pragma unroll
@@ -219,10 +219,10 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
         }
         __syncthreads();
         if (ks > 0) return;
+        for (int v = 1; v < ksplit; ++v) {                // in wavefront order
 #pragma unroll
-        for (int t = 0; t < DX_TILE; ++t)
-            acc[t] = ((acc[t] + partial[t * kWave + lane]) + partial[(DX_TILE + t) * kWave + lane]) +
-                     partial[(2 * DX_TILE + t) * kWave + lane];
+            for (int t = 0; t < DX_TILE; ++t) acc[t] += partial[((v - 1) * DX_TILE + t) * kWave + lane];
+        }
     }
     // only the pixels inside the caller's window of the padded image are stored
     if (lane_ok) {
@@ -492,12 +492,15 @@ int launch_cv_grad_input_chan(const float* xpad, const float* wq, const float* u
     // (Up to 1024 tiles per image: with 256 output channels a tile's wavefront walks 36 taps, and at small
     // batches too few tiles exist to hide that -- 256 -> 256 at 16 x 16, one image: 55 against 174 us;
     // at 32 images the split still is a little ahead, 437 against 491 us.)
-    const int ksplit = (halves == 1 && g.H * tiles_w * c_blocks <= 1024 && g.Kc % (4 * kcb) == 0) ? 4 : 1;
+    // With 128 output channels (two chunks) the split is in two: 64 -> 128 at 28 x 28 is 3840 tiles for 32 images,
+    // not quite four per SIMD, and the launch ends on the SIMDs that hold four.
+    const bool few_tiles = halves == 1 && g.H * tiles_w * c_blocks <= 1024;
+    const int ksplit = !few_tiles ? 1 : g.Kc % (4 * kcb) == 0 ? 4 : g.Kc % (2 * kcb) == 0 ? 2 : 1;
     // One item per workgroup.  Without the split a workgroup is a single wavefront: the
     // wavefronts do not cooperate, their running times differ (border tiles, rows outside the window),
     // and a CU takes a new workgroup only when a whole one has left, so in larger workgroups the slots
     // of the early finishers would idle.
-    const int wg_waves = ksplit == 4 ? 4 : 1;
+    const int wg_waves = ksplit;
     // a last tile with at most half its pixels inside the row goes to the end of the launch
     const bool partial_last = tiles_w > 1 && (g.W - (int64_t)(tiles_w - 1) * span) * 2 <= span;
     const int64_t lead_items = partial_last ? g.B * g.H * (tiles_w - 1) * c_blocks : n_items;
@@ -507,7 +510,7 @@ int launch_cv_grad_input_chan(const float* xpad, const float* wq, const float* u
     if (blocks > 0x7fffffffLL) return fail(SNNTC_ERR_TOO_LARGE, "conv backward: grid too large");
     dim3 grid((unsigned)blocks), block(wg_waves * kWave);
     const size_t lds = (size_t)wg_waves * 2 * (span + g.Kw) * kcb * sizeof(float) +
-                       (ksplit == 4 ? (size_t)3 * DX_TILE * kWave * sizeof(float) : 0);
+                       (ksplit > 1 ? (size_t)(ksplit - 1) * DX_TILE * kWave * sizeof(float) : 0);
     void (*kern)(const float*, const float*, const float*, const float*, float*, CropGeom, int, int, int, int, int, int,
                  int, int, int, int, int, int, int64_t, int64_t, int, float, int);
     if (halves == 2)

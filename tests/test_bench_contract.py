@@ -30,7 +30,7 @@ def test_carried_counters_name_their_source():
     sys.path.insert(0, ROOT)
     import bench
     c = bench.carried_counters("cfg3", "scan")
-    assert c["hbm_bytes_per_launch"] > 0 and 0 < c["valu_busy"] <= 1.1 and "commit" in c["source"]
+    assert c["hbm_bytes_per_launch"] > 0 and 0 < c["valu_busy"] <= 1.0 and "commit" in c["source"]
     assert bench.carried_counters("cfg3", "no_such_kernel") == {}
 
 
