@@ -197,6 +197,13 @@ CONV_CASES = [
     (12, 2, 7, 7, 512, 8, 3, 3, 1, 1, True, True, "baseline"),      # rows of 7 patches: tiles of 4 and 3
     (13, 1, 6, 9, 512, 8, 3, 2, 2, 2, False, True, "reftest"),      # VALID, stride 2, two-column kernel
     (14, 1, 4, 5, 640, 8, 3, 3, 1, 1, True, False, "reftest"),      # channel count not a power of two, P = 5760
+    # few input channels and patches of at least 64 entries: the patch order comes from counts shared between
+    # neighbouring patches
+    (15, 2, 40, 37, 3, 16, 7, 7, 2, 2, True, True, "baseline"),     # the 7x7/2 stem on an odd image: partial last tiles
+    (16, 2, 12, 12, 1, 8, 8, 8, 1, 1, True, True, "reftest"),       # one channel
+    (17, 1, 9, 20, 16, 8, 3, 3, 1, 1, False, True, "reftest"),      # 16 channels, VALID
+    (18, 1, 10, 9, 31, 8, 8, 2, 1, 1, True, False, "reftest"),      # columns of 248 entries
+    (19, 2, 9, 30, 8, 8, 3, 3, 2, 5, False, True, "reftest"),       # stride wider than the kernel: no shared columns
 ]
 
 
@@ -228,6 +235,7 @@ def test_conv_forward_backward(seed, B, H, W, C, Kc, Kh, Kw, Sh, Sw, same, bias,
 
 
 @pytest.mark.parametrize("C,Kh,Kw,Sh,Sw", [(32, 3, 3, 1, 1), (64, 3, 3, 1, 1), (3, 3, 3, 1, 1), (40, 2, 3, 1, 2),
+                                           (3, 7, 7, 2, 2), (8, 3, 5, 1, 2),
                                            (128, 3, 3, 1, 1), (256, 3, 3, 1, 1), (512, 3, 3, 1, 1)])
 def test_conv_sort_with_heavy_ties(C, Kh, Kw, Sh, Sw):
     """Quantised inputs: most values repeat inside a patch (and SAME padding adds runs of 1e5), so
