@@ -485,7 +485,7 @@ int launch_cv_grad_input_chan(const float* xpad, const float* wq, const float* u
     const int tiles_w = (int)((g.W + span - 1) / span);
     const int c_blocks = halves == 2 ? 1 : (int)((g.C + kWave - 1) / kWave);
     const int64_t n_items = g.B * g.H * tiles_w * c_blocks;
-    const int kcb = g.Kc % 64 == 0 ? 64 : (g.Kc % 32 == 0 ? 32 : 16);
+    int kcb = g.Kc % 64 == 0 ? 64 : (g.Kc % 32 == 0 ? 32 : 16);
     // small images with at least four chunks of output channels: split the channels over the
     // wavefronts of a workgroup.  Decided by the layer's geometry alone, never by the batch: the
     // order of the additions, and with it the last bits of dX, must not depend on the batch size.
@@ -494,8 +494,10 @@ int launch_cv_grad_input_chan(const float* xpad, const float* wq, const float* u
     // at 32 images the split still is a little ahead, 437 against 491 us.)
     // With 128 output channels (two chunks) the split is in two: 64 -> 128 at 28 x 28 is 3840 tiles for 32 images,
     // not quite four per SIMD, and the launch ends on the SIMDs that hold four.
-    const bool few_tiles = halves == 1 && g.H * tiles_w * c_blocks <= 1024;
-    const int ksplit = !few_tiles ? 1 : g.Kc % (4 * kcb) == 0 ? 4 : g.Kc % (2 * kcb) == 0 ? 2 : 1;
+    // Layers with at most 32 input channels and 64 output channels on small images: two chunks of 32.
+    const bool few_tiles = g.H * tiles_w * c_blocks <= 1024;
+    if (halves == 2 && few_tiles && g.Kc == 64) kcb = 32;
+    const int ksplit = !few_tiles ? 1 : (halves == 1 && g.Kc % (4 * kcb) == 0) ? 4 : g.Kc % (2 * kcb) == 0 ? 2 : 1;
     // One item per workgroup.  Without the split a workgroup is a single wavefront: the
     // wavefronts do not cooperate, their running times differ (border tiles, rows outside the window),
     // and a CU takes a new workgroup only when a whole one has left, so in larger workgroups the slots

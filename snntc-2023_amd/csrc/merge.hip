@@ -365,7 +365,7 @@ MergePlan merge_plan(const ConvGeom& g) {
         // 28 x 28, 32 images: 237 against 318 us with four)
         int tw8 = tw_max;
         while (tw8 > 1 && merge_lds_bytes(C, Kh, Kw, Sw, tw8, 8) > MERGE_LDS_CAP) --tw8;
-        if (tw8 >= (tw_max < 8 ? tw_max : 8)) {
+        if (tw8 >= 2 && tw8 >= (tw_max < 8 ? tw_max : 8) && merge_lds_bytes(C, Kh, Kw, Sw, tw8, 8) <= MERGE_LDS_CAP) {
             const int tiles = ((int)g.Nw + tw8 - 1) / tw8;
             tw8 = ((int)g.Nw + tiles - 1) / tiles;
             MergePlan p8{true, false, tw8, merge_lds_bytes(C, Kh, Kw, Sw, tw8, 8)};

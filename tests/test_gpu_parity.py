@@ -204,6 +204,7 @@ CONV_CASES = [
     (17, 1, 9, 20, 16, 8, 3, 3, 1, 1, False, True, "reftest"),      # 16 channels, VALID
     (18, 1, 10, 9, 31, 8, 8, 2, 1, 1, True, False, "reftest"),      # columns of 248 entries
     (19, 2, 9, 30, 8, 8, 3, 3, 2, 5, False, True, "reftest"),       # stride wider than the kernel: no shared columns
+    (20, 2, 13, 7, 96, 4, 3, 6, 3, 2, False, True, "reftest"),      # many channels, a single patch per output row
 ]
 
 
