@@ -828,11 +828,12 @@ __device__ __forceinline__ void read_columns(__attribute__((address_space(3))) c
 // neuron cannot have fired) and falls while wsum > 0: in exact arithmetic the causal set closes
 // at the first step where D reaches zero.  In fp32 the reference's own tests (products rounded
 // on their own, sign-corrected compares) can disagree with the sign of D only while |D| is
-// within a few ulp of the quantities compared.  So a chunk of eight inputs runs as
-//     wsum += w ; ysum = fma(x, w, ysum) ; t = fma(-x, wsum, ysum)          (3 instructions)
-// and the minimum of the eight t is compared once with
+// within a few ulp of the quantities compared.  So a chunk of eight inputs only accumulates,
+//     wsum += w ; ysum = fma(x, w, ysum),
+// and is accepted as a whole if t_u = fma(-x_u, wsum_u, ysum_u) is known to lie above
 //     thr = 4u * |ysum_end| + 36u * x_last * max|w|        (u = 2^-24)
-// If the minimum is above thr (and the chunk's first input is not negative) none of the
+// after each of its inputs (filter_chunk bounds the eight t from the last one, see there).
+// If they all are above thr (and the chunk's first input is not negative) none of the
 // reference's tests before the chunk's eight inputs can close the set:
 //   * wsum_{k-1} > 0: closing before input k needs ysum_{k-1} <= x_k*wsum_{k-1}*(1+u); the sums
 //     after input k differ from those before by the input and two roundings, which puts D_k
@@ -846,7 +847,7 @@ __device__ __forceinline__ void read_columns(__attribute__((address_space(3))) c
 // records the chunk and sits out; after the loop every lane evaluates its recorded chunk with
 // the reference's tests (the eight-step block above, fed per lane), which finds the close in
 // all but contrived cases, and otherwise walks on step by step.  NaN sums never pass a
-// reference test and never close; a NaN minimum or threshold fails the fast test.
+// reference test and never close; a NaN bound or threshold fails the fast test.
 //
 // CH (1 or 2) adjacent neurons per lane: one row address and one 4- or 8-byte LDS read serve CH
 // scans, and a wavefront covers 64*CH/COLS segments.  Workgroups, slices and items are laid out as
@@ -854,22 +855,44 @@ __device__ __forceinline__ void read_columns(__attribute__((address_space(3))) c
 // ---------------------------------------------------------------------------------------------
 constexpr float FILTER_REL = 0x1p-22f;                    // 4u
 constexpr float FILTER_W = 9.0f * 0x1p-22f;               // 36u, times max|w| of the slice
+// The fast loop does not evaluate the eight t of a chunk: it bounds them from the last one.  With the
+// sums as computed, D_u = ysum_u - x_u*wsum_u obeys  D_{u-1} = D_u + (x_u - x_{u-1})*wsum_{u-1} - e_u,
+// |e_u| <= u*(|ysum_u| + x_u*|wsum_u|) (the roundings of the two sums), hence for every u of the chunk
+//     D_u >= D_7 + (x_7 - x_0) * min(0, wsum_0 .. wsum_7) - 7 * max|e|:
+// D only falls while the weight sum is positive, and where the sum is negative it can have been lower
+// earlier by at most that much.  The lane keeps the smallest weight sum of the chunk (one three-way
+// minimum per two inputs, started at zero), evaluates t_7 and accepts the chunk if
+//     fma(x_7 - x_0, min, t_7)  >  thr + 12u * 1.01 * (|ysum_7| + x_7*|wsum_7| + 14*x_7*max|w|)
+// (the second term covers the seven e_u, the roundings of t_u, t_7, x_7 - x_0 and of the bound itself;
+// sums inside the chunk differ from the final ones by at most seven inputs).  Every t_u then exceeds
+// thr, which is the condition above.  With a weight sum that stays positive the bound is t_7 itself, so
+// a chunk fails exactly where it failed before, give or take the wider margin (a few 10^-6 of the sums).
+// Two additions, one half of a minimum per input instead of three and a half instructions.
+constexpr float FILTER_END_Y = 0x1p-19f;                  // 32u >= 4u + 12.2u, times |ysum_7|
+constexpr float FILTER_END_XW = 0x1p-20f;                 // 16u >= 12.2u, times x_7 * |wsum_7|
+constexpr float FILTER_END_W = 0x1p-16f;                  // 256u >= 36u + 170u, times x_7 * max|w| of the slice
 
 // Eight inputs for one scan of every lane.  Lanes in the mask `open` that pass the test keep the new
 // sums; open lanes that fail keep the old ones, take the chunk's first index as kflag and leave
 // `open`.  The arithmetic does not depend on EXEC or branches (lanes that are not open compute along
 // and discard), so the compiler is free to interleave it with the LDS traffic of the next chunk; the
 // decision works on lane masks in scalar registers: one compare, three mask operations, three selects.
+// dx = x[7] - x[0], x7s = FILTER_END_XW * x[7], thrx = FILTER_END_W * max|w| * x[7].
 __device__ __forceinline__ void filter_chunk(float& wsum, float& ysum, int& kflag, uint64_t& open, int k, float thrx,
-                                             const float (&x)[CHUNK], const float (&w)[CHUNK]) {
-    float wb = wsum, yb = ysum, m = INFINITY;
+                                             float dx, float x7s, const float (&x)[CHUNK], const float (&w)[CHUNK]) {
+    float wb = wsum, yb = ysum, m = 0.0f;
 #pragma unroll
-    for (int u = 0; u < CHUNK; ++u) {
+    for (int u = 0; u < CHUNK; u += 2) {
         wb += w[u];
         yb = __fmaf_rn(x[u], w[u], yb);
-        m = fminf(m, __fmaf_rn(-x[u], wb, yb));
+        const float w0 = wb;
+        wb += w[u + 1];
+        yb = __fmaf_rn(x[u + 1], w[u + 1], yb);
+        m = fminf(fminf(m, w0), wb);
     }
-    const float thr = __fmaf_rn(FILTER_REL, fabsf(yb), thrx);
+    const float t7 = __fmaf_rn(-x[CHUNK - 1], wb, yb);
+    const float bound = __fmaf_rn(dx, m, t7);
+    const float thr = __fmaf_rn(FILTER_END_Y, fabsf(yb), __fmaf_rn(x7s, fabsf(wb), thrx));
     uint64_t stop;
     // (two statements: the first has scalar results only, so the masks stay uniform values for the compiler
     // also where no branch depends on them)
@@ -877,7 +900,7 @@ __device__ __forceinline__ void filter_chunk(float& wsum, float& ysum, int& kfla
         "s_andn2_b64 %[stop], %[open], vcc\n"
         "s_and_b64 %[open], %[open], vcc\n"
         : [open] "+s"(open), [stop] "=&s"(stop)
-        : [m] "v"(m), [thr] "v"(thr)
+        : [m] "v"(bound), [thr] "v"(thr)
         : "vcc", "scc");
     asm("v_cndmask_b32_e64 %[ws], %[ws], %[wb], %[open]\n"
         "v_cndmask_b32_e64 %[ys], %[ys], %[yb], %[open]\n"
@@ -968,7 +991,9 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
     const int j0 = slice * COLS;
     const int rows = I + np.bias;
     // the slice, and the largest |w| in it (the threads' shares of the copy, then the workgroup's)
-    const float thr_w = FILTER_W * block_max(fill_weight_slice<COLS>(wl, w, rows, J, j0), wl + rows * COLS);
+    const float w_max = block_max(fill_weight_slice<COLS>(wl, w, rows, J, j0), wl + rows * COLS);
+    const float thr_w = FILTER_W * w_max;                   // margin of the accumulate-only rounds below
+    const float end_w = FILTER_END_W * w_max;               // margin of the fast loop
 
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -1143,10 +1168,11 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
                         x[4] = __int_as_float(quad_broadcast<0>(xh)); x[5] = __int_as_float(quad_broadcast<1>(xh));
                         x[6] = __int_as_float(quad_broadcast<2>(xh)); x[7] = __int_as_float(quad_broadcast<3>(xh));
                     }
-                    const float thrx = x[CHUNK - 1] * thr_w;
+                    const float thrx = x[CHUNK - 1] * end_w, x7s = x[CHUNK - 1] * FILTER_END_XW;
+                    const float dx = x[CHUNK - 1] - x[0];
 #pragma unroll
                     for (int c = 0; c < CH; ++c)
-                        filter_chunk(wsum[c], ysum[c], kflag[c], open[c], k, thrx, x, wv[ph % 2][c]);
+                        filter_chunk(wsum[c], ysum[c], kflag[c], open[c], k, thrx, dx, x7s, x, wv[ph % 2][c]);
                 };
                 for (int k0 = kmin;; k0 += RING * CHUNK) {
                     rotate_wave_priority(k0 / (RING * CHUNK) + (wave >> 2));
