@@ -21,41 +21,47 @@ namespace {
 // rows of the TILE + Kw - 1 patches one kernel row can touch are staged in a wavefront-private
 // piece of LDS (lane = output channel while staging) and read back as broadcasts, four output
 // channels per read.  Gather form: no atomics, fixed summation order.
+//
+// The mask x <= ym is evaluated arithmetically (dx_mac8).  That is exact while MAX_SPIKE_TIME is at
+// most 2^86 and no two unequal spike times lie closer together than 1 / dx_mask_scale (2^-109 for
+// MAX_SPIKE_TIME = 1e5): differences that small exist only between values below 2^-85.
 // ---------------------------------------------------------------------------------------------
 constexpr int DX_TILE = 8;
 
-// Sixteen masked MACs  acc += upm_k * (x <= ym_k ? w_k : 0).  ym_k arrive as broadcast LDS reads; the
-// sixteen upm_k sit in ONE register (lane r of every row of 16 lanes holds upm of channel r) and
-// are fed to the FMA through its DPP row broadcast, which costs no instruction and no LDS
-// bandwidth -- with both operands read as broadcasts the kernel was bound by the LDS pipe.
-// Two temporaries alternate so that a DPP instruction never reads a register written by one of
-// the two instructions before it.
-#define SNNTC_DX_SEL(K, T)                                  \
-    "v_cmp_le_f32_e32 vcc, %[x], %[y" #K "]\n"              \
-    "v_cndmask_b32_e32 %[" #T "], 0, %[w" #K "], vcc\n"
-#define SNNTC_DX_FMA(K, T) \
-    "v_fmac_f32_dpp %[acc], %[u], %[" #T "] row_newbcast:" #K " row_mask:0xf bank_mask:0xf\n"
+// Eight masked MACs  acc += upm_k * (x <= ym_k ? w_k : 0)  without a compare or a select: with
+//   m = clamp01(x * BIG - ym_k * BIG)       (one fused multiply-add with the clamp output modifier)
+// m is exactly 1 where x > ym_k and exactly 0 where x <= ym_k: the fused operation rounds the exact
+// value of (x - ym_k) * BIG, whose sign is that of x - ym_k, and BIG (dx_mask_scale) is large enough
+// that the smallest difference two unequal spike times can have maps to at least 1 while MAX * BIG stays finite.
+// Then t = w_k - m * w_k is w_k or 0 (both exact) and acc += upm_k * t.  All three are plain
+// multiply-adds on vector registers, which this chip issues faster than compares, selects and DPP
+// operands (about 2.8 against 4.2 cycles each with several wavefronts per SIMD).  ny_k = -ym_k * BIG
+// (+inf for outputs that take no part, so m = 1) and upm_k arrive as broadcast LDS reads.  The
+// schedule keeps every result two other instructions away from its first use.
+#define SNNTC_DX_M(K, T) "v_fma_f32 %[" #T "], %[x], %[big], %[y" #K "] clamp\n"
+#define SNNTC_DX_T(K, T) "v_fma_f32 %[" #T "], -%[" #T "], %[w" #K "], %[w" #K "]\n"
+#define SNNTC_DX_F(K, T) "v_fmac_f32_e32 %[acc], %[u" #K "], %[" #T "]\n"
 
-__device__ __forceinline__ void dx_mac16(float& acc, float x, float u, const float (&y)[16], const float* w) {
-    float ta, tb;
+__device__ __forceinline__ void dx_mac8(float& acc, float x, float big, const float* u, const float* y,
+                                        const float* w) {
+    float ta, tb, tc;
     asm volatile(
-        SNNTC_DX_SEL(0, ta) SNNTC_DX_SEL(1, tb) SNNTC_DX_FMA(0, ta)
-        SNNTC_DX_SEL(2, ta) SNNTC_DX_FMA(1, tb) SNNTC_DX_SEL(3, tb) SNNTC_DX_FMA(2, ta)
-        SNNTC_DX_SEL(4, ta) SNNTC_DX_FMA(3, tb) SNNTC_DX_SEL(5, tb) SNNTC_DX_FMA(4, ta)
-        SNNTC_DX_SEL(6, ta) SNNTC_DX_FMA(5, tb) SNNTC_DX_SEL(7, tb) SNNTC_DX_FMA(6, ta)
-        SNNTC_DX_SEL(8, ta) SNNTC_DX_FMA(7, tb) SNNTC_DX_SEL(9, tb) SNNTC_DX_FMA(8, ta)
-        SNNTC_DX_SEL(10, ta) SNNTC_DX_FMA(9, tb) SNNTC_DX_SEL(11, tb) SNNTC_DX_FMA(10, ta)
-        SNNTC_DX_SEL(12, ta) SNNTC_DX_FMA(11, tb) SNNTC_DX_SEL(13, tb) SNNTC_DX_FMA(12, ta)
-        SNNTC_DX_SEL(14, ta) SNNTC_DX_FMA(13, tb) SNNTC_DX_SEL(15, tb) SNNTC_DX_FMA(14, ta)
-        "s_nop 1\n" SNNTC_DX_FMA(15, tb)
-        : [acc] "+v"(acc), [ta] "=&v"(ta), [tb] "=&v"(tb)
-        : [x] "v"(x), [u] "v"(u), [y0] "v"(y[0]), [y1] "v"(y[1]), [y2] "v"(y[2]), [y3] "v"(y[3]), [y4] "v"(y[4]),
-          [y5] "v"(y[5]), [y6] "v"(y[6]), [y7] "v"(y[7]), [y8] "v"(y[8]), [y9] "v"(y[9]), [y10] "v"(y[10]),
-          [y11] "v"(y[11]), [y12] "v"(y[12]), [y13] "v"(y[13]), [y14] "v"(y[14]), [y15] "v"(y[15]),
-          [w0] "v"(w[0]), [w1] "v"(w[1]), [w2] "v"(w[2]), [w3] "v"(w[3]), [w4] "v"(w[4]), [w5] "v"(w[5]),
-          [w6] "v"(w[6]), [w7] "v"(w[7]), [w8] "v"(w[8]), [w9] "v"(w[9]), [w10] "v"(w[10]), [w11] "v"(w[11]),
-          [w12] "v"(w[12]), [w13] "v"(w[13]), [w14] "v"(w[14]), [w15] "v"(w[15])
-        : "vcc");
+        SNNTC_DX_M(0, ta)
+        SNNTC_DX_M(1, tb) SNNTC_DX_T(0, ta)
+        SNNTC_DX_M(2, tc) SNNTC_DX_T(1, tb) SNNTC_DX_F(0, ta)
+        SNNTC_DX_M(3, ta) SNNTC_DX_T(2, tc) SNNTC_DX_F(1, tb)
+        SNNTC_DX_M(4, tb) SNNTC_DX_T(3, ta) SNNTC_DX_F(2, tc)
+        SNNTC_DX_M(5, tc) SNNTC_DX_T(4, tb) SNNTC_DX_F(3, ta)
+        SNNTC_DX_M(6, ta) SNNTC_DX_T(5, tc) SNNTC_DX_F(4, tb)
+        SNNTC_DX_M(7, tb) SNNTC_DX_T(6, ta) SNNTC_DX_F(5, tc)
+        SNNTC_DX_T(7, tb) SNNTC_DX_F(6, ta)
+        SNNTC_DX_F(7, tb)
+        : [acc] "+v"(acc), [ta] "=&v"(ta), [tb] "=&v"(tb), [tc] "=&v"(tc)
+        : [x] "v"(x), [big] "v"(big), [y0] "v"(y[0]), [y1] "v"(y[1]), [y2] "v"(y[2]), [y3] "v"(y[3]), [y4] "v"(y[4]),
+          [y5] "v"(y[5]), [y6] "v"(y[6]), [y7] "v"(y[7]), [u0] "v"(u[0]), [u1] "v"(u[1]), [u2] "v"(u[2]),
+          [u3] "v"(u[3]), [u4] "v"(u[4]), [u5] "v"(u[5]), [u6] "v"(u[6]), [u7] "v"(u[7]), [w0] "v"(w[0]),
+          [w1] "v"(w[1]), [w2] "v"(w[2]), [w3] "v"(w[3]), [w4] "v"(w[4]), [w5] "v"(w[5]), [w6] "v"(w[6]),
+          [w7] "v"(w[7]));
 }
 
 // HALVES = 2 is for layers with at most 32 input channels: the two halves of a wavefront take the
@@ -68,7 +74,7 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
                           const float* __restrict__ upm, const float* __restrict__ ym,
                           float* __restrict__ dx, CropGeom crop, int H, int W, int C, int Kc, int Kh, int Kw, int Sh,
                           int Sw, int Nh, int Nw, int tiles_w, int c_blocks, int64_t n_items, int64_t lead_items,
-                          int lead_blocks, float max_cmp, int ksplit) {
+                          int lead_blocks, float max_cmp, int ksplit, float big) {
     extern __shared__ __align__(16) float staged[];      // per wavefront: [2][n_slots + 1][KCB]; ksplit = 4: then `partial`
     constexpr int SPAN = DX_TILE * HALVES;               // pixels of one wavefront
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -103,7 +109,7 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
     float* __restrict__ ys = staged + (size_t)wave * 2 * (n_slots + 1) * KCB;
     float* __restrict__ us = ys + (n_slots + 1) * KCB;
     if (lane < KCB) {                                    // the spare slot
-        ys[n_slots * KCB + lane] = -INFINITY;
+        ys[n_slots * KCB + lane] = INFINITY;             // in the scaled form the loop below produces
         us[n_slots * KCB + lane] = 0.0f;
     }
 
@@ -162,6 +168,15 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
                 __builtin_amdgcn_wave_barrier();
+                // ym -> -ym * BIG, the operand of dx_mac8 (-inf, an output that takes no part, becomes +inf);
+                // slots that were not loaded hold anything and are never read
+                for (int i = lane; i < n_slots * (KCB / 4); i += kWave) {
+                    float4 v4 = reinterpret_cast<float4*>(ys)[i];
+                    v4.x *= -big; v4.y *= -big; v4.z *= -big; v4.w *= -big;
+                    reinterpret_cast<float4*>(ys)[i] = v4;
+                }
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                __builtin_amdgcn_wave_barrier();
                 for (int kw = 0; kw < Kw; ++kw) {
                     // wq[tap][kc / 4][c][kc % 4]: the 16-byte pieces the lanes fetch together are
                     // neighbours in memory
@@ -182,28 +197,20 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
                         if (HALVES == 1) slot = __builtin_amdgcn_readfirstlane(slot);   // same for every lane
                         const float* __restrict__ yrow = ys + slot * KCB;
                         const float* __restrict__ urow = us + slot * KCB;
-                        // groups of 16 output channels; the operands of the next group are read
-                        // while the current one computes
-                        float yq[2][16], u16[2];
-#pragma unroll
-                        for (int v = 0; v < 16; v += 4) {
-                            const float4 y4 = *reinterpret_cast<const float4*>(yrow + v);
-                            yq[0][v] = y4.x; yq[0][v + 1] = y4.y; yq[0][v + 2] = y4.z; yq[0][v + 3] = y4.w;
-                        }
-                        u16[0] = urow[lane & 15];             // lane r of every row of 16: upm of channel q+r
+                        // groups of 16 output channels: eight broadcast reads, then 48 multiply-adds
 #pragma unroll
                         for (int g = 0; g < KCB / 16; ++g) {
-                            if (g + 1 < KCB / 16) {
+                            float yq[16], uq[16];
 #pragma unroll
-                                for (int v = 0; v < 16; v += 4) {
-                                    const float4 y4 = *reinterpret_cast<const float4*>(yrow + (g + 1) * 16 + v);
-                                    yq[(g + 1) & 1][v] = y4.x; yq[(g + 1) & 1][v + 1] = y4.y;
-                                    yq[(g + 1) & 1][v + 2] = y4.z; yq[(g + 1) & 1][v + 3] = y4.w;
-                                }
-                                u16[(g + 1) & 1] = urow[(g + 1) * 16 + (lane & 15)];
+                            for (int v = 0; v < 16; v += 4) {
+                                const float4 y4 = *reinterpret_cast<const float4*>(yrow + g * 16 + v);
+                                const float4 u4 = *reinterpret_cast<const float4*>(urow + g * 16 + v);
+                                yq[v] = y4.x; yq[v + 1] = y4.y; yq[v + 2] = y4.z; yq[v + 3] = y4.w;
+                                uq[v] = u4.x; uq[v + 1] = u4.y; uq[v + 2] = u4.z; uq[v + 3] = u4.w;
                             }
                             __builtin_amdgcn_sched_barrier(0);
-                            dx_mac16(acc[t], xv[t], u16[g & 1], yq[g & 1], &wreg[g * 16]);
+                            dx_mac8(acc[t], xv[t], big, &uq[0], &yq[0], &wreg[g * 16]);
+                            dx_mac8(acc[t], xv[t], big, &uq[8], &yq[8], &wreg[g * 16 + 8]);
                         }
                     }
                 }
@@ -476,6 +483,16 @@ bool cv_grad_input_chan_supported(const ConvGeom& g) {
            g.Nw * g.Kc * 4 < 0x7fffffffLL;               // an output row of ym / upm behind one buffer descriptor
 }
 
+// The factor BIG of dx_mac8: the largest power of two with MAX_SPIKE_TIME * BIG <= 2^126.
+static float dx_mask_scale(float max_time) {
+    int e = 0;
+    if (max_time > 1.0f) {
+        if (max_time < 0x1p86f) frexpf(max_time, &e);     // max_time < 2^e
+        else e = 86;
+    }
+    return ldexpf(1.0f, 126 - e);
+}
+
 // wq: the weights regrouped by launch_backward_prologue (mode 2)
 int launch_cv_grad_input_chan(const float* xpad, const float* wq, const float* upm, const float* ym,
                               float* dx, const CropGeom& crop, const ConvGeom& g, const NeuronParams& np,
@@ -514,7 +531,7 @@ int launch_cv_grad_input_chan(const float* xpad, const float* wq, const float* u
     const size_t lds = (size_t)wg_waves * 2 * (span + g.Kw) * kcb * sizeof(float) +
                        (ksplit > 1 ? (size_t)(ksplit - 1) * DX_TILE * kWave * sizeof(float) : 0);
     void (*kern)(const float*, const float*, const float*, const float*, float*, CropGeom, int, int, int, int, int, int,
-                 int, int, int, int, int, int, int64_t, int64_t, int, float, int);
+                 int, int, int, int, int, int, int64_t, int64_t, int, float, int, float);
     if (halves == 2)
         kern = kcb == 64 ? cv_grad_input_chan_kernel<64, 2> : kcb == 32 ? cv_grad_input_chan_kernel<32, 2>
                                                                          : cv_grad_input_chan_kernel<16, 2>;
@@ -525,7 +542,7 @@ int launch_cv_grad_input_chan(const float* xpad, const float* wq, const float* u
         KernelTimerScope timer_("cv_grad_input", stream);
         hipLaunchKernelGGL(kern, grid, block, lds, stream, xpad, wq, upm, ym, dx, crop, (int)g.H, (int)g.W, (int)g.C,
                            (int)g.Kc, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.Nh, (int)g.Nw, tiles_w,
-                           c_blocks, n_items, lead_items, (int)lead_blocks, np.max_cmp, ksplit);
+                           c_blocks, n_items, lead_items, (int)lead_blocks, np.max_cmp, ksplit, dx_mask_scale(np.max_time));
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;
