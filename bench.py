@@ -466,6 +466,7 @@ def measure(torch, snn, _lib, dev, key, steps, warmup, use_graph=True, want_cpu=
     torch.cuda.synchronize()
     prof = _lib.profile_collect()
     _lib.profile_enable(False)
+    snn.check_scan_health(dev)          # raises if a classifier-head scan gave up its bounded wait (NaN outputs)
 
     acc = account(torch, snn, wl.layers(), wl.extras)
     kernels = {}

@@ -27,6 +27,7 @@ namespace {
 // MAX_SPIKE_TIME = 1e5): differences that small exist only between values below 2^-85.
 // ---------------------------------------------------------------------------------------------
 constexpr int DX_TILE = 8;
+constexpr int DX_WAVES3 = 4;           // wavefronts per SIMD the KW = 3 variant is compiled for
 
 // Eight masked MACs  acc += upm_k * (x <= ym_k ? w_k : 0)  without a compare or a select: with
 //   m = clamp01(x * BIG - ym_k * BIG)       (one fused multiply-add with the clamp output modifier)
@@ -68,8 +69,15 @@ __device__ __forceinline__ void dx_mac8(float& acc, float x, float big, const fl
 // same channels of two neighbouring 8-pixel tiles, so no lane idles.  Which patch lies under a tap
 // then differs between the halves; a half whose patch does not exist reads a spare slot that holds
 // (ym, upm) = (-inf, 0) and so adds nothing.
-template <int KCB, int HALVES>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KCB == 64 && HALVES == 2 ? 3 : 4)))
+//
+// KW = 3 (the layer's kernel is three columns wide; 0: any width): the sweep is turned inside out.  A slot's
+// operands are read once per DX_GK output channels and serve the up to three (pixel, tap) pairs that meet
+// that patch, with the weights of all three taps of those channels in registers.  That takes far fewer
+// registers than a whole weight row per tap, so more wavefronts share a SIMD and cover each other's waits.
+constexpr int DX_GK = 8;
+template <int KCB, int HALVES, int KW>
+__global__ void __launch_bounds__(256)
+    __attribute__((amdgpu_waves_per_eu(KW == 3 ? DX_WAVES3 : KCB == 64 && HALVES == 2 ? 3 : 4)))
 cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restrict__ wq,
                           const float* __restrict__ upm, const float* __restrict__ ym,
                           float* __restrict__ dx, CropGeom crop, int H, int W, int C, int Kc, int Kh, int Kw, int Sh,
@@ -131,6 +139,29 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
         const int ow = p0 + t - crop.left;
         if (__any(xv[t] <= max_cmp && ow >= 0 && ow < crop.w)) live |= 1u << t;
     }
+    // KW = 3: bit s of `exists` says that slot s of the wavefront holds a patch; slots that do not are
+    // filled once with (+inf, 0), a term that adds nothing, and skipped by everything that writes LDS
+    // afterwards, so a lane may read any slot.  Bit 3 * d + kw of `work` says that the d-th slot of a
+    // half and tap kw meet a pixel with work (for some lane).
+    unsigned exists = 0, work = 0;
+    float bigv = big;
+    if constexpr (KW == 3) {
+        for (int sl = 0; sl < n_slots; ++sl) {
+            const int ww = w0 - 2 + sl;
+            if (ww >= 0 && ww % Sw == 0 && ww / Sw < Nw) exists |= 1u << sl;
+            else if (lane < KCB) { ys[sl * KCB + lane] = INFINITY; us[sl * KCB + lane] = 0.0f; }
+        }
+#pragma unroll
+        for (int d = 0; d < DX_TILE + 2; ++d) {
+            const bool any_patch = (exists >> d & 1u) || (HALVES == 2 && (exists >> (d + DX_TILE) & 1u));
+#pragma unroll
+            for (int kw = 0; kw < 3; ++kw) {
+                const int t = d - 2 + kw;                                 // the pixel that meets it under tap kw
+                if (t >= 0 && t < DX_TILE && any_patch && (live >> t & 1u)) work |= 1u << (3 * d + kw);
+            }
+        }
+        asm volatile("v_mov_b32 %0, %1" : "=v"(bigv) : "s"(big));         // one register for all the blocks below
+    }
     if (live != 0) {
         for (int kh = 0; kh < Kh; ++kh) {
             const int hh = h - kh;
@@ -171,12 +202,73 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
                 // ym -> -ym * BIG, the operand of dx_mac8 (-inf, an output that takes no part, becomes +inf);
                 // slots that were not loaded hold anything and are never read
                 for (int i = lane; i < n_slots * (KCB / 4); i += kWave) {
+                    if (KW == 3 && !(exists >> (i / (KCB / 4)) & 1u)) continue;
                     float4 v4 = reinterpret_cast<float4*>(ys)[i];
                     v4.x *= -big; v4.y *= -big; v4.z *= -big; v4.w *= -big;
                     reinterpret_cast<float4*>(ys)[i] = v4;
                 }
                 __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
                 __builtin_amdgcn_wave_barrier();
+                if constexpr (KW == 3) {
+                    // wq[tap][kc / 4][c][kc % 4]: the 16-byte pieces the lanes fetch together are neighbours
+                    // in memory.  Two register sets: the weights of the next DX_GK output channels are
+                    // fetched while the current ones are in use.
+                    const float4* __restrict__ wbase =
+                        reinterpret_cast<const float4*>(wq) + ((size_t)(kh * 3) * (Kc / 4) + kc0 / 4) * C + cc;
+                    const size_t tap_stride = (size_t)(Kc / 4) * C;
+                    auto load_w = [&](float (&wr)[3][DX_GK], int g) {
+#pragma unroll
+                        for (int kw = 0; kw < 3; ++kw)
+#pragma unroll
+                            for (int q = 0; q < DX_GK; q += 4) {
+                                const float4 v4 = wbase[kw * tap_stride + (size_t)(g * (DX_GK / 4) + q / 4) * C];
+                                wr[kw][q] = v4.x; wr[kw][q + 1] = v4.y; wr[kw][q + 2] = v4.z; wr[kw][q + 3] = v4.w;
+                            }
+                    };
+                    const float* __restrict__ ybase = ys + half * DX_TILE * KCB;
+                    constexpr int US = (SPAN + 3) * KCB;                  // from a slot's ym row to its upm row
+                    auto read_slot = [&](const float* __restrict__ yg, int d, float (&yd)[DX_GK], float (&ud)[DX_GK]) {
+#pragma unroll
+                        for (int v = 0; v < DX_GK; v += 4) {
+                            const float4 y4 = *reinterpret_cast<const float4*>(yg + d * KCB + v);
+                            const float4 u4 = *reinterpret_cast<const float4*>(yg + US + d * KCB + v);
+                            yd[v] = y4.x; yd[v + 1] = y4.y; yd[v + 2] = y4.z; yd[v + 3] = y4.w;
+                            ud[v] = u4.x; ud[v + 1] = u4.y; ud[v + 2] = u4.z; ud[v + 3] = u4.w;
+                        }
+                    };
+                    // all slots of a half against the three taps of DX_GK output channels; the operands of the
+                    // next slot are read while the current one computes
+                    auto sweep = [&](const float (&wr)[3][DX_GK], const float* __restrict__ yg) {
+                        float yq[2][DX_GK], uq[2][DX_GK];
+                        // the bits are tested where they are used: as thirty loop-invariant conditions they would
+                        // take sixty scalar registers
+                        unsigned wk = work;
+                        asm volatile("" : "+s"(wk));
+                        read_slot(yg, 0, yq[0], uq[0]);
+#pragma unroll
+                        for (int d = 0; d < DX_TILE + 2; ++d) {
+                            if (d + 1 < DX_TILE + 2) read_slot(yg, d + 1, yq[(d + 1) & 1], uq[(d + 1) & 1]);
+                            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                            for (int kw = 0; kw < 3; ++kw) {
+                                const int t = d - 2 + kw;
+                                if (t < 0 || t >= DX_TILE) continue;
+                                if (wk >> (3 * d + kw) & 1u) dx_mac8(acc[t], xv[t], bigv, uq[d & 1], yq[d & 1], wr[kw]);
+                            }
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    };
+                    float wa[3][DX_GK], wb[3][DX_GK];
+                    load_w(wa, 0);
+#pragma unroll 1
+                    for (int g = 0; g < KCB / DX_GK; g += 2) {
+                        load_w(wb, g + 1);
+                        sweep(wa, ybase + g * DX_GK);
+                        if (g + 2 < KCB / DX_GK) load_w(wa, g + 2);
+                        sweep(wb, ybase + (g + 1) * DX_GK);
+                    }
+                    continue;
+                }
                 for (int kw = 0; kw < Kw; ++kw) {
                     // wq[tap][kc / 4][c][kc % 4]: the 16-byte pieces the lanes fetch together are
                     // neighbours in memory
@@ -532,12 +624,20 @@ int launch_cv_grad_input_chan(const float* xpad, const float* wq, const float* u
                        (ksplit > 1 ? (size_t)(ksplit - 1) * DX_TILE * kWave * sizeof(float) : 0);
     void (*kern)(const float*, const float*, const float*, const float*, float*, CropGeom, int, int, int, int, int, int,
                  int, int, int, int, int, int, int64_t, int64_t, int, float, int, float);
-    if (halves == 2)
-        kern = kcb == 64 ? cv_grad_input_chan_kernel<64, 2> : kcb == 32 ? cv_grad_input_chan_kernel<32, 2>
-                                                                         : cv_grad_input_chan_kernel<16, 2>;
-    else
-        kern = kcb == 64 ? cv_grad_input_chan_kernel<64, 1> : kcb == 32 ? cv_grad_input_chan_kernel<32, 1>
-                                                                         : cv_grad_input_chan_kernel<16, 1>;
+    if (g.Kw == 3) {
+        if (halves == 2)
+            kern = kcb == 64 ? cv_grad_input_chan_kernel<64, 2, 3> : kcb == 32 ? cv_grad_input_chan_kernel<32, 2, 3>
+                                                                                : cv_grad_input_chan_kernel<16, 2, 3>;
+        else
+            kern = kcb == 64 ? cv_grad_input_chan_kernel<64, 1, 3> : kcb == 32 ? cv_grad_input_chan_kernel<32, 1, 3>
+                                                                                : cv_grad_input_chan_kernel<16, 1, 3>;
+    } else if (halves == 2) {
+        kern = kcb == 64 ? cv_grad_input_chan_kernel<64, 2, 0> : kcb == 32 ? cv_grad_input_chan_kernel<32, 2, 0>
+                                                                            : cv_grad_input_chan_kernel<16, 2, 0>;
+    } else {
+        kern = kcb == 64 ? cv_grad_input_chan_kernel<64, 1, 0> : kcb == 32 ? cv_grad_input_chan_kernel<32, 1, 0>
+                                                                            : cv_grad_input_chan_kernel<16, 1, 0>;
+    }
     {
         KernelTimerScope timer_("cv_grad_input", stream);
         hipLaunchKernelGGL(kern, grid, block, lds, stream, xpad, wq, upm, ym, dx, crop, (int)g.H, (int)g.W, (int)g.C,
