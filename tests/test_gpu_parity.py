@@ -631,6 +631,41 @@ def test_conv_weight_gradient_over_the_whole_range_of_time_differences(max_time,
     assert np.isfinite(dw.cpu().numpy()).all()
 
 
+@pytest.mark.parametrize("C,Kc,K", [(32, 64, 3), (64, 32, 3), (32, 16, 5)])
+def test_conv_input_gradient_mask_at_its_edges(C, Kc, K):
+    """The channel dX kernels evaluate the mask x <= y arithmetically, as clamp01((x - y) * 2^109) (for
+    MAX_SPIKE_TIME = 1e5).  Pixel and spike times from a handful of values, so that most pairs are exact ties
+    (mask true), neighbouring floats (1 and the float above it), zeros on both sides, and values a few powers of two above
+    the smallest difference the scale resolves: one wrong decision moves dX by a whole term, far outside the
+    band.  K = 3 takes the slot-major sweep, K = 5 the tap-major one."""
+    import snntc_amd as snn
+    max_time = 1e5
+    rng = np.random.default_rng(C + Kc + K)
+    one_up = np.nextafter(np.float32(1), np.float32(2))
+    values = np.array([0.0, 2.0 ** -100, 2.0 ** -60, 1.0, one_up, 1.5, 7.0, 99999.0], np.float32)
+    B, H, W = 2, 9, 12
+    pad = K // 2
+    xpad = values[rng.integers(0, len(values), (B, H + 2 * pad, W + 2 * pad, C))]
+    xpad[rng.random(xpad.shape) < 0.05] = np.float32(max_time)
+    P = K * K * C
+    w = rng.standard_normal((P + 1, Kc)).astype(np.float32)
+    p = capi.cv_params(K, K, 1, 1, same=True, biasvolt=1.0, max_time=max_time)
+    Nh, Nw, _ = capi.cv_dims(xpad.shape, p)
+    out = np.zeros((2 * B, Nh, Nw, Kc), np.float32)
+    out[:B] = values[rng.integers(0, len(values), (B, Nh, Nw, Kc))]
+    out[B:] = rng.standard_normal((B, Nh, Nw, Kc)).astype(np.float32)
+    dead = rng.random((B, Nh, Nw, Kc)) < 0.1
+    out[:B][dead] = np.float32(max_time); out[B:][dead] = 0.0
+    g = np.zeros((2 * B, Nh, Nw, Kc), np.float32); g[:B] = rng.standard_normal((B, Nh, Nw, Kc))
+    dx, dw, _ = snn.snncv_grad(t(g), t(xpad), t(w), p, t(out))
+    torch.cuda.synchronize()
+    rdx, rdw, _ = capi.cv_backward_dev(g, xpad, w, p, out, wide=True)
+    ao = out.copy(); ao[B:] = np.abs(ao[B:])
+    adx, adw, _ = capi.cv_backward_dev(np.abs(g), xpad, np.abs(w), p, ao, wide=True)
+    check_grad(dx.cpu().numpy(), rdx, adx, "dX")
+    check_grad(dw.cpu().numpy(), rdw, adw, "dW")
+
+
 @pytest.mark.parametrize("J", [9, 70])
 def test_dense_weight_gradient_at_the_edge_of_its_input_domain(J):
     """The dW kernels are exact for inputs down to -MAX_SPIKE_TIME (they scale y - x by the power of two
