@@ -65,26 +65,27 @@ __device__ __forceinline__ void dx_mac8(float& acc, float x, float big, const fl
           [w7] "v"(w[7]));
 }
 
-// HALVES = 2 is for layers with at most 32 input channels: the two halves of a wavefront take the
-// same channels of two neighbouring 8-pixel tiles, so no lane idles.  Which patch lies under a tap
-// then differs between the halves; a half whose patch does not exist reads a spare slot that holds
-// (ym, upm) = (-inf, 0) and so adds nothing.
+// MULTI is for layers with at most 32 input channels: the wavefront is cut into 2, 4, 8 or 16 parts
+// of 32, 16, 8 or 4 lanes (`1 << parts_shift` of them) that take the same channels of as many neighbouring
+// 8-pixel tiles, so few lanes idle.  Which patch lies under a tap then differs between the parts; a
+// part whose patch does not exist reads a slot that holds (ym, upm) = (-inf, 0) and so adds nothing.
 //
 // KW = 3 (the layer's kernel is three columns wide; 0: any width): the sweep is turned inside out.  A slot's
 // operands are read once per DX_GK output channels and serve the up to three (pixel, tap) pairs that meet
 // that patch, with the weights of all three taps of those channels in registers.  That takes far fewer
 // registers than a whole weight row per tap, so more wavefronts share a SIMD and cover each other's waits.
 constexpr int DX_GK = 8;
-template <int KCB, int HALVES, int KW>
+template <int KCB, bool MULTI, int KW>
 __global__ void __launch_bounds__(256)
-    __attribute__((amdgpu_waves_per_eu(KW == 3 ? DX_WAVES3 : KCB == 64 && HALVES == 2 ? 3 : 4)))
+    __attribute__((amdgpu_waves_per_eu(KW == 3 ? DX_WAVES3 : KCB == 64 && MULTI ? 3 : 4)))
 cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restrict__ wq,
                           const float* __restrict__ upm, const float* __restrict__ ym,
                           float* __restrict__ dx, CropGeom crop, int H, int W, int C, int Kc, int Kh, int Kw, int Sh,
                           int Sw, int Nh, int Nw, int tiles_w, int c_blocks, int64_t n_items, int64_t lead_items,
-                          int lead_blocks, float max_cmp, int ksplit, float big) {
-    extern __shared__ __align__(16) float staged[];      // per wavefront: [2][n_slots + 1][KCB]; ksplit = 4: then `partial`
-    constexpr int SPAN = DX_TILE * HALVES;               // pixels of one wavefront
+                          int lead_blocks, float max_cmp, int ksplit, float big, int parts_shift) {
+    extern __shared__ __align__(16) float staged[];      // per wavefront: [2][n_slots + 1][KCB]; ksplit > 1: then `partial`
+    const int parts = MULTI ? 1 << parts_shift : 1;
+    const int span = DX_TILE * parts;                    // pixels of one wavefront
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     // ksplit = 1: a tile per single-wavefront workgroup.  ksplit = 2 or 4 (layers with few tiles and many
     // output channels): a tile per workgroup of that many wavefronts, each takes its share of the output
@@ -100,7 +101,7 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
     const int ks = wave;                                 // 0 without the split
     if (item >= (lead ? lead_items : n_items - lead_items)) return;
     const int lane = threadIdx.x % kWave;
-    const int half = HALVES == 2 ? lane / 32 : 0;
+    const int part = MULTI ? lane >> (6 - parts_shift) : 0;
     const int tiles_lead = lead_items < n_items ? tiles_w - 1 : tiles_w;
     const int cb = (int)(item % c_blocks);
     int64_t rest = item / c_blocks;
@@ -108,12 +109,12 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
     if (lead) { tw = (int)(rest % tiles_lead); rest /= tiles_lead; }
     const int h = (int)(rest % H);
     const int a = (int)(rest / H);
-    const int w0 = tw * SPAN;                            // first pixel of the wavefront
-    const int p0 = w0 + half * DX_TILE;                  // first pixel of this lane
-    const int c = HALVES == 2 ? (lane & 31) : cb * kWave + lane;
+    const int w0 = tw * span;                            // first pixel of the wavefront
+    const int p0 = w0 + part * DX_TILE;                  // first pixel of this lane
+    const int c = MULTI ? (lane & ((kWave >> parts_shift) - 1)) : cb * kWave + lane;
     const bool lane_ok = c < C;
     const unsigned cc = (unsigned)(lane_ok ? c : C - 1);
-    const int n_slots = SPAN + Kw - 1;                   // slot d: the patch whose left column is w0-Kw+1+d
+    const int n_slots = span + Kw - 1;                   // slot d: the patch whose left column is w0-Kw+1+d
     float* __restrict__ ys = staged + (size_t)wave * 2 * (n_slots + 1) * KCB;
     float* __restrict__ us = ys + (n_slots + 1) * KCB;
     if (lane < KCB) {                                    // the spare slot
@@ -139,21 +140,27 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
         const int ow = p0 + t - crop.left;
         if (__any(xv[t] <= max_cmp && ow >= 0 && ow < crop.w)) live |= 1u << t;
     }
-    // KW = 3: bit s of `exists` says that slot s of the wavefront holds a patch; slots that do not are
-    // filled once with (+inf, 0), a term that adds nothing, and skipped by everything that writes LDS
-    // afterwards, so a lane may read any slot.  Bit 3 * d + kw of `work` says that the d-th slot of a
-    // half and tap kw meet a pixel with work (for some lane).
-    unsigned exists = 0, work = 0;
+    // KW = 3: slots that hold no patch are filled with (+inf, 0), a term that adds nothing, so a lane may read
+    // any slot.  With a column stride of 1 those are the slots outside [slot_lo, slot_hi): they are filled once and
+    // left alone by the rescaling pass of every staging round; otherwise they are filled again after every round.
+    // Bit 3 * d + kw of `work` says that the d-th slot of a part and tap kw meet a pixel with work (for some lane).
+    auto slot_exists = [&](int sl) {
+        const int ww = w0 - Kw + 1 + sl;
+        if (ww < 0) return false;
+        return Sw == 1 ? ww < Nw : (ww % Sw == 0 && ww / Sw < Nw);
+    };
+    auto fill_empty_slots = [&]() {
+        for (int sl = 0; sl < n_slots; ++sl)
+            if (!slot_exists(sl) && lane < KCB) { ys[sl * KCB + lane] = INFINITY; us[sl * KCB + lane] = 0.0f; }
+    };
+    const int slot_lo = max(0, Kw - 1 - w0), slot_hi = min(n_slots, Nw + Kw - 1 - w0);
+    unsigned work = 0;
     float bigv = big;
     if constexpr (KW == 3) {
-        for (int sl = 0; sl < n_slots; ++sl) {
-            const int ww = w0 - 2 + sl;
-            if (ww >= 0 && ww % Sw == 0 && ww / Sw < Nw) exists |= 1u << sl;
-            else if (lane < KCB) { ys[sl * KCB + lane] = INFINITY; us[sl * KCB + lane] = 0.0f; }
-        }
 #pragma unroll
         for (int d = 0; d < DX_TILE + 2; ++d) {
-            const bool any_patch = (exists >> d & 1u) || (HALVES == 2 && (exists >> (d + DX_TILE) & 1u));
+            bool any_patch = false;
+            for (int pt = 0; pt < parts; ++pt) any_patch = any_patch || slot_exists(d + pt * DX_TILE);
 #pragma unroll
             for (int kw = 0; kw < 3; ++kw) {
                 const int t = d - 2 + kw;                                 // the pixel that meets it under tap kw
@@ -161,6 +168,7 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
             }
         }
         asm volatile("v_mov_b32 %0, %1" : "=v"(bigv) : "s"(big));         // one register for all the blocks below
+        if (Sw == 1) fill_empty_slots();
     }
     if (live != 0) {
         for (int kh = 0; kh < Kh; ++kh) {
@@ -202,11 +210,12 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
                 // ym -> -ym * BIG, the operand of dx_mac8 (-inf, an output that takes no part, becomes +inf);
                 // slots that were not loaded hold anything and are never read
                 for (int i = lane; i < n_slots * (KCB / 4); i += kWave) {
-                    if (KW == 3 && !(exists >> (i / (KCB / 4)) & 1u)) continue;
+                    if (KW == 3 && Sw == 1 && (i / (KCB / 4) < slot_lo || i / (KCB / 4) >= slot_hi)) continue;
                     float4 v4 = reinterpret_cast<float4*>(ys)[i];
                     v4.x *= -big; v4.y *= -big; v4.z *= -big; v4.w *= -big;
                     reinterpret_cast<float4*>(ys)[i] = v4;
                 }
+                if (KW == 3 && Sw != 1) fill_empty_slots();
                 __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
                 __builtin_amdgcn_wave_barrier();
                 if constexpr (KW == 3) {
@@ -225,8 +234,8 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
                                 wr[kw][q] = v4.x; wr[kw][q + 1] = v4.y; wr[kw][q + 2] = v4.z; wr[kw][q + 3] = v4.w;
                             }
                     };
-                    const float* __restrict__ ybase = ys + half * DX_TILE * KCB;
-                    constexpr int US = (SPAN + 3) * KCB;                  // from a slot's ym row to its upm row
+                    const float* __restrict__ ybase = ys + part * DX_TILE * KCB;
+                    const int US = (span + 3) * KCB;                      // from a slot's ym row to its upm row
                     auto read_slot = [&](const float* __restrict__ yg, int d, float (&yd)[DX_GK], float (&ud)[DX_GK]) {
 #pragma unroll
                         for (int v = 0; v < DX_GK; v += 4) {
@@ -286,7 +295,7 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
                         const bool has_patch = p0 + t < W && ww >= 0 && ww % Sw == 0 && ww / Sw < Nw;
                         if (!(live >> t & 1) || !__any(has_patch)) continue;
                         int slot = has_patch ? p0 + t - w0 - kw + Kw - 1 : n_slots;
-                        if (HALVES == 1) slot = __builtin_amdgcn_readfirstlane(slot);   // same for every lane
+                        if (!MULTI) slot = __builtin_amdgcn_readfirstlane(slot);   // same for every lane
                         const float* __restrict__ yrow = ys + slot * KCB;
                         const float* __restrict__ urow = us + slot * KCB;
                         // groups of 16 output channels: eight broadcast reads, then 48 multiply-adds
@@ -568,12 +577,53 @@ cv_grad_weight_narrow_kernel(const float* __restrict__ xpad, const float* __rest
 
 }  // namespace
 
-bool cv_grad_input_chan_supported(const ConvGeom& g) {
-    // the staging buffer (four wavefronts, up to 2 * TILE + Kw patches) has to fit the default 64 KB of LDS
-    // (plus the 6 KB the output-channel split keeps for its partial sums)
-    return g.C >= 32 && g.Kc % 16 == 0 && (2 * DX_TILE + g.Kw) * 64 * 8 * 4 + 3 * DX_TILE * kWave * 4 <= 64 * 1024 &&
-           g.Nw * g.Kc * 4 < 0x7fffffffLL;               // an output row of ym / upm behind one buffer descriptor
+// Launch shape of the channel-lane dX kernel for a layer (decided by its geometry alone, never by the batch: the
+// order of the additions, and with it the last bits of dX, must not depend on the batch size).
+struct DxPlan {
+    bool ok;
+    int parts_shift, span, tiles_w, c_blocks, kcb, ksplit;
+    size_t lds;
+};
+static DxPlan dx_plan(const ConvGeom& g) {
+    DxPlan p{};
+    if (g.C < 1 || g.Kc % 16 != 0 || g.Nw * g.Kc * 4 >= 0x7fffffffLL) return p;   // (an output row of ym / upm behind one buffer descriptor)
+    // Fewer than 32 channels: only with the slot-major sweep of three-column kernels.  The tap-major one pays
+    // a few dozen scalar instructions per (pixel, tap) to find the patch, which 16 output channels of 3 or 4
+    // input channels do not cover (7x7/2 on 3 channels at 224 x 224, B = 32: 2.8 ms against 2.2 ms through
+    // patch space).
+    if (g.C < 32 && g.Kw != 3) return p;
+    // parts of a wavefront: as many as the channels leave room for, but no wider a tile than the row needs
+    int parts = g.C > 32 ? 1 : g.C > 16 ? 2 : g.C > 8 ? 4 : g.C > 4 ? 8 : 16;
+    while (parts > 2 && DX_TILE * (parts / 2) >= g.W) parts /= 2;
+    p.parts_shift = parts == 1 ? 0 : parts == 2 ? 1 : parts == 4 ? 2 : parts == 8 ? 3 : 4;
+    p.span = DX_TILE * parts;
+    p.tiles_w = (int)((g.W + p.span - 1) / p.span);
+    p.c_blocks = parts > 1 ? 1 : (int)((g.C + kWave - 1) / kWave);
+    p.kcb = g.Kc % 64 == 0 ? 64 : (g.Kc % 32 == 0 ? 32 : 16);
+    // small images with at least four chunks of output channels: split the channels over the
+    // wavefronts of a workgroup.
+    // (Up to 1024 tiles per image: with 256 output channels a tile's wavefront walks 36 taps, and at small
+    // batches too few tiles exist to hide that -- 256 -> 256 at 16 x 16, one image: 55 against 174 us;
+    // at 32 images the split still is a little ahead, 437 against 491 us.)
+    // With 128 output channels (two chunks) the split is in two: 64 -> 128 at 28 x 28 is 3840 tiles for 32 images,
+    // not quite four per SIMD, and the launch ends on the SIMDs that hold four.
+    // Layers with at most 32 input channels and 64 output channels on small images: two chunks of 32.
+    const bool few_tiles = g.H * p.tiles_w * p.c_blocks <= 1024;
+    if (parts > 1 && few_tiles && g.Kc == 64) p.kcb = 32;
+    // the staged rows of a wavefront stay near 12 KB, so that LDS holds them for sixteen wavefronts of a CU
+    auto wave_lds = [&](int kcb) { return (size_t)2 * (p.span + g.Kw) * kcb * sizeof(float); };
+    while (p.kcb > 16 && wave_lds(p.kcb) > 12 * 1024) p.kcb /= 2;
+    p.ksplit = !few_tiles ? 1 : (parts == 1 && g.Kc % (4 * p.kcb) == 0) ? 4 : g.Kc % (2 * p.kcb) == 0 ? 2 : 1;
+    auto total_lds = [&]() {
+        return p.ksplit * wave_lds(p.kcb) + (p.ksplit > 1 ? (size_t)(p.ksplit - 1) * DX_TILE * kWave * sizeof(float) : 0);
+    };
+    while (p.ksplit > 1 && total_lds() > 64 * 1024) p.ksplit /= 2;
+    p.lds = total_lds();
+    p.ok = p.lds <= 64 * 1024;                            // the default limit of a workgroup
+    return p;
 }
+
+bool cv_grad_input_chan_supported(const ConvGeom& g) { return dx_plan(g).ok; }
 
 // The factor BIG of dx_mac8: the largest power of two with MAX_SPIKE_TIME * BIG <= 2^126.
 static float dx_mask_scale(float max_time) {
@@ -589,24 +639,11 @@ static float dx_mask_scale(float max_time) {
 int launch_cv_grad_input_chan(const float* xpad, const float* wq, const float* upm, const float* ym,
                               float* dx, const CropGeom& crop, const ConvGeom& g, const NeuronParams& np,
                               hipStream_t stream) {
-    const int halves = g.C <= 32 ? 2 : 1;
-    const int span = DX_TILE * halves;
-    const int tiles_w = (int)((g.W + span - 1) / span);
-    const int c_blocks = halves == 2 ? 1 : (int)((g.C + kWave - 1) / kWave);
+    const DxPlan pl = dx_plan(g);
+    if (!pl.ok) return fail(SNNTC_ERR_UNSUPPORTED, "conv backward: no channel-lane launch shape for this layer");
+    const int span = pl.span, tiles_w = pl.tiles_w, c_blocks = pl.c_blocks, kcb = pl.kcb, ksplit = pl.ksplit;
+    const bool multi = pl.parts_shift > 0;
     const int64_t n_items = g.B * g.H * tiles_w * c_blocks;
-    int kcb = g.Kc % 64 == 0 ? 64 : (g.Kc % 32 == 0 ? 32 : 16);
-    // small images with at least four chunks of output channels: split the channels over the
-    // wavefronts of a workgroup.  Decided by the layer's geometry alone, never by the batch: the
-    // order of the additions, and with it the last bits of dX, must not depend on the batch size.
-    // (Up to 1024 tiles per image: with 256 output channels a tile's wavefront walks 36 taps, and at small
-    // batches too few tiles exist to hide that -- 256 -> 256 at 16 x 16, one image: 55 against 174 us;
-    // at 32 images the split still is a little ahead, 437 against 491 us.)
-    // With 128 output channels (two chunks) the split is in two: 64 -> 128 at 28 x 28 is 3840 tiles for 32 images,
-    // not quite four per SIMD, and the launch ends on the SIMDs that hold four.
-    // Layers with at most 32 input channels and 64 output channels on small images: two chunks of 32.
-    const bool few_tiles = g.H * tiles_w * c_blocks <= 1024;
-    if (halves == 2 && few_tiles && g.Kc == 64) kcb = 32;
-    const int ksplit = !few_tiles ? 1 : (halves == 1 && g.Kc % (4 * kcb) == 0) ? 4 : g.Kc % (2 * kcb) == 0 ? 2 : 1;
     // One item per workgroup.  Without the split a workgroup is a single wavefront: the
     // wavefronts do not cooperate, their running times differ (border tiles, rows outside the window),
     // and a CU takes a new workgroup only when a whole one has left, so in larger workgroups the slots
@@ -620,29 +657,29 @@ int launch_cv_grad_input_chan(const float* xpad, const float* wq, const float* u
     const int64_t blocks = lead_blocks + (n_items - lead_items);
     if (blocks > 0x7fffffffLL) return fail(SNNTC_ERR_TOO_LARGE, "conv backward: grid too large");
     dim3 grid((unsigned)blocks), block(wg_waves * kWave);
-    const size_t lds = (size_t)wg_waves * 2 * (span + g.Kw) * kcb * sizeof(float) +
-                       (ksplit > 1 ? (size_t)(ksplit - 1) * DX_TILE * kWave * sizeof(float) : 0);
+    const size_t lds = pl.lds;
     void (*kern)(const float*, const float*, const float*, const float*, float*, CropGeom, int, int, int, int, int, int,
-                 int, int, int, int, int, int, int64_t, int64_t, int, float, int, float);
+                 int, int, int, int, int, int, int64_t, int64_t, int, float, int, float, int);
     if (g.Kw == 3) {
-        if (halves == 2)
-            kern = kcb == 64 ? cv_grad_input_chan_kernel<64, 2, 3> : kcb == 32 ? cv_grad_input_chan_kernel<32, 2, 3>
-                                                                                : cv_grad_input_chan_kernel<16, 2, 3>;
+        if (multi)
+            kern = kcb == 64 ? cv_grad_input_chan_kernel<64, true, 3> : kcb == 32 ? cv_grad_input_chan_kernel<32, true, 3>
+                                                                                   : cv_grad_input_chan_kernel<16, true, 3>;
         else
-            kern = kcb == 64 ? cv_grad_input_chan_kernel<64, 1, 3> : kcb == 32 ? cv_grad_input_chan_kernel<32, 1, 3>
-                                                                                : cv_grad_input_chan_kernel<16, 1, 3>;
-    } else if (halves == 2) {
-        kern = kcb == 64 ? cv_grad_input_chan_kernel<64, 2, 0> : kcb == 32 ? cv_grad_input_chan_kernel<32, 2, 0>
-                                                                            : cv_grad_input_chan_kernel<16, 2, 0>;
+            kern = kcb == 64 ? cv_grad_input_chan_kernel<64, false, 3> : kcb == 32 ? cv_grad_input_chan_kernel<32, false, 3>
+                                                                                    : cv_grad_input_chan_kernel<16, false, 3>;
+    } else if (multi) {
+        kern = kcb == 64 ? cv_grad_input_chan_kernel<64, true, 0> : kcb == 32 ? cv_grad_input_chan_kernel<32, true, 0>
+                                                                               : cv_grad_input_chan_kernel<16, true, 0>;
     } else {
-        kern = kcb == 64 ? cv_grad_input_chan_kernel<64, 1, 0> : kcb == 32 ? cv_grad_input_chan_kernel<32, 1, 0>
-                                                                            : cv_grad_input_chan_kernel<16, 1, 0>;
+        kern = kcb == 64 ? cv_grad_input_chan_kernel<64, false, 0> : kcb == 32 ? cv_grad_input_chan_kernel<32, false, 0>
+                                                                                : cv_grad_input_chan_kernel<16, false, 0>;
     }
     {
         KernelTimerScope timer_("cv_grad_input", stream);
         hipLaunchKernelGGL(kern, grid, block, lds, stream, xpad, wq, upm, ym, dx, crop, (int)g.H, (int)g.W, (int)g.C,
                            (int)g.Kc, (int)g.Kh, (int)g.Kw, (int)g.Sh, (int)g.Sw, (int)g.Nh, (int)g.Nw, tiles_w,
-                           c_blocks, n_items, lead_items, (int)lead_blocks, np.max_cmp, ksplit, dx_mask_scale(np.max_time));
+                           c_blocks, n_items, lead_items, (int)lead_blocks, np.max_cmp, ksplit, dx_mask_scale(np.max_time),
+                           pl.parts_shift);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
     return SNNTC_OK;

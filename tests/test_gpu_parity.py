@@ -205,6 +205,14 @@ CONV_CASES = [
     (18, 1, 10, 9, 31, 8, 8, 2, 1, 1, True, False, "reftest"),      # columns of 248 entries
     (19, 2, 9, 30, 8, 8, 3, 3, 2, 5, False, True, "reftest"),       # stride wider than the kernel: no shared columns
     (20, 2, 13, 7, 96, 4, 3, 6, 3, 2, False, True, "reftest"),      # many channels, a single patch per output row
+    # fewer than 32 input channels with a multiple of 16 output channels: dX by channel lanes with the wavefront cut
+    # into 4, 8 or 16 parts that take neighbouring tiles
+    (21, 2, 14, 30, 16, 32, 3, 3, 1, 1, True, True, "baseline"),    # 16 channels: four parts
+    (22, 2, 10, 70, 8, 16, 3, 3, 1, 1, True, False, "baseline"),    # 8 channels: eight parts, two tiles per row
+    (23, 1, 9, 150, 4, 16, 3, 3, 1, 1, True, True, "baseline"),     # 4 channels: sixteen parts, tiles of 128 pixels
+    (24, 2, 11, 40, 24, 48, 5, 5, 1, 1, True, True, "baseline"),    # 24 of 32 lanes per part, five-column kernel
+    (25, 2, 12, 33, 12, 64, 3, 3, 2, 2, True, False, "baseline"),   # 12 of 16 lanes, stride 2: every second slot empty
+    (26, 1, 8, 20, 2, 16, 3, 3, 1, 2, False, True, "reftest"),      # two channels, VALID, column stride 2
 ]
 
 
