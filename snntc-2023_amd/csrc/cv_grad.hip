@@ -167,9 +167,9 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
                 if (t >= 0 && t < DX_TILE && any_patch && (live >> t & 1u)) work |= 1u << (3 * d + kw);
             }
         }
-        asm volatile("v_mov_b32 %0, %1" : "=v"(bigv) : "s"(big));         // one register for all the blocks below
         if (Sw == 1) fill_empty_slots();
     }
+    asm volatile("v_mov_b32 %0, %1" : "=v"(bigv) : "s"(big));             // one register for all the blocks below
     if (live != 0) {
         for (int kh = 0; kh < Kh; ++kh) {
             const int hh = h - kh;
@@ -292,7 +292,8 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
 #pragma unroll
                     for (int t = 0; t < DX_TILE; ++t) {
                         const int ww = p0 + t - kw;
-                        const bool has_patch = p0 + t < W && ww >= 0 && ww % Sw == 0 && ww / Sw < Nw;
+                        // (no division for the usual column stride of 1)
+                        const bool has_patch = p0 + t < W && ww >= 0 && (Sw == 1 ? ww < Nw : (ww % Sw == 0 && ww / Sw < Nw));
                         if (!(live >> t & 1) || !__any(has_patch)) continue;
                         int slot = has_patch ? p0 + t - w0 - kw + Kw - 1 : n_slots;
                         if (!MULTI) slot = __builtin_amdgcn_readfirstlane(slot);   // same for every lane
@@ -310,8 +311,8 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
                                 uq[v] = u4.x; uq[v + 1] = u4.y; uq[v + 2] = u4.z; uq[v + 3] = u4.w;
                             }
                             __builtin_amdgcn_sched_barrier(0);
-                            dx_mac8(acc[t], xv[t], big, &uq[0], &yq[0], &wreg[g * 16]);
-                            dx_mac8(acc[t], xv[t], big, &uq[8], &yq[8], &wreg[g * 16 + 8]);
+                            dx_mac8(acc[t], xv[t], bigv, &uq[0], &yq[0], &wreg[g * 16]);
+                            dx_mac8(acc[t], xv[t], bigv, &uq[8], &yq[8], &wreg[g * 16 + 8]);
                         }
                     }
                 }
