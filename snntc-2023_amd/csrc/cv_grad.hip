@@ -179,7 +179,7 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
             const size_t row0 = (size_t)(a * Nh + nh) * Nw;
             const int kc_share = Kc / ksplit;
             for (int kc0 = ks * kc_share; kc0 < (ks + 1) * kc_share; kc0 += KCB) {
-                // stage the patch row: slots whose patch does not exist are never read
+                // stage the patch row (only slots whose patch exists are loaded)
                 __builtin_amdgcn_wave_barrier();
                 // The rows go from memory straight into LDS (buffer loads with the LDS bit: lane l of a load
                 // writes dword l behind the load's LDS base).  A load covers 64 / KCB neighbouring slots --
@@ -207,8 +207,9 @@ cv_grad_input_chan_kernel(const float* __restrict__ xpad, const float* __restric
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
                 __builtin_amdgcn_wave_barrier();
-                // ym -> -ym * BIG, the operand of dx_mac8 (-inf, an output that takes no part, becomes +inf);
-                // slots that were not loaded hold anything and are never read
+                // ym -> -ym * BIG, the operand of dx_mac8 (-inf, an output that takes no part, becomes +inf).
+                // Slots that were not loaded: the tap-major sweep never reads them (it reads the spare slot
+                // instead), the slot-major one reads them as (+inf, 0), see fill_empty_slots
                 for (int i = lane; i < n_slots * (KCB / 4); i += kWave) {
                     if (KW == 3 && Sw == 1 && (i / (KCB / 4) < slot_lo || i / (KCB / 4) >= slot_hi)) continue;
                     float4 v4 = reinterpret_cast<float4*>(ys)[i];
