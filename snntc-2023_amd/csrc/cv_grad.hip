@@ -1,4 +1,4 @@
-// Backward kernels specialised for conv layers whose channel count is a multiple of 32.
+// Backward kernels specialised for conv layers: lanes are input channels (dX) or output channels (dW).
 //
 // Same contract as grad.hip (snntc/snncvgrad_kernels.cu.cc:15-161): with up = grad*1/S masked by
 // y <= MAX-0.1 (arrays upm / ym), patch s = (a, nh, nw), element i = (kh*Kw + kw)*C + c,

@@ -596,7 +596,8 @@ reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ ou
 }
 
 // ---------------------------------------------------------------------------------------------
-// Conv dX for layers the channel-lane kernel does not take (fewer than 32 input channels): the
+// Conv dX for layers the channel-lane kernel does not take (output channels not a multiple of 16, or fewer
+// than 32 input channels under a kernel that is not three columns wide): the
 // gradient per patch element, dxp[S, P], comes from the dense kernel above run over the implicit
 // patches; here every element of the padded image adds up the patch elements that alias it, in
 // (kh, kw) order.  Gather form: no atomics, fixed summation order.
