@@ -256,7 +256,7 @@ def account(torch, snn, layers, extras=None):
       scan          : bytes 4*(2*S*I + (I+b)*J + 2*S*J)            flops 4*steps
       dX kernels    : bytes 4*(2*S*J + in + I*J + in)              flops 2*pairs
       grad_weight   : bytes 4*(2*S*J + in + (I+b)*J)               flops 3*pairs
-      prep_upstream : bytes 4*(3*S*J + 2*S*J + 2*I*J)              flops S*J   (carries the weight copy dX reads)
+      prep_upstream : bytes 4*(3*S*J + S*J + 2*I*J)                flops S*J   (carries the weight copy dX reads)
       fc_backward_narrow (J <= 16, the three above in one launch): bytes 4*(3*S*J + 2*in + 2*(I+b)*J), flops 5*pairs + S*J
       pad_time : bytes 4*(in + out) ;  min_pool / min_pool_grad : bytes 4*(in + 2*out)
     `in` is the op's input tensor (B*I dense, B*H*W*C padded image for conv)."""
@@ -312,7 +312,7 @@ def account(torch, snn, layers, extras=None):
         if want_dx:
             add("fc_grad_input" if dense else "cv_grad_input", 2.0 * pairs, 4.0 * (2.0 * S * J + 2.0 * n_in + I * J))
         add("grad_weight", 3.0 * pairs, 4.0 * (2.0 * S * J + n_in + (I + bias) * J))
-        add("prep_upstream", float(S * J), 4.0 * (5.0 * S * J + (2.0 * I * J if want_dx else 0.0)))
+        add("prep_upstream", float(S * J), 4.0 * (4.0 * S * J + (2.0 * I * J if want_dx else 0.0)))
     for name, nbytes in (extras or {}).items():
         add(name, 0.0, nbytes)
     return acc

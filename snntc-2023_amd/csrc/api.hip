@@ -166,7 +166,7 @@ int forward_chain(const SegmentSource& src, const FcFwdWs& ws, const float* w, f
 
 // Backward scratch.  `rows` is the weight row count including a possible bias row; the partial-sum
 // area is sized for the worst case of 256 slices only when slicing can happen at all.
-struct BwdWs { float* upm; float* ym; float* wt; float* dxp; float* partial; int max_split; size_t bytes; };
+struct BwdWs { float* upm; float* wt; float* dxp; float* partial; int max_split; size_t bytes; };
 // patch_scratch: elements of the per-patch gradient of conv layers whose dX goes through patch space
 // narrow_split: slices the one-launch backward of a narrow dense layer needs (0: not that path)
 BwdWs bwd_ws(void* ws, int64_t S, int64_t rows, int64_t J, int64_t min_base_blocks, int64_t patch_scratch = 0,
@@ -174,7 +174,6 @@ BwdWs bwd_ws(void* ws, int64_t S, int64_t rows, int64_t J, int64_t min_base_bloc
     Carver c(ws);
     BwdWs r;
     r.upm = c.take<float>(S * J);
-    r.ym = c.take<float>(S * J);
     r.wt = c.take<float>(rows * J);
     r.dxp = c.take<float>(patch_scratch);
     r.max_split = weight_grad_splits(S, min_base_blocks);
@@ -597,11 +596,11 @@ int snntc_fc_backward(const float* grad, const float* x, const float* w, const f
         return launch_fc_backward_narrow(x, w, grad, oldout, oldout + B * J, dx, dw, ws.partial, dparams, 6, B, I, J,
                                          np, st);
     // wt[J, I] for dX (the bias row is not needed) is written by the same launch
-    rc = launch_backward_prologue(grad, oldout, oldout + B * J, ws.upm, ws.ym, B * J, np, dx ? 1 : 0, w, ws.wt, I, J,
+    rc = launch_backward_prologue(grad, oldout, oldout + B * J, ws.upm, B * J, np, dx ? 1 : 0, w, ws.wt, I, J,
                                   0, dparams, 6, st);
     if (rc) return rc;
     if (dx) {
-        rc = launch_fc_grad_input(x, ws.wt, ws.upm, ws.ym, dx, B, I, J, I, st);
+        rc = launch_fc_grad_input(x, ws.wt, ws.upm, oldout, dx, B, I, J, I, st);
         if (rc) return rc;
     }
     if (!dw) return SNNTC_OK;
@@ -609,7 +608,7 @@ int snntc_fc_backward(const float* grad, const float* x, const float* w, const f
     src.base = x; src.conv = 0; src.I = (int)I;
     int nsplit = weight_grad_splits(B, grad_weight_blocks(w_rows, J));
     if (nsplit > ws.max_split) nsplit = ws.max_split;
-    rc = launch_grad_weight_rows(src, ws.upm, ws.ym, nsplit > 1 ? ws.partial : dw, nsplit, B, J, 0, np, st);
+    rc = launch_grad_weight_rows(src, ws.upm, oldout, nsplit > 1 ? ws.partial : dw, nsplit, B, J, 0, np, st);
     if (rc) return rc;
     return launch_reduce_partials(ws.partial, dw, w_rows * J, nsplit, st);
 }
@@ -696,14 +695,14 @@ static int cv_backward_impl(const float* grad, const float* xpad, const float* w
     // the weight copy dX reads from is written by the same launch: regrouped for the channel kernel,
     // wt[Kc, P] for the generic one
     const bool chan_dx = cv_grad_input_chan_supported(g);
-    rc = launch_backward_prologue(grad, oldout, oldout + g.S * Kc, ws.upm, ws.ym, g.S * Kc, np,
+    rc = launch_backward_prologue(grad, oldout, oldout + g.S * Kc, ws.upm, g.S * Kc, np,
                                   !dxpad ? 0 : chan_dx ? 2 : 1, w, ws.wt, g.P, Kc, g.C, dparams, 12, st);
     if (rc) return rc;
     if (dxpad) {
         if (chan_dx) {
-            rc = launch_cv_grad_input_chan(xpad, ws.wt, ws.upm, ws.ym, dxpad, crop, g, np, st);
+            rc = launch_cv_grad_input_chan(xpad, ws.wt, ws.upm, oldout, dxpad, crop, g, np, st);
         } else {
-            rc = launch_cv_grad_input(conv_source(xpad, g), ws.wt, ws.upm, ws.ym, ws.dxp, dxpad, crop, g, g.P, st);
+            rc = launch_cv_grad_input(conv_source(xpad, g), ws.wt, ws.upm, oldout, ws.dxp, dxpad, crop, g, g.P, st);
         }
         if (rc) return rc;
     }
@@ -714,9 +713,9 @@ static int cv_backward_impl(const float* grad, const float* xpad, const float* w
     float* dst = nsplit > 1 ? ws.partial : dw;
     const SegmentSource src = conv_source(xpad, g);
     if (wide) {
-        rc = launch_cv_grad_weight_wide(xpad, ws.upm, ws.ym, dst, nsplit, g, w_rows, np, st);
+        rc = launch_cv_grad_weight_wide(xpad, ws.upm, oldout, dst, nsplit, g, w_rows, np, st);
     } else {
-        rc = launch_grad_weight_rows(src, ws.upm, ws.ym, dst, nsplit, g.S, Kc, 0, np, st);
+        rc = launch_grad_weight_rows(src, ws.upm, oldout, dst, nsplit, g.S, Kc, 0, np, st);
     }
     if (rc) return rc;
     return launch_reduce_partials(ws.partial, dw, w_rows * Kc, nsplit, st);

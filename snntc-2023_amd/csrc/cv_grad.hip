@@ -1,7 +1,7 @@
 // Backward kernels specialised for conv layers: lanes are input channels (dX) or output channels (dW).
 //
-// Same contract as grad.hip (snntc/snncvgrad_kernels.cu.cc:15-161): with up = grad*1/S masked by
-// y <= MAX-0.1 (arrays upm / ym), patch s = (a, nh, nw), element i = (kh*Kw + kw)*C + c,
+// Same contract as grad.hip (snntc/snncvgrad_kernels.cu.cc:15-161): with upm = grad*1/S, zero where
+// y > MAX-0.1, and ym the spike times y themselves, patch s = (a, nh, nw), element i = (kh*Kw + kw)*C + c,
 //   dXpad[a,h,w,c] = sum over patches covering (h,w) and over kc of [x <= ym[s,kc]] upm[s,kc] W[i,kc]
 //   dW[i,kc]       = sum over patches of min(x_si - ym[s,kc], 0) * upm[s,kc]
 // Both kernels put the channel (dX) or the output channel (dW) on the lanes, so everything that

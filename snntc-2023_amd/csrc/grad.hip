@@ -9,9 +9,10 @@
 // accumulated in gather form (every input pixel sums over the output pixels whose window covers
 // it), so no atomics are needed and the result does not depend on scheduling.
 //
-// The validity test on y is folded into two small arrays prepared once per call:
-//   upm = valid ? up : 0,   ym = valid ? y : -inf      (x <= -inf is false for every finite x)
-// and the weight-gradient mask is folded into arithmetic: for x <= y the term (x-y) is <= 0 and
+// The validity test on y is folded into one array prepared once per call,
+//   upm = valid ? up : 0,
+// so that a term of an output that takes no part vanishes whatever its mask says (the kernels read y
+// itself, under the parameter name ym); the weight-gradient mask is folded into arithmetic: for x <= y the term (x-y) is <= 0 and
 // for x > y it is > 0, hence [x <= y](x - y) == min(x - y, 0).
 #include "snntc_common.h"
 
@@ -19,7 +20,7 @@ namespace snntc {
 namespace {
 
 // First launch of a backward pass.  The elementwise pass over the layer's outputs,
-//   upm = valid ? grad * rcp : 0,  ym = valid ? y : -inf   (valid: y <= MAX - 0.1),
+//   upm = valid ? grad * rcp : 0   (valid: y <= MAX - 0.1),
 // and the weight copy dX reads from do not depend on each other: one launch does both, the first
 // prep_blocks workgroups the former, the rest the latter.
 //   mode 1: wt[cols, rows] = w[rows, cols]^T, a 32 x 32 tile per workgroup
@@ -27,8 +28,7 @@ namespace {
 //           multiple of 4; chan = C)
 __global__ void __launch_bounds__(256)
 backward_prologue_kernel(const float* __restrict__ grad, const float* __restrict__ y,
-                         const float* __restrict__ rcp, float* __restrict__ upm, float* __restrict__ ym,
-                         int64_t n, float max_cmp, int prep_blocks, int mode, const float* __restrict__ w,
+                         const float* __restrict__ rcp, float* __restrict__ upm, int64_t n, float max_cmp, int prep_blocks, int mode, const float* __restrict__ w,
                          float* __restrict__ wt, int rows, int cols, int chan, float* __restrict__ zeros,
                          int n_zeros) {
     __shared__ float tile[32][33];
@@ -39,7 +39,6 @@ backward_prologue_kernel(const float* __restrict__ grad, const float* __restrict
         const float yv = y[t];
         const bool valid = yv <= max_cmp;
         upm[t] = valid ? grad[t] * rcp[t] : 0.0f;
-        ym[t] = valid ? yv : -INFINITY;
         return;
     }
     const int blk = (int)blockIdx.x - prep_blocks;
@@ -634,8 +633,7 @@ int blocks_for(int64_t n, int block) { return (int)((n + block - 1) / block); }
 
 }  // namespace
 
-int launch_backward_prologue(const float* grad, const float* y, const float* rcp, float* upm, float* ym,
-                             int64_t n, const NeuronParams& np, int mode, const float* w, float* wt, int64_t rows,
+int launch_backward_prologue(const float* grad, const float* y, const float* rcp, float* upm, int64_t n, const NeuronParams& np, int mode, const float* w, float* wt, int64_t rows,
                              int64_t cols, int64_t chan, float* zeros, int n_zeros, hipStream_t stream) {
     if (!zeros) n_zeros = 0;
     const int64_t prep_blocks = (n + 255) / 256;
@@ -648,7 +646,7 @@ int launch_backward_prologue(const float* grad, const float* y, const float* rcp
     {
         KernelTimerScope timer_("prep_upstream", stream);
         hipLaunchKernelGGL(backward_prologue_kernel, dim3((unsigned)(prep_blocks + copy_blocks)), dim3(256), 0, stream,
-                           grad, y, rcp, upm, ym, n, np.max_cmp, (int)prep_blocks, mode, w, wt, (int)rows, (int)cols,
+                           grad, y, rcp, upm, n, np.max_cmp, (int)prep_blocks, mode, w, wt, (int)rows, (int)cols,
                            (int)chan, zeros, n_zeros);
     }
     SNNTC_HIP_CHECK(hipGetLastError());

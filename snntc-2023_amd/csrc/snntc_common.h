@@ -175,13 +175,11 @@ int read_scan_giveups(int64_t* count, hipStream_t stream);
 int scan_prepare_device(int dev, int* cu_count_out);
 int merge_prepare_device(int dev);
 
-// upm = valid ? grad*rcp : 0 ; ym = valid ? y : -inf   (valid: y <= MAX-0.1), n elements each, and,
-// in the same launch, the weight copy dX reads from: mode 0 none, mode 1
+// upm = valid ? grad*rcp : 0   (valid: y <= MAX-0.1; n elements), and, in the same launch, the weight copy dX reads from: mode 0 none, mode 1
 // wt[cols, rows] = w[rows, cols]^T, mode 2 the regrouped copy of a conv layer's weights
 // (wt[tap][cols / 4][chan][cols % 4] from w[(tap, chan), cols], rows = taps * chan).  `zeros`, if not
 // NULL, are n_zeros (<= 256) floats the launch clears: the op's all-zero dParams output.
-int launch_backward_prologue(const float* grad, const float* y, const float* rcp, float* upm, float* ym,
-                             int64_t n, const NeuronParams& np, int mode, const float* w, float* wt, int64_t rows,
+int launch_backward_prologue(const float* grad, const float* y, const float* rcp, float* upm, int64_t n, const NeuronParams& np, int mode, const float* w, float* wt, int64_t rows,
                              int64_t cols, int64_t chan, float* zeros, int n_zeros, hipStream_t stream);
 
 int launch_fc_grad_input(const float* x, const float* wt, const float* upm, const float* ym, float* dx,
