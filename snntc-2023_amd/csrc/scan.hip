@@ -1023,8 +1023,24 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
                                                        n_segs * stride * (int)sizeof(float));
         const int lane_bytes = ((seg - seg0) * stride + quad_lane) * (int)sizeof(float);
         const int n_seg = n_real[seg];
-        const int n_full = n_seg & ~(CHUNK - 1);
         const float first_x = xs[0];
+        // The ring of (x, row) entries the fast loop below consumes (see there).  Its first round is requested
+        // here, next to the two loads above and before anything waits for them: practically every item
+        // starts its first pass at input 0, and the round trips would otherwise follow one another.
+        constexpr int RING = 8;                             // chunks of entries held or on their way
+        float rxl[RING], rxh[RING];
+        int rpl[RING], rph[RING];
+        auto request = [&](int slot, int k) {
+            const int kb = (k <= last_chunk ? k : 0) * (int)sizeof(float);
+            rxl[slot] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rows_of_item.xs, lane_bytes, kb, 0));
+            rxh[slot] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rows_of_item.xs, lane_bytes + 16, kb, 0));
+            rpl[slot] = (int)__builtin_amdgcn_raw_buffer_load_b32(rows_of_item.pr, lane_bytes, kb, 0);
+            rph[slot] = (int)__builtin_amdgcn_raw_buffer_load_b32(rows_of_item.pr, lane_bytes + 16, kb, 0);
+        };
+#pragma unroll
+        for (int b = 0; b < RING - 1; ++b) request(b, b * CHUNK);
+        bool ring_at_zero = true;                           // the ring holds the entries from input 0 on
+        const int n_full = n_seg & ~(CHUNK - 1);
 
         // Per scan: the running sums, the number of inputs they hold (kcur), and where the scan stands:
         //   armed    waits to run the fast loop from kcur (no reference test can close before kcur)
@@ -1094,17 +1110,7 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
                 // move per input time (shared by the lane's CH scans).
                 // Per phase, with c the chunk being consumed: request the entries of chunk c+RING-1, read
                 // the weights of chunk c+1 from LDS, run chunk c.
-                constexpr int RING = 8;                     // chunks of entries held or on their way
-                float rxl[RING], rxh[RING];
-                int rpl[RING], rph[RING];
                 float wv[2][CH][CHUNK];                     // [buffer][scan][step]
-                auto request = [&](int slot, int k) {
-                    const int kb = (k <= last_chunk ? k : 0) * (int)sizeof(float);
-                    rxl[slot] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rows_of_item.xs, lane_bytes, kb, 0));
-                    rxh[slot] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rows_of_item.xs, lane_bytes + 16, kb, 0));
-                    rpl[slot] = (int)__builtin_amdgcn_raw_buffer_load_b32(rows_of_item.pr, lane_bytes, kb, 0);
-                    rph[slot] = (int)__builtin_amdgcn_raw_buffer_load_b32(rows_of_item.pr, lane_bytes + 16, kb, 0);
-                };
                 auto weights = [&](int slot, float (&wo)[CH][CHUNK]) {
                     unsigned al[4], ah[4];
                     quad_row_addresses<ROW_SHIFT>(rpl[slot], wbase, al);
@@ -1137,8 +1143,11 @@ scan_filter_kernel(const float* __restrict__ sorted, const int32_t* __restrict__
                         xq[buf][4] = hi.x; xq[buf][5] = hi.y; xq[buf][6] = hi.z; xq[buf][7] = hi.w;
                     }
                 };
+                if (!(ring_at_zero && kmin == 0)) {
 #pragma unroll
-                for (int b = 0; b < RING - 1; ++b) request(b, kmin + b * CHUNK);
+                    for (int b = 0; b < RING - 1; ++b) request(b, kmin + b * CHUNK);
+                }
+                ring_at_zero = false;
                 weights(0, wv[0]);
                 // (every lane "uses" the first chunk's times here: otherwise the compiler moves their loads
                 // under the writers' branch of stage_times and waits for all 28 requests there)
