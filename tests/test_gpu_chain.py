@@ -19,10 +19,11 @@ def t(a):
 @pytest.mark.parametrize("seed,B,H,W,C,Kc,K,S,dist", [
     (0, 3, 10, 10, 32, 32, 3, 1, "baseline"),      # channel-lane dX kernel, merged patch sort
     (1, 2, 9, 13, 64, 48, 3, 1, "reftest"),        # non-square image
-    (2, 4, 8, 8, 3, 16, 3, 1, "baseline"),         # few input channels: patch-space dX + col2im
+    (2, 4, 8, 8, 3, 16, 3, 1, "baseline"),         # few input channels: channel lanes, the wavefront in parts
     (3, 2, 11, 11, 40, 32, 3, 2, "baseline"),      # stride 2: uneven SAME padding
-    (4, 2, 12, 12, 16, 8, 5, 1, "reftest"),        # 5x5 kernel, two pixels of padding
+    (4, 2, 12, 12, 16, 8, 5, 1, "reftest"),        # 5x5 kernel, two pixels of padding: patch-space dX + col2im
     (5, 300, 8, 8, 32, 64, 3, 1, "baseline"),      # a launch large enough for the filtered scan
+    (6, 2, 9, 70, 8, 16, 3, 1, "baseline"),        # eight channels, rows of two 64-pixel tiles
 ])
 def test_conv_ops_with_a_second_destination_and_a_gradient_window(seed, B, H, W, C, Kc, K, S, dist):
     import snntc_amd as snn
