@@ -13,9 +13,10 @@ namespace snntc {
 namespace {
 
 // ---------------------------------------------------------------------------------------------
-// dX.  A wavefront owns TILE consecutive pixels of one image row and 64 (or 32) channels; lane =
-// channel.  For every kernel tap (kh, kw) the lane keeps its weight row W[(kh,kw,c), 0..KCB) in
-// registers and sweeps the tile: the patch under the tap is the same for all lanes.  The rows come
+// dX.  A wavefront owns TILE consecutive pixels of one image row and 64 channels (fewer channels: more
+// tiles, see MULTI); lane = channel.  Tap-major sweep (any kernel width): for every kernel tap (kh, kw) the
+// lane keeps its weight row W[(kh,kw,c), 0..KCB) in registers and sweeps the tile; the patch under the tap is
+// the same for all lanes.  Slot-major sweep (three-column kernels): see KW below.  The weights come
 // from a copy of W regrouped as [tap][kc / 4][c][kc % 4] (written by backward_prologue_kernel): read from W itself,
 // every 16-byte fetch of a wavefront touches 64 different cache lines instead of 8.  The ym / upm
 // rows of the TILE + Kw - 1 patches one kernel row can touch are staged in a wavefront-private
@@ -68,12 +69,15 @@ __device__ __forceinline__ void dx_mac8(float& acc, float x, float big, const fl
 // MULTI is for layers with at most 32 input channels: the wavefront is cut into 2, 4, 8 or 16 parts
 // of 32, 16, 8 or 4 lanes (`1 << parts_shift` of them) that take the same channels of as many neighbouring
 // 8-pixel tiles, so few lanes idle.  Which patch lies under a tap then differs between the parts; a
-// part whose patch does not exist reads a slot that holds (ym, upm) = (-inf, 0) and so adds nothing.
+// part whose patch does not exist reads a slot that holds (ym, upm) = (-inf, 0) -- +inf in the scaled form
+// of dx_mac8 -- and so adds nothing.
 //
 // KW = 3 (the layer's kernel is three columns wide; 0: any width): the sweep is turned inside out.  A slot's
 // operands are read once per DX_GK output channels and serve the up to three (pixel, tap) pairs that meet
 // that patch, with the weights of all three taps of those channels in registers.  That takes far fewer
-// registers than a whole weight row per tap, so more wavefronts share a SIMD and cover each other's waits.
+// registers than a whole weight row per tap; they go into a second set of weights and of slot operands,
+// fetched while the current ones are in use, and fewer LDS reads are needed (80 instead of 192 per tile and
+// 16 output channels).
 constexpr int DX_GK = 8;
 template <int KCB, bool MULTI, int KW>
 __global__ void __launch_bounds__(256)
