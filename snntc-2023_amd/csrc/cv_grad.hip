@@ -465,40 +465,21 @@ cv_grad_weight_wide_kernel(const float* __restrict__ xpad, const float* __restri
 
 // ---------------------------------------------------------------------------------------------
 // dW for layers with at most 32 output channels.  Lane = (half, kc): the two halves of a wavefront
-// take alternate patches, so no lane idles.  The 32 inputs of a patch that a block's rows need sit
-// in two registers (lane r of every row of 16 lanes holds inputs r and 16 + r of the half's own
-// patch) and reach the subtraction through its DPP row broadcast: still three instructions per
-// MAC, with a different patch in each half.  Partial sums of the halves and of the four
-// wavefronts are added in a fixed order through LDS.
+// take alternate patches, so no lane idles.  The 32 inputs of a patch that a block's rows need are
+// fetched two per lane (lane r of the first 16 lanes of a half fetches inputs r and 16 + r of the half's own
+// patch), left in a 256-byte buffer of the wavefront in LDS and read back by every lane of the half as
+// eight 16-byte broadcasts: with the inputs in vector registers a term is the two plain multiply-adds of
+// the wide kernel (scaled_lead), where a DPP operand, a minimum and a multiply-add used to cost twice
+// the issue time.  Partial sums of the halves and of the four wavefronts are added in a fixed order
+// through LDS.
 // ---------------------------------------------------------------------------------------------
-#define SNNTC_DW_ROW(R, A)                                                                       \
-    "v_sub_f32_dpp %[d], %[x], %[y] row_newbcast:" #R " row_mask:0xf bank_mask:0xf\n"             \
-    "v_min_f32_e32 %[d], 0, %[d]\n"                                                              \
-    "v_fmac_f32_e32 %[" #A "], %[d], %[u]\n"
-
-__device__ __forceinline__ void dw_rows16(float (&acc)[DWW_RI], int base, float x, float y, float u) {
-    float d;
-    float* a = acc + base;
-    // the leading s_nop covers the two wait states a DPP read needs after a vector write of the same
-    // register, should the compiler have placed a copy into x right before the block
-    asm volatile(
-        "s_nop 1\n"
-        SNNTC_DW_ROW(0, a0) SNNTC_DW_ROW(1, a1) SNNTC_DW_ROW(2, a2) SNNTC_DW_ROW(3, a3)
-        SNNTC_DW_ROW(4, a4) SNNTC_DW_ROW(5, a5) SNNTC_DW_ROW(6, a6) SNNTC_DW_ROW(7, a7)
-        SNNTC_DW_ROW(8, a8) SNNTC_DW_ROW(9, a9) SNNTC_DW_ROW(10, a10) SNNTC_DW_ROW(11, a11)
-        SNNTC_DW_ROW(12, a12) SNNTC_DW_ROW(13, a13) SNNTC_DW_ROW(14, a14) SNNTC_DW_ROW(15, a15)
-        : [d] "=&v"(d), [a0] "+v"(a[0]), [a1] "+v"(a[1]), [a2] "+v"(a[2]), [a3] "+v"(a[3]), [a4] "+v"(a[4]),
-          [a5] "+v"(a[5]), [a6] "+v"(a[6]), [a7] "+v"(a[7]), [a8] "+v"(a[8]), [a9] "+v"(a[9]), [a10] "+v"(a[10]),
-          [a11] "+v"(a[11]), [a12] "+v"(a[12]), [a13] "+v"(a[13]), [a14] "+v"(a[14]), [a15] "+v"(a[15])
-        : [x] "v"(x), [y] "v"(y), [u] "v"(u));
-}
-
 __global__ void __launch_bounds__(256)
 cv_grad_weight_narrow_kernel(const float* __restrict__ xpad, const float* __restrict__ upm,
                              const float* __restrict__ ym, float* __restrict__ dst, int S, int Kc, int rows,
                              int seg_per_slice, int H, int W, int C, int Kw, int Sh, int Sw, int Nh, int Nw,
-                             int bias_row, float biasvolt, int /*s_safe*/, float /*neg_s*/, float /*post*/) {
+                             int bias_row, float biasvolt, int /*s_safe*/, float neg_s, float post) {
     __shared__ float red[4][DWW_RI + 1][kWave];
+    __shared__ __align__(16) float xstage[4][2][DWW_RI];   // [wavefront][half][input]
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int half = lane >> 5, kc = lane & 31;
@@ -559,9 +540,29 @@ cv_grad_weight_narrow_kernel(const float* __restrict__ xpad, const float* __rest
                 x0n = px0[0]; x1n = px0[second]; yn = *py;
                 un = s < s_hi ? *pu : 0.0f;
             }
-            dw_rows16(acc, 0, x0, yv, uv);
-            if (n_rows > 16) dw_rows16(acc, 16, x1, yv, uv);     // block-uniform
-            if (with_bias) acc_bias = __fmaf_rn(fminf(biasvolt - yv, 0.0f), uv, acc_bias);
+            // the inputs of the half's patch, from the lanes that fetched them to all
+            __builtin_amdgcn_wave_barrier();
+            if ((lane & 16) == 0) {
+                xstage[wave][half][l16] = x0;
+                xstage[wave][half][l16 + 16] = x1;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            const float ys = yv * -neg_s;
+            const float4* __restrict__ xq = reinterpret_cast<const float4*>(xstage[wave][half]);
+            auto rows16 = [&](int base) {
+                float xr[16];
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float4 x4 = xq[base / 4 + v];
+                    xr[4 * v] = x4.x; xr[4 * v + 1] = x4.y; xr[4 * v + 2] = x4.z; xr[4 * v + 3] = x4.w;
+                }
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[base + r] = __fmaf_rn(scaled_lead(xr[r], neg_s, ys), uv, acc[base + r]);
+            };
+            rows16(0);
+            if (n_rows > 16) rows16(16);                  // block-uniform
+            if (with_bias) acc_bias = __fmaf_rn(scaled_lead(biasvolt, neg_s, ys), uv, acc_bias);
         }
     }
 #pragma unroll
@@ -576,7 +577,7 @@ cv_grad_weight_narrow_kernel(const float* __restrict__ xpad, const float* __rest
             float sum = 0.0f;
 #pragma unroll
             for (int wv = 0; wv < 4; ++wv) sum = (sum + red[wv][r][kc]) + red[wv][r][kc + 32];
-            out[(size_t)(r == DWW_RI ? bias_row : i0 + r) * Kc + kc] = sum;
+            out[(size_t)(r == DWW_RI ? bias_row : i0 + r) * Kc + kc] = sum * post;
         }
     }
 }
