@@ -64,12 +64,14 @@ __device__ __forceinline__ void count_before_f32(const float* list, int n, const
 }
 
 // Merges the ascending key lists A[0..nA) and B[0..nB) (all keys distinct once `orB` is or-ed into
-// the keys of B; both lists are followed by an all-ones sentinel) into out[0..nA+nB), with one
+// the keys of B and those of A have become (a | orA) - subA; both lists are followed by an all-ones
+// sentinel, which stays above every key under these changes) into out[0..nA+nB), with one
 // wavefront, and ends `out` with a sentinel of its own.  A lane produces RUNS runs of E consecutive
 // outputs each (independent chains of LDS reads that overlap): a binary search along the diagonal
 // i + j = first output finds how many of a run's outputs come from A, then one output per step.  `out` must not overlap the inputs (the lanes of a wavefront read and write side by side).
 template <int RUNS>
-__device__ __forceinline__ void wave_merge(const u64* A, int nA, const u64* B, int nB, u64 orB, u64* out, int lane) {
+__device__ __forceinline__ void wave_merge(const u64* A, int nA, const u64* B, int nB, u64 orB, u64* out, int lane,
+                                           u64 orA = 0, u64 subA = 0) {
     const int n = nA + nB;
     const int E = (n + kWave * RUNS - 1) / (kWave * RUNS);
     int d0[RUNS], d1[RUNS], lo[RUNS], hi[RUNS];
@@ -94,7 +96,7 @@ __device__ __forceinline__ void wave_merge(const u64* A, int nA, const u64* B, i
 #pragma unroll
         for (int r = 0; r < RUNS; ++r) {
             const bool open = lo[r] < hi[r];
-            const bool a_first = a[r] < (b[r] | orB);                  // A[i] goes before B[j-1]: i is too small
+            const bool a_first = ((a[r] | orA) - subA) < (b[r] | orB); // A[i] goes before B[j-1]: i is too small
             lo[r] = (open && a_first) ? mid[r] + 1 : lo[r];
             hi[r] = (open && !a_first) ? mid[r] : hi[r];
         }
@@ -105,7 +107,7 @@ __device__ __forceinline__ void wave_merge(const u64* A, int nA, const u64* B, i
     for (int u = 0; u < E; ++u) {
         u64 a[RUNS], b[RUNS];
 #pragma unroll
-        for (int r = 0; r < RUNS; ++r) { a[r] = A[i[r]]; b[r] = B[j[r]] | orB; }   // sentinels stand in for an exhausted list
+        for (int r = 0; r < RUNS; ++r) { a[r] = (A[i[r]] | orA) - subA; b[r] = B[j[r]] | orB; }   // sentinels stand in for an exhausted list
 #pragma unroll
         for (int r = 0; r < RUNS; ++r) {
             const bool live = d0[r] + u < d1[r];
@@ -296,18 +298,7 @@ merge_patches_kernel(const float* __restrict__ pix_z, const int32_t* __restrict_
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
     u64* my_out = out_keys + (size_t)wave * out_stride;
-    for (int j = wave; j < TW && nw0 + j < Nw; j += THREADS / kWave) {
-        // column 0 with 1, the result with 2, ...: the merge that takes in column kw writes the
-        // patch buffer when Kw - 1 - kw is even and the other buffer otherwise, so that the last
-        // one lands in the patch buffer
-        const u64* cols = col_keys + (size_t)(j * Sw) * col_stride;
-        u64* other = my_out + P + 1;
-        const u64* acc = cols;
-        for (int kw = 1; kw < Kw; ++kw) {
-            u64* dst = ((Kw - 1 - kw) & 1) ? other : my_out;
-            wave_merge<MERGE_RUNS>(acc, kw * KhC, cols + (size_t)kw * col_stride, KhC, (u64)kw << 16, dst, lane);
-            acc = dst;
-        }
+    auto store_patch = [&](int j) {
         const size_t s = (size_t)(a * Nh + nh) * Nw + nw0 + j;
         float* so = sorted + s * stride;
         int32_t* po = perm + s * stride;
@@ -326,6 +317,51 @@ merge_patches_kernel(const float* __restrict__ pix_z, const int32_t* __restrict_
             po[e] = id;
         }
         if (lane == 0) n_real[s] = below;
+    };
+    u64* other = my_out + P + 1;
+    const int n_patches = min(TW, Nw - nw0);
+    if (Kw == 3 && Sw == 1) {
+        // Neighbouring patches j and j + 1 share the columns j + 1 and j + 2: their merge M is made once,
+        // with the column numbers of patch j in the keys (1 and 2), and serves both -- patch j is column j
+        // merged with M, patch j + 1 is M, its column numbers lowered by one, merged with column j + 3.
+        // Eight column lengths of sequential merging per pair of patches instead of ten.  (Keys are
+        // distinct and the result of a merge is their ascending order, whatever was merged first.)
+        // A wavefront takes a run of neighbouring patches, as long as the others' give or take one, in
+        // pairs plus a single one where their number is odd.
+        constexpr u64 ONE_COLUMN = 1ull << 16;
+        constexpr int WAVES = THREADS / kWave;
+        const int base = n_patches / WAVES, extra = n_patches - base * WAVES;
+        const int j_first = wave * base + min(wave, extra), j_end = j_first + base + (wave < extra ? 1 : 0);
+        for (int j = j_first; j < j_end; j += 2) {
+            const u64* cols = col_keys + (size_t)j * col_stride;
+            if (j + 1 < j_end) {
+                wave_merge<MERGE_RUNS>(cols + col_stride, KhC, cols + 2 * col_stride, KhC, 2 * ONE_COLUMN, other, lane,
+                                       ONE_COLUMN, 0);
+                wave_merge<MERGE_RUNS>(cols, KhC, other, 2 * KhC, 0, my_out, lane);
+                store_patch(j);
+                wave_merge<MERGE_RUNS>(other, 2 * KhC, cols + 3 * col_stride, KhC, 2 * ONE_COLUMN, my_out, lane, 0,
+                                       ONE_COLUMN);
+                store_patch(j + 1);
+            } else {
+                wave_merge<MERGE_RUNS>(cols, KhC, cols + col_stride, KhC, ONE_COLUMN, other, lane);
+                wave_merge<MERGE_RUNS>(other, 2 * KhC, cols + 2 * col_stride, KhC, 2 * ONE_COLUMN, my_out, lane);
+                store_patch(j);
+            }
+        }
+        return;
+    }
+    for (int j = wave; j < n_patches; j += THREADS / kWave) {
+        // column 0 with 1, the result with 2, ...: the merge that takes in column kw writes the
+        // patch buffer when Kw - 1 - kw is even and the other buffer otherwise, so that the last
+        // one lands in the patch buffer
+        const u64* cols = col_keys + (size_t)(j * Sw) * col_stride;
+        const u64* acc = cols;
+        for (int kw = 1; kw < Kw; ++kw) {
+            u64* dst = ((Kw - 1 - kw) & 1) ? other : my_out;
+            wave_merge<MERGE_RUNS>(acc, kw * KhC, cols + (size_t)kw * col_stride, KhC, (u64)kw << 16, dst, lane);
+            acc = dst;
+        }
+        store_patch(j);
     }
 }
 
