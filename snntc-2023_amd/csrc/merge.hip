@@ -124,20 +124,20 @@ __device__ __forceinline__ void wave_merge(const u64* A, int nA, const u64* B, i
 // outputs): for patches so long that a buffer pair per wavefront does not fit in LDS.  The caller puts
 // a workgroup barrier behind it before anyone reads `out`.
 __device__ __forceinline__ void block_merge(const u64* A, int nA, const u64* B, int nB, u64 orB, u64* out, int tid,
-                                            int nthreads) {
+                                            int nthreads, u64 orA = 0, u64 subA = 0) {
     const int n = nA + nB;
     const int E = (n + nthreads - 1) / nthreads;
     const int d0 = min(tid * E, n), d1 = min(d0 + E, n);
     int lo = max(0, d0 - nB), hi = min(d0, nA);
     while (lo < hi) {                                          // co-rank of the run's first output
         const int mid = (lo + hi) >> 1;
-        const bool a_first = A[mid] < (B[d0 - mid - 1] | orB);
+        const bool a_first = ((A[mid] | orA) - subA) < (B[d0 - mid - 1] | orB);
         lo = a_first ? mid + 1 : lo;
         hi = a_first ? hi : mid;
     }
     int i = lo, j = d0 - lo;
     for (int e = d0; e < d1; ++e) {
-        const u64 a = A[i], b = B[j] | orB;                    // sentinels stand in for an exhausted list
+        const u64 a = (A[i] | orA) - subA, b = B[j] | orB;     // sentinels stand in for an exhausted list
         const bool take_a = a < b;
         out[e] = take_a ? a : b;
         i += take_a ? 1 : 0;
@@ -255,16 +255,8 @@ merge_patches_kernel(const float* __restrict__ pix_z, const int32_t* __restrict_
         // ---- patches, one at a time, by the whole workgroup ------------------------------------------
         __shared__ int below_count;
         u64* other = out_keys + P + 1;
-        for (int j = 0; j < TW && nw0 + j < Nw; ++j) {
-            const u64* cols = col_keys + (size_t)(j * Sw) * col_stride;
-            const u64* acc = cols;
-            if (threadIdx.x == 0) below_count = 0;
-            for (int kw = 1; kw < Kw; ++kw) {
-                u64* dst = ((Kw - 1 - kw) & 1) ? other : out_keys;
-                block_merge(acc, kw * KhC, cols + (size_t)kw * col_stride, KhC, (u64)kw << 16, dst, threadIdx.x, THREADS);
-                __syncthreads();
-                acc = dst;
-            }
+        const u64* acc = nullptr;
+        auto store_patch = [&](int j) {                       // (entered and left by the whole workgroup)
             const size_t s = (size_t)(a * Nh + nh) * Nw + nw0 + j;
             float* so = sorted + s * stride;
             int32_t* po = perm + s * stride;
@@ -286,8 +278,50 @@ merge_patches_kernel(const float* __restrict__ pix_z, const int32_t* __restrict_
             for (int d = kWave / 2; d > 0; d >>= 1) below += __shfl_xor(below, d, kWave);
             if (threadIdx.x % kWave == 0 && below != 0) atomicAdd(&below_count, below);
             __syncthreads();                                  // the buffers are free again, the count is complete
-            if (threadIdx.x == 0) n_real[s] = below_count;
+            if (threadIdx.x == 0) { n_real[s] = below_count; below_count = 0; }
             __syncthreads();
+        };
+        if (threadIdx.x == 0) below_count = 0;
+        __syncthreads();
+        const int n_patches = min(TW, Nw - nw0);
+        if (Kw == 3 && Sw == 1) {
+            // pairs of neighbouring patches share the merge of their two common columns (see the wavefront form below)
+            constexpr u64 ONE_COLUMN = 1ull << 16;
+            for (int j = 0; j < n_patches; j += 2) {
+                const u64* cols = col_keys + (size_t)j * col_stride;
+                if (j + 1 < n_patches) {
+                    block_merge(cols + col_stride, KhC, cols + 2 * col_stride, KhC, 2 * ONE_COLUMN, other, threadIdx.x,
+                                THREADS, ONE_COLUMN, 0);
+                    __syncthreads();
+                    block_merge(cols, KhC, other, 2 * KhC, 0, out_keys, threadIdx.x, THREADS);
+                    __syncthreads();
+                    acc = out_keys;
+                    store_patch(j);
+                    block_merge(other, 2 * KhC, cols + 3 * col_stride, KhC, 2 * ONE_COLUMN, out_keys, threadIdx.x, THREADS,
+                                0, ONE_COLUMN);
+                    __syncthreads();
+                    store_patch(j + 1);
+                } else {
+                    block_merge(cols, KhC, cols + col_stride, KhC, ONE_COLUMN, other, threadIdx.x, THREADS);
+                    __syncthreads();
+                    block_merge(other, 2 * KhC, cols + 2 * col_stride, KhC, 2 * ONE_COLUMN, out_keys, threadIdx.x, THREADS);
+                    __syncthreads();
+                    acc = out_keys;
+                    store_patch(j);
+                }
+            }
+            return;
+        }
+        for (int j = 0; j < n_patches; ++j) {
+            const u64* cols = col_keys + (size_t)(j * Sw) * col_stride;
+            acc = cols;
+            for (int kw = 1; kw < Kw; ++kw) {
+                u64* dst = ((Kw - 1 - kw) & 1) ? other : out_keys;
+                block_merge(acc, kw * KhC, cols + (size_t)kw * col_stride, KhC, (u64)kw << 16, dst, threadIdx.x, THREADS);
+                __syncthreads();
+                acc = dst;
+            }
+            store_patch(j);
         }
         return;
     }
