@@ -28,13 +28,26 @@ namespace {
 //           multiple of 4; chan = C)
 __global__ void __launch_bounds__(256)
 backward_prologue_kernel(const float* __restrict__ grad, const float* __restrict__ y,
-                         const float* __restrict__ rcp, float* __restrict__ upm, int64_t n, float max_cmp, int prep_blocks, int mode, const float* __restrict__ w,
+                         const float* __restrict__ rcp, float* __restrict__ upm, int64_t n, float max_cmp,
+                         int prep_blocks, int vec4, int mode, const float* __restrict__ w,
                          float* __restrict__ wt, int rows, int cols, int chan, float* __restrict__ zeros,
                          int n_zeros) {
     __shared__ float tile[32][33];
     if (blockIdx.x == 0 && (int)threadIdx.x < n_zeros) zeros[threadIdx.x] = 0.0f;    // the dParams output
     if ((int)blockIdx.x < prep_blocks) {
         const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+        if (vec4) {                                      // n a multiple of 4, the arrays 16-byte aligned
+            if (4 * t >= n) return;
+            const float4 yv = reinterpret_cast<const float4*>(y)[t], gv = reinterpret_cast<const float4*>(grad)[t];
+            const float4 rv = reinterpret_cast<const float4*>(rcp)[t];
+            float4 u;
+            u.x = yv.x <= max_cmp ? gv.x * rv.x : 0.0f;
+            u.y = yv.y <= max_cmp ? gv.y * rv.y : 0.0f;
+            u.z = yv.z <= max_cmp ? gv.z * rv.z : 0.0f;
+            u.w = yv.w <= max_cmp ? gv.w * rv.w : 0.0f;
+            reinterpret_cast<float4*>(upm)[t] = u;
+            return;
+        }
         if (t >= n) return;
         const float yv = y[t];
         const bool valid = yv <= max_cmp;
@@ -633,10 +646,12 @@ int blocks_for(int64_t n, int block) { return (int)((n + block - 1) / block); }
 
 }  // namespace
 
-int launch_backward_prologue(const float* grad, const float* y, const float* rcp, float* upm, int64_t n, const NeuronParams& np, int mode, const float* w, float* wt, int64_t rows,
+int launch_backward_prologue(const float* grad, const float* y, const float* rcp, float* upm, int64_t n,
+                             const NeuronParams& np, int mode, const float* w, float* wt, int64_t rows,
                              int64_t cols, int64_t chan, float* zeros, int n_zeros, hipStream_t stream) {
     if (!zeros) n_zeros = 0;
-    const int64_t prep_blocks = (n + 255) / 256;
+    const bool vec4 = n % 4 == 0 && (((uintptr_t)grad | (uintptr_t)y | (uintptr_t)rcp | (uintptr_t)upm) & 15) == 0;
+    const int64_t prep_blocks = vec4 ? (n / 4 + 255) / 256 : (n + 255) / 256;
     int64_t copy_blocks = 0;
     if (mode == 1) copy_blocks = ((cols + 31) / 32) * ((rows + 31) / 32);
     else if (mode == 2) copy_blocks = (rows * (cols / 4) + 255) / 256;
@@ -646,7 +661,7 @@ int launch_backward_prologue(const float* grad, const float* y, const float* rcp
     {
         KernelTimerScope timer_("prep_upstream", stream);
         hipLaunchKernelGGL(backward_prologue_kernel, dim3((unsigned)(prep_blocks + copy_blocks)), dim3(256), 0, stream,
-                           grad, y, rcp, upm, n, np.max_cmp, (int)prep_blocks, mode, w, wt, (int)rows, (int)cols,
+                           grad, y, rcp, upm, n, np.max_cmp, (int)prep_blocks, vec4 ? 1 : 0, mode, w, wt, (int)rows, (int)cols,
                            (int)chan, zeros, n_zeros);
     }
     SNNTC_HIP_CHECK(hipGetLastError());
